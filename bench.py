@@ -1,0 +1,293 @@
+#!/usr/bin/env python3
+"""
+Benchmark of the gated linear scan on one MI355X.
+
+A step is one forward + one backward scan over one batch of the Mamba-like
+configuration, fp32 [B=8, C=2048, T=4096] (a = sigmoid(N(0,1)), b, grad_h ~
+N(0,1), seed 0), with every tensor already resident in HBM and every output
+pre-allocated. The headline value is the achieved HBM bandwidth of the step in
+algorithmic bytes (32 B per element: forward reads a, b and writes h = 12 B;
+backward reads a, h, grad_h and writes grad_a, grad_b = 20 B).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-configs]
+
+Prints ONE JSON line. Besides the contract fields it carries
+  roofline      the dominant kernel (backward) against the 8 TB/s HBM peak, its
+                duration measured with HIP events on the launch stream;
+  roofline_fwd  the same for the forward kernel;
+  cpu_baseline  the reference's single-threaded CPU loop on the same tensors,
+                timed on this host (oracle/_ref if it was built, else the C
+                restatement in oracle/);
+  configs       forward and forward+backward GB/s of the other four synthetic
+                configurations (buffer sets rotated so that the 256 MB
+                Infinity Cache cannot serve them).
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+METRIC = "scan HBM GB/s and % of MI355X peak, fwd and fwd+bwd, fp32 [B,C,T]"
+FWD_BYTES = {4: 12, 2: 6}
+BWD_BYTES = {4: 20, 2: 10}
+
+
+def make_config(n, torch):
+    """Inputs of synthetic configuration n (1-based), on the CPU generator, seed 0."""
+    torch.manual_seed(0)
+    dtype = torch.float32
+    if n == 1:
+        shape = (4, 256, 1024)
+        a, b = torch.rand(shape), torch.randn(shape)
+    elif n == 2:
+        shape = (8, 2048, 4096)
+        a, b = torch.sigmoid(torch.randn(shape)), torch.randn(shape)
+    elif n == 3:
+        shape = (1, 64, 1 << 20)
+        a, b = 0.9 + 0.1 * torch.rand(shape), torch.randn(shape)
+    elif n in (4, 40):
+        shape = (16, 1024, 2048)
+        a, b = torch.sigmoid(2 + torch.randn(shape)), 0.5 * torch.randn(shape)
+        dtype = torch.bfloat16 if n == 4 else torch.float16
+    elif n == 5:
+        shape = (256, 512, 64)
+        a, b = torch.rand(shape), torch.randn(shape)
+    else:
+        raise ValueError(n)
+    gh = torch.randn(shape)
+    return tuple(x.to(dtype) for x in (a, b, gh))
+
+
+class DeviceSet:
+    """One set of device tensors for forward + backward, flattened to [rows, T]."""
+
+    def __init__(self, a, b, gh, dev, torch):
+        T = a.shape[-1]
+        self.a = a.reshape(-1, T).to(dev)
+        self.b = b.reshape(-1, T).to(dev)
+        self.gh = gh.reshape(-1, T).to(dev)
+        self.h = torch.empty_like(self.a)
+        self.ga = torch.empty_like(self.a)
+        self.gb = torch.empty_like(self.a)
+
+    def clone(self, torch):
+        c = object.__new__(DeviceSet)
+        for k, v in self.__dict__.items():
+            setattr(c, k, v.clone())
+        return c
+
+
+def time_kernels(sets, steps, warmup, hip, torch):
+    """Runs (forward; backward) `steps` times, rotating over `sets`.
+
+    Returns (wall seconds per step, mean fwd kernel ms, mean bwd kernel ms),
+    the kernel times from HIP events recorded on the launch stream around each
+    launch.
+    """
+    for i in range(warmup):
+        s = sets[i % len(sets)]
+        hip.scan_forward_out(s.a, s.b, s.h)
+        hip.scan_backward_out(s.a, s.h, s.gh, s.ga, s.gb)
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        s = sets[i % len(sets)]
+        ev[i][0].record()
+        hip.scan_forward_out(s.a, s.b, s.h)
+        ev[i][1].record()
+        hip.scan_backward_out(s.a, s.h, s.gh, s.ga, s.gb)
+        ev[i][2].record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+    fwd = [e[0].elapsed_time(e[1]) for e in ev]
+    bwd = [e[1].elapsed_time(e[2]) for e in ev]
+    return wall, statistics.fmean(fwd), statistics.fmean(bwd), min(fwd), min(bwd)
+
+
+def cpu_baseline(a, b, gh, reps):
+    """The reference's CPU loop on the same tensors, one thread."""
+    import numpy as np
+    import torch
+
+    import oracle
+
+    T = a.shape[-1]
+    n = a.numel()
+    ext = oracle.ref_ext()
+    if ext is not None:
+        kind = "reference"
+        a2, b2, gh2 = (x.reshape(-1, T).contiguous() for x in (a, b, gh))
+        h, ga, gb = torch.empty_like(a2), torch.empty_like(a2), torch.empty_like(a2)
+
+        def fwd():
+            ext.simple_linear_scan_cpu(a2, b2, h)
+
+        def bwd():
+            ext.simple_linear_scan_backward_cpu(a2, h, gh2, ga, gb)
+    else:
+        kind = "port"
+        a2, b2, gh2 = (np.ascontiguousarray(x.reshape(-1, T).numpy()) for x in (a, b, gh))
+        state = {}
+
+        def fwd():
+            state["h"] = oracle.fwd(a2, b2)
+
+        def bwd():
+            oracle.bwd(a2, state["h"], gh2)
+
+    times = {"fwd": [], "bwd": []}
+    for rep in range(reps + 1):
+        for name, fn in (("fwd", fwd), ("bwd", bwd)):
+            t0 = time.perf_counter()
+            fn()
+            dt = time.perf_counter() - t0
+            if rep > 0:  # first pass is the warm-up
+                times[name].append(dt)
+    tf, tb = statistics.median(times["fwd"]), statistics.median(times["bwd"])
+    return {
+        "value": round(32 * n / (tf + tb) / 1e9, 3),
+        "unit": "GB/s",
+        "cores": 1,
+        "kind": kind,
+        "sample": f"the full workload ({n} elements), 1 warm-up + {reps} repetitions per direction, median",
+        "fwd_GBps": round(12 * n / tf / 1e9, 3),
+        "bwd_GBps": round(20 * n / tb / 1e9, 3),
+        "fwd_s": round(tf, 4),
+        "bwd_s": round(tb, 4),
+        "elements_per_s": round(n / (tf + tb)),
+        "host_cpus": os.cpu_count(),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-configs", action="store_true", help="skip the other four configurations")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (rows are independent, so more GPUs would "
+                 "just split the rows with no communication); use --gpus 1")
+
+    import torch
+
+    from scanscam_amd import hip
+
+    if not hip.has_hip_ops:
+        sys.exit("bench.py: scanscam_amd/libscanscam_hip.so is missing; build it first")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    dev = torch.device("cuda:0")
+
+    a, b, gh = make_config(2, torch)
+    n = a.numel()
+    sets = [DeviceSet(a, b, gh, dev, torch)]
+    wall, fwd_ms, bwd_ms, fwd_min, bwd_min = time_kernels(sets, args.steps, args.warmup, hip, torch)
+    fwd_gbps = FWD_BYTES[4] * n / (fwd_ms * 1e-3) / 1e9
+    bwd_gbps = BWD_BYTES[4] * n / (bwd_ms * 1e-3) / 1e9
+    step_gbps = 32 * n / wall / 1e9
+    plan_f = hip.resolve_plan(sets[0].a.shape[0], sets[0].a.shape[1], torch.float32, hip.FORWARD)
+
+    out = {
+        "metric": METRIC,
+        "value": round(step_gbps, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "configs[1]: forward + backward fp32 scan, [B=8, C=2048, T=4096], a=sigmoid(N(0,1)), "
+                        "b, grad_h ~ N(0,1), seed 0; value = 32 B/element * elements / step time",
+            "elements": n,
+            "plan": repr(plan_f),
+        },
+        "frac_of_peak": round(step_gbps / HBM_PEAK_GBPS, 4),
+        "elements_per_s": round(n / wall),
+        "fwd": {"ms": round(fwd_ms, 4), "min_ms": round(fwd_min, 4), "GBps": round(fwd_gbps, 1),
+                "frac": round(fwd_gbps / HBM_PEAK_GBPS, 4)},
+        "fwd_bwd": {"ms": round(fwd_ms + bwd_ms, 4), "GBps": round(32 * n / ((fwd_ms + bwd_ms) * 1e-3) / 1e9, 1),
+                    "frac": round(32 * n / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)},
+        "roofline": {
+            "kernel": "scan_row_kernel<float, 4, 4, REV=true> (backward)",
+            "bound": "hbm",
+            "achieved": round(bwd_gbps, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(bwd_gbps / HBM_PEAK_GBPS, 4),
+            "traffic": None,
+            "bytes_per_launch": BWD_BYTES[4] * n,
+            "avg_ms": round(bwd_ms, 4),
+            "min_ms": round(bwd_min, 4),
+        },
+        "roofline_fwd": {
+            "kernel": "scan_row_kernel<float, 4, 4, REV=false> (forward)",
+            "bound": "hbm",
+            "achieved": round(fwd_gbps, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(fwd_gbps / HBM_PEAK_GBPS, 4),
+            "traffic": None,
+            "bytes_per_launch": FWD_BYTES[4] * n,
+            "avg_ms": round(fwd_ms, 4),
+            "min_ms": round(fwd_min, 4),
+        },
+    }
+    del sets
+
+    if not args.no_configs:
+        others = {}
+        for key, cfg in (("1", 1), ("3", 3), ("4_bf16", 4), ("4_f16", 40), ("5", 5)):
+            ca, cb, cgh = make_config(cfg, torch)
+            esize = ca.element_size()
+            cn = ca.numel()
+            first = DeviceSet(ca, cb, cgh, dev, torch)
+            # Enough distinct buffer sets that a pass cannot be served from the
+            # 256 MB Infinity Cache: at least 1 GiB of tensors in rotation.
+            per_set = 6 * cn * esize
+            nsets = max(1, min(64, -(-(1 << 30) // per_set)))
+            csets = [first] + [first.clone(torch) for _ in range(nsets - 1)]
+            steps = max(args.steps, 2 * nsets)
+            w, f_ms, b_ms, _, _ = time_kernels(csets, steps, max(args.warmup, nsets), hip, torch)
+            rows, T = first.a.shape
+            others[key] = {
+                "shape": list(ca.shape),
+                "dtype": str(ca.dtype).replace("torch.", ""),
+                "plan": repr(hip.resolve_plan(rows, T, ca.dtype, hip.FORWARD)),
+                "buffer_sets": nsets,
+                "fwd_ms": round(f_ms, 4),
+                "fwd_GBps": round(FWD_BYTES[esize] * cn / (f_ms * 1e-3) / 1e9, 1),
+                "fwd_frac": round(FWD_BYTES[esize] * cn / (f_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                "fwd_bwd_ms": round(f_ms + b_ms, 4),
+                "fwd_bwd_GBps": round((FWD_BYTES[esize] + BWD_BYTES[esize]) * cn / ((f_ms + b_ms) * 1e-3) / 1e9, 1),
+                "fwd_bwd_frac": round((FWD_BYTES[esize] + BWD_BYTES[esize]) * cn / ((f_ms + b_ms) * 1e-3) / 1e9
+                                      / HBM_PEAK_GBPS, 4),
+                "elements_per_s_fwd_bwd": round(cn / ((f_ms + b_ms) * 1e-3)),
+            }
+            del csets, first
+            torch.cuda.empty_cache()
+        out["configs"] = others
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(a, b, gh, reps=5)
+
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

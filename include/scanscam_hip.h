@@ -1,0 +1,129 @@
+/*
+ * scanscam_hip.h -- C ABI of libscanscam_hip.so: the first-order gated linear
+ * scan h[t] = a[t]*h[t-1] + b[t] and its reverse-time backward pass as HIP
+ * kernels for gfx950 (MI355X).
+ *
+ * These entry points are what a binding of the reference's native layer would
+ * call for this path. The reference exposes it through pybind11 functions
+ * taking torch tensors (src/scanscam_cuda.cu:725-737); here the same calls take
+ * plain device pointers and sizes.
+ *
+ * Conventions (same as the reference's native functions):
+ *   - every tensor is a dense row-major [rows, T] array on the current HIP
+ *     device, scanned along T, all of one storage type;
+ *   - the caller allocates every output and the workspace; the library
+ *     allocates nothing, keeps no state and is re-entrant;
+ *   - calls are asynchronous: kernels are enqueued on `stream` (0 = the null
+ *     stream) and the call returns at once;
+ *   - the return value is 0 on success or a SCANSCAM_E* code; nothing is
+ *     launched when an error is returned.
+ * rows == 0 or T == 0 is a successful no-op.
+ */
+#ifndef SCANSCAM_HIP_H
+#define SCANSCAM_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Storage types. Arithmetic is always fp32. */
+enum {
+    SCANSCAM_F32 = 0,
+    SCANSCAM_BF16 = 1, /* no counterpart in the reference (float/double only, src/scanscam_cpu.hpp:43) */
+    SCANSCAM_F16 = 2
+};
+
+enum { SCANSCAM_FORWARD = 0, SCANSCAM_BACKWARD = 1 };
+
+/* Error codes. */
+enum {
+    SCANSCAM_OK = 0,
+    SCANSCAM_EINVAL = 1,    /* null pointer, negative size, T >= 2^31 - 2^20 */
+    SCANSCAM_EDTYPE = 2,    /* unknown storage type */
+    SCANSCAM_EALIGN = 3,    /* pointer not aligned to its element size, or workspace not to 8 bytes */
+    SCANSCAM_EPLAN = 4,     /* explicit plan not valid for this shape / alignment */
+    SCANSCAM_EWORKSPACE = 5,/* workspace missing or smaller than scanscam_workspace_bytes() */
+    SCANSCAM_ELAUNCH = 6    /* the HIP runtime refused the launch */
+};
+
+/* Kernel families. */
+enum {
+    SCANSCAM_MODE_AUTO = 0,
+    SCANSCAM_MODE_SMALL = 1,   /* T <= 64*vec: several rows per wave, no carries */
+    SCANSCAM_MODE_ROW = 2,     /* a workgroup (or part of one) walks a whole row */
+    SCANSCAM_MODE_LOOKBACK = 3 /* rows cut into tiles over workgroups, decoupled look-back carries */
+};
+
+/*
+ * Explicit launch plan, for tuning and for tests that must force one kernel
+ * family on a small input. Zero in any field means "choose for me".
+ *   vec            elements per lane per load: 16/sizeof(storage) or 1
+ *   unroll         64-lane chunks per wave per tile: 1, 2, 4 or 8 (1 or 4 when vec == 1)
+ *   waves          waves per workgroup, 1..16 (at most 8 when unroll == 4, 4 when unroll == 8)
+ *   waves_per_row  ROW only: power of two dividing `waves`
+ */
+typedef struct scanscam_plan {
+    int32_t mode;
+    int32_t vec;
+    int32_t unroll;
+    int32_t waves;
+    int32_t waves_per_row;
+} scanscam_plan;
+
+/*
+ * Forward scan: h[r,t] = a[r,t]*h[r,t-1] + b[r,t], h[r,-1] = 0.
+ * Replaces blocked_linear_scan(gate, value, output), src/scanscam_cuda.cu:260-307
+ * (arithmetic of simple_linear_scan_cpu, src/scanscam_cpu.hpp:30-52).
+ */
+int scanscam_scan_fwd(const void *a, const void *b, void *h, int64_t rows, int64_t T, int dtype,
+                      void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Backward scan: gb[r,t] = gh[r,t] + a[r,t+1]*gb[r,t+1] (gb[r,T] = 0),
+ * ga[r,t] = gb[r,t]*h[r,t-1] (h[r,-1] = 0); `h` is the saved forward output.
+ * Replaces blocked_linear_scan_backward(gate, output, outGrad, gateGradOut,
+ * valueGradOut), src/scanscam_cuda.cu:427-469 (arithmetic of
+ * simple_linear_scan_backward_cpu, src/scanscam_cpu.hpp:80-113).
+ */
+int scanscam_scan_bwd(const void *a, const void *h, const void *gh, void *ga, void *gb, int64_t rows,
+                      int64_t T, int dtype, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Bytes of device workspace the two calls above need for this shape (0 for
+ * most shapes; non-zero when long rows are split over workgroups). The
+ * reference's kernels need none, so this has no counterpart there. The
+ * workspace need not be initialised; its contents are clobbered. Two calls
+ * that may overlap in time need separate workspaces.
+ */
+size_t scanscam_workspace_bytes(int64_t rows, int64_t T, int dtype, int direction);
+
+/* The same three calls with an explicit plan (plan == NULL means automatic). */
+int scanscam_scan_fwd_plan(const void *a, const void *b, void *h, int64_t rows, int64_t T, int dtype,
+                           void *workspace, size_t workspace_bytes, void *stream, const scanscam_plan *plan);
+int scanscam_scan_bwd_plan(const void *a, const void *h, const void *gh, void *ga, void *gb, int64_t rows,
+                           int64_t T, int dtype, void *workspace, size_t workspace_bytes, void *stream,
+                           const scanscam_plan *plan);
+size_t scanscam_workspace_bytes_plan(int64_t rows, int64_t T, int dtype, int direction,
+                                     const scanscam_plan *plan);
+
+/*
+ * Writes the plan the automatic choice resolves to for this shape (assuming
+ * 16-byte aligned pointers) into *out. Returns 0 or an error code.
+ */
+int scanscam_resolve_plan(int64_t rows, int64_t T, int dtype, int direction, const scanscam_plan *plan,
+                          scanscam_plan *out);
+
+/* Static, never-freed description of an error code. */
+const char *scanscam_strerror(int code);
+
+/* ABI version of this header: bumped on any incompatible change. */
+int scanscam_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* SCANSCAM_HIP_H */

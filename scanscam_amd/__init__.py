@@ -1,0 +1,11 @@
+"""
+scanscam_amd: the first-order gated linear scan ``h[t] = gate[t] * h[t-1] + value[t]``
+and its backward pass as hand-written HIP kernels for MI355X (gfx950), behind
+the Python surface of unixpickle/scanscam (``scanscam/__init__.py:1-3``).
+
+    from scanscam_amd import scan
+    h = scan(gate, value)        # [N x ... x T] tensors on an AMD GPU; differentiable
+"""
+from .op import Scan, is_transpose_contig, scan
+
+__all__ = ["scan", "Scan", "is_transpose_contig"]

@@ -1,0 +1,288 @@
+// C ABI of libscanscam_hip.so (declared in include/scanscam_hip.h): argument
+// checks, the choice of kernel family and launch shape, and the launches.
+#include "scanscam_hip.h"
+
+#include "scan_launch.hpp"
+
+namespace {
+
+using scanscam::kDescBase;
+using scanscam::kDescWords;
+using scanscam::kModeLookback;
+using scanscam::kModeRow;
+using scanscam::kModeSmall;
+using scanscam::kWave;
+using scanscam::Launch;
+using scanscam::ScanArgs;
+
+// Clears the look-back workspace (a kernel, not a memset, so that a caller may
+// capture the launch sequence in a HIP graph).
+__global__ __launch_bounds__(256) void scan_ws_clear_kernel(uint64_t *ws, int64_t words)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < words) ws[i] = 0;
+}
+
+constexpr int64_t kMaxT = (int64_t(1) << 31) - (int64_t(1) << 20);
+
+int elem_size(int dtype)
+{
+    switch (dtype) {
+    case SCANSCAM_F32: return 4;
+    case SCANSCAM_BF16:
+    case SCANSCAM_F16: return 2;
+    default: return 0;
+    }
+}
+
+bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
+
+int pow2_ceil(int64_t v)
+{
+    int p = 1;
+    while (p < v) p <<= 1;
+    return p;
+}
+
+bool unroll_ok(int vec, int full, int unroll)
+{
+    if (vec == full) return unroll == 1 || unroll == 2 || unroll == 4 || unroll == 8;
+    return unroll == 1 || unroll == 4;
+}
+
+struct Resolved {
+    Launch l;
+    int nch;
+    int tiles_per_row;
+    size_t ws_bytes;
+};
+
+// Turns (shape, alignment, optional user plan) into a launch. `aligned16` says
+// whether every tensor base is 16-byte aligned.
+int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool aligned16, Resolved *out)
+{
+    const int esize = elem_size(dtype);
+    if (esize == 0) return SCANSCAM_EDTYPE;
+    if (rows < 0 || T < 0 || T >= kMaxT) return SCANSCAM_EINVAL;
+    const int full = 16 / esize;
+    scanscam_plan u = {0, 0, 0, 0, 0};
+    if (user) u = *user;
+
+    Launch &l = out->l;
+    l = Launch{0, 0, 0, 0, 1, 64, 0};
+    const bool vec_possible = aligned16 && (T % full == 0);
+    l.vec = u.vec ? u.vec : (vec_possible ? full : 1);
+    if (l.vec != 1 && l.vec != full) return SCANSCAM_EPLAN;
+    if (l.vec == full && full != 1 && !vec_possible) return SCANSCAM_EPLAN;
+
+    const int64_t chunk = (int64_t)kWave * l.vec;
+    const int64_t nch64 = (T + chunk - 1) / chunk;
+    const int nch = (int)nch64;
+    out->nch = nch;
+    out->tiles_per_row = 0;
+    out->ws_bytes = 0;
+    if (rows == 0 || T == 0) return SCANSCAM_OK;
+
+    l.mode = u.mode;
+    if (l.mode == SCANSCAM_MODE_AUTO) {
+        if (T <= chunk) l.mode = kModeSmall;
+        else if (nch >= 64 && rows < 2048) l.mode = kModeLookback;
+        else l.mode = kModeRow;
+    }
+
+    if (l.mode == kModeSmall) {
+        if (T > chunk) return SCANSCAM_EPLAN;
+        l.group = pow2_ceil((T + l.vec - 1) / l.vec);
+        l.unroll = u.unroll ? u.unroll : 4;
+        l.waves = u.waves ? u.waves : 4;
+        const int64_t rows_per_wg = (int64_t)l.waves * l.unroll * (kWave / l.group);
+        l.grid = (rows + rows_per_wg - 1) / rows_per_wg;
+    } else if (l.mode == kModeRow) {
+        l.unroll = u.unroll;
+        l.waves = u.waves;
+        l.wpr = u.waves_per_row;
+        if (!l.unroll && !l.waves && !l.wpr) {
+            if (nch <= 4) {
+                l.unroll = (l.vec == full) ? pow2_ceil(nch) : (nch == 1 ? 1 : 4);
+                l.wpr = 1;
+                l.waves = 4;
+            } else if (rows < 2048 && nch >= 16) {
+                l.unroll = 1;
+                l.wpr = 16;
+                l.waves = 16;
+            } else {
+                l.unroll = (l.vec == full && nch <= 8) ? 2 : 4;
+                l.wpr = 4;
+                l.waves = 4;
+            }
+        } else {
+            if (!l.unroll) l.unroll = 4;
+            if (!l.waves) l.waves = l.wpr ? l.wpr : 4;
+            if (!l.wpr) l.wpr = l.waves;
+        }
+        if (!is_pow2(l.wpr) || l.wpr > l.waves || l.waves % l.wpr != 0) return SCANSCAM_EPLAN;
+        const int rows_per_wg = l.waves / l.wpr;
+        l.grid = (rows + rows_per_wg - 1) / rows_per_wg;
+    } else if (l.mode == kModeLookback) {
+        l.unroll = u.unroll ? u.unroll : 4;
+        l.waves = u.waves ? u.waves : 4;
+        const int tile_chunks = l.waves * l.unroll;
+        out->tiles_per_row = (nch + tile_chunks - 1) / tile_chunks;
+        l.grid = rows * (int64_t)out->tiles_per_row;
+        if (l.grid >= (int64_t(1) << 31)) return SCANSCAM_EINVAL;
+        out->ws_bytes = (size_t)(kDescBase + l.grid * kDescWords) * sizeof(uint64_t);
+    } else {
+        return SCANSCAM_EPLAN;
+    }
+
+    if (!unroll_ok(l.vec, full, l.unroll)) return SCANSCAM_EPLAN;
+    if (l.waves < 1 || l.waves > scanscam::kMaxWaves ||
+        l.waves * kWave > scanscam::max_threads_for_unroll(l.unroll))
+        return SCANSCAM_EPLAN;
+    if (l.grid >= (int64_t(1) << 31)) return SCANSCAM_EINVAL;
+    return SCANSCAM_OK;
+}
+
+bool aligned_to(const void *p, size_t n) { return (reinterpret_cast<uintptr_t>(p) % n) == 0; }
+
+int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y1, int64_t rows, int64_t T,
+        int dtype, void *workspace, size_t workspace_bytes, void *stream, const scanscam_plan *plan)
+{
+    const int esize = elem_size(dtype);
+    if (esize == 0) return SCANSCAM_EDTYPE;
+    if (rows < 0 || T < 0 || T >= kMaxT) return SCANSCAM_EINVAL;
+    if (rows == 0 || T == 0) return SCANSCAM_OK;
+    if (!a || !x || !y0 || (rev && (!h || !y1))) return SCANSCAM_EINVAL;
+
+    const void *ptrs[5] = {a, x, y0, rev ? h : a, rev ? y1 : y0};
+    bool aligned16 = true;
+    for (const void *p : ptrs) {
+        if (!aligned_to(p, (size_t)esize)) return SCANSCAM_EALIGN;
+        aligned16 = aligned16 && aligned_to(p, 16);
+    }
+
+    Resolved r;
+    const int rc = resolve(plan, rows, T, dtype, aligned16, &r);
+    if (rc != SCANSCAM_OK) return rc;
+
+    ScanArgs args;
+    args.a = a;
+    args.x = x;
+    args.h = h;
+    args.y0 = y0;
+    args.y1 = y1;
+    args.rows = rows;
+    args.T = (int32_t)T;
+    args.nch = r.nch;
+    args.wpr = r.l.wpr;
+    args.group = r.l.group;
+    args.tiles_per_row = r.tiles_per_row;
+    args.ws = nullptr;
+
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (r.l.mode == kModeLookback) {
+        if (!workspace || workspace_bytes < r.ws_bytes) return SCANSCAM_EWORKSPACE;
+        if (!aligned_to(workspace, 8)) return SCANSCAM_EALIGN;
+        args.ws = static_cast<uint64_t *>(workspace);
+        const int64_t words = (int64_t)(r.ws_bytes / sizeof(uint64_t));
+        hipLaunchKernelGGL(scan_ws_clear_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0,
+                           s, args.ws, words);
+        if (hipGetLastError() != hipSuccess) return SCANSCAM_ELAUNCH;
+    }
+
+    hipError_t e = hipErrorInvalidValue;
+    switch (dtype) {
+    case SCANSCAM_F32: e = scanscam::launch_scan<float>(args, r.l, rev, s); break;
+    case SCANSCAM_BF16: e = scanscam::launch_scan<__bf16>(args, r.l, rev, s); break;
+    case SCANSCAM_F16: e = scanscam::launch_scan<_Float16>(args, r.l, rev, s); break;
+    }
+    return e == hipSuccess ? SCANSCAM_OK : SCANSCAM_ELAUNCH;
+}
+
+size_t workspace_for(int64_t rows, int64_t T, int dtype, const scanscam_plan *plan)
+{
+    // The caller's pointers are not known yet: cover both the 16-byte aligned
+    // and the unaligned choice.
+    size_t need = 0;
+    for (int al = 0; al < 2; al++) {
+        Resolved r;
+        if (resolve(plan, rows, T, dtype, al != 0, &r) == SCANSCAM_OK && r.ws_bytes > need) need = r.ws_bytes;
+    }
+    return need;
+}
+
+}  // namespace
+
+extern "C" {
+
+int scanscam_scan_fwd(const void *a, const void *b, void *h, int64_t rows, int64_t T, int dtype,
+                      void *workspace, size_t workspace_bytes, void *stream)
+{
+    return run(false, a, b, nullptr, h, nullptr, rows, T, dtype, workspace, workspace_bytes, stream, nullptr);
+}
+
+int scanscam_scan_bwd(const void *a, const void *h, const void *gh, void *ga, void *gb, int64_t rows,
+                      int64_t T, int dtype, void *workspace, size_t workspace_bytes, void *stream)
+{
+    return run(true, a, gh, h, gb, ga, rows, T, dtype, workspace, workspace_bytes, stream, nullptr);
+}
+
+size_t scanscam_workspace_bytes(int64_t rows, int64_t T, int dtype, int direction)
+{
+    (void)direction;
+    return workspace_for(rows, T, dtype, nullptr);
+}
+
+int scanscam_scan_fwd_plan(const void *a, const void *b, void *h, int64_t rows, int64_t T, int dtype,
+                           void *workspace, size_t workspace_bytes, void *stream, const scanscam_plan *plan)
+{
+    return run(false, a, b, nullptr, h, nullptr, rows, T, dtype, workspace, workspace_bytes, stream, plan);
+}
+
+int scanscam_scan_bwd_plan(const void *a, const void *h, const void *gh, void *ga, void *gb, int64_t rows,
+                           int64_t T, int dtype, void *workspace, size_t workspace_bytes, void *stream,
+                           const scanscam_plan *plan)
+{
+    return run(true, a, gh, h, gb, ga, rows, T, dtype, workspace, workspace_bytes, stream, plan);
+}
+
+size_t scanscam_workspace_bytes_plan(int64_t rows, int64_t T, int dtype, int direction,
+                                     const scanscam_plan *plan)
+{
+    (void)direction;
+    return workspace_for(rows, T, dtype, plan);
+}
+
+int scanscam_resolve_plan(int64_t rows, int64_t T, int dtype, int direction, const scanscam_plan *plan,
+                          scanscam_plan *out)
+{
+    (void)direction;
+    if (!out) return SCANSCAM_EINVAL;
+    Resolved r;
+    const int rc = resolve(plan, rows, T, dtype, true, &r);
+    if (rc != SCANSCAM_OK) return rc;
+    out->mode = r.l.mode;
+    out->vec = r.l.vec;
+    out->unroll = r.l.unroll;
+    out->waves = r.l.waves;
+    out->waves_per_row = r.l.mode == kModeRow ? r.l.wpr : 0;
+    return SCANSCAM_OK;
+}
+
+const char *scanscam_strerror(int code)
+{
+    switch (code) {
+    case SCANSCAM_OK: return "ok";
+    case SCANSCAM_EINVAL: return "invalid argument (null pointer, negative or too large size)";
+    case SCANSCAM_EDTYPE: return "unsupported storage type";
+    case SCANSCAM_EALIGN: return "pointer not aligned to its element size (or workspace not to 8 bytes)";
+    case SCANSCAM_EPLAN: return "launch plan not valid for this shape or alignment";
+    case SCANSCAM_EWORKSPACE: return "workspace missing or smaller than scanscam_workspace_bytes()";
+    case SCANSCAM_ELAUNCH: return "HIP runtime refused the kernel launch";
+    default: return "unknown scanscam error code";
+    }
+}
+
+int scanscam_abi_version(void) { return 1; }
+
+}  // extern "C"

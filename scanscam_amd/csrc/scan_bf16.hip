@@ -1,0 +1,6 @@
+// Kernel instantiations for __bf16 storage (fp32 arithmetic).
+#include "scan_launch.hpp"
+
+namespace scanscam {
+SCANSCAM_DEFINE_LAUNCH(__bf16)
+}  // namespace scanscam

@@ -1,0 +1,6 @@
+// Kernel instantiations for _Float16 storage (fp32 arithmetic).
+#include "scan_launch.hpp"
+
+namespace scanscam {
+SCANSCAM_DEFINE_LAUNCH(_Float16)
+}  // namespace scanscam

@@ -1,0 +1,6 @@
+// Kernel instantiations for float storage (fp32 arithmetic).
+#include "scan_launch.hpp"
+
+namespace scanscam {
+SCANSCAM_DEFINE_LAUNCH(float)
+}  // namespace scanscam

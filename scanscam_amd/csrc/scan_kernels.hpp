@@ -1,0 +1,576 @@
+// First-order gated linear scan for gfx950 (MI355X): device code.
+//
+//   forward   h[t]  = a[t] * h[t-1] + b[t],            h[-1] = 0
+//   backward  gb[t] = gh[t] + a[t+1] * gb[t+1],        gb[T] = 0
+//             ga[t] = gb[t] * h[t-1],                  h[-1] = 0
+//
+// (the arithmetic of the reference's CPU loops, src/scanscam_cpu.hpp:17-27 and
+// :64-77, which its CUDA kernels src/scanscam_cuda.cu:144-258, 366-425 also
+// compute). Both directions are the same scan over affine maps h -> A*h + B,
+// composed as (A2, B2) o (A1, B1) = (A2*A1, A2*B1 + B2); the backward pass is
+// that scan run over reversed time with gate a[t+1] and value gh[t].
+//
+// Data layout: every tensor is a dense row-major [rows, T] array, scanned along
+// T. A lane owns one 16-byte vector (VEC elements) of a 64-lane "chunk"
+// (64*VEC consecutive elements of one row), so every load and store
+// instruction of a wave covers one contiguous 1 KiB span. For the backward
+// pass lane l owns vector 63-l of the chunk and reads its components in
+// descending order: the span per instruction is unchanged, and the scan
+// runs "forwards" over lanes in both directions.
+//
+// Per chunk a lane (1) folds its VEC elements into one affine pair, (2) takes
+// part in a wave64 inclusive scan of the pairs on DPP lane moves (row_shr 1, 2,
+// 4, 8, row_bcast 15, row_bcast 31), (3) once the carry into the chunk is
+// known, replays its VEC elements from its own carry-in and stores them.
+// Chunk-to-chunk carries are single FMAs; wave-to-wave carries go through LDS;
+// tile-to-tile carries go through registers (ROW kernel, one workgroup walks a
+// row) or through a decoupled look-back chain in global memory (LOOKBACK
+// kernel, the tiles of a row are spread over workgroups).
+//
+// The op is HBM-bound (12 B/element forward, 20 B/element backward in fp32) and
+// has no contraction in it, so no MFMA is used anywhere.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#ifndef SCANSCAM_NT_LOAD
+#define SCANSCAM_NT_LOAD 1
+#endif
+#ifndef SCANSCAM_NT_STORE
+#define SCANSCAM_NT_STORE 1
+#endif
+
+namespace scanscam {
+
+constexpr int kWave = 64;
+constexpr int kMaxWaves = 16;
+
+// ---------------------------------------------------------------------------
+// Kernel arguments (plain pointers; the host fills them per launch).
+// ---------------------------------------------------------------------------
+struct ScanArgs {
+    const void *a;   // gates                       [rows, T]
+    const void *x;   // forward: b      backward: gh
+    const void *h;   // forward: unused backward: saved forward output
+    void *y0;        // forward: h      backward: gb (value grad)
+    void *y1;        // forward: unused backward: ga (gate grad)
+    int64_t rows;
+    int32_t T;
+    int32_t nch;            // chunks per row = ceil(T / (64*VEC))
+    int32_t wpr;            // ROW: waves cooperating on one row
+    int32_t group;          // SMALL: lanes per row (power of two, <= 64)
+    int32_t tiles_per_row;  // LOOKBACK: tiles per row
+    uint64_t *ws;           // LOOKBACK: ticket counter + tile descriptors
+};
+
+// Look-back workspace layout, in 64-bit words. Word 0 is the ticket counter,
+// word 1 is raised if a look-back wait ever expired (results are then NaN);
+// each tile owns kDescWords words from kDescBase on:
+//   [0] {1, bits(A)}  [1] {1, bits(B)}   the tile's own aggregate
+//   [2] {1, bits(h)}                     the scan value at the tile's end
+// The upper half is a ready flag; the workspace is zeroed before each launch,
+// so every word is self-validating and no fence is needed around it.
+constexpr int kDescBase = 8;
+constexpr int kDescWords = 4;
+
+// ---------------------------------------------------------------------------
+// Storage types: float, __bf16, _Float16. All arithmetic is fp32.
+// ---------------------------------------------------------------------------
+template <int BYTES> struct RawT;
+template <> struct RawT<16> { typedef uint32_t type __attribute__((ext_vector_type(4))); };
+template <> struct RawT<8> { typedef uint32_t type __attribute__((ext_vector_type(2))); };
+template <> struct RawT<4> { typedef uint32_t type; };
+template <> struct RawT<2> { typedef uint16_t type; };
+
+template <typename ST, int VEC> struct Elems { ST e[VEC]; };
+
+template <typename ST, int VEC> struct Vec {
+    using raw_t = typename RawT<sizeof(ST) * VEC>::type;
+
+    static __device__ __forceinline__ raw_t zero_raw()
+    {
+        Elems<ST, VEC> z;
+#pragma unroll
+        for (int k = 0; k < VEC; k++) z.e[k] = (ST)0.0f;
+        return __builtin_bit_cast(raw_t, z);
+    }
+    static __device__ __forceinline__ raw_t load(const ST *p)
+    {
+        const raw_t *q = reinterpret_cast<const raw_t *>(p);
+#if SCANSCAM_NT_LOAD
+        return __builtin_nontemporal_load(q);
+#else
+        return *q;
+#endif
+    }
+    static __device__ __forceinline__ void store(ST *p, raw_t r)
+    {
+        raw_t *q = reinterpret_cast<raw_t *>(p);
+#if SCANSCAM_NT_STORE
+        __builtin_nontemporal_store(r, q);
+#else
+        *q = r;
+#endif
+    }
+    static __device__ __forceinline__ void unpack(raw_t r, float (&f)[VEC])
+    {
+        Elems<ST, VEC> e = __builtin_bit_cast(Elems<ST, VEC>, r);
+#pragma unroll
+        for (int k = 0; k < VEC; k++) f[k] = (float)e.e[k];
+    }
+    static __device__ __forceinline__ raw_t pack(const float (&f)[VEC])
+    {
+        Elems<ST, VEC> e;
+#pragma unroll
+        for (int k = 0; k < VEC; k++) e.e[k] = (ST)f[k];
+        return __builtin_bit_cast(raw_t, e);
+    }
+};
+
+// ---------------------------------------------------------------------------
+// Lane moves.
+// ---------------------------------------------------------------------------
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_move(float old, float src)
+{
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, src),
+                                           CTRL, ROW_MASK, 0xf, false));
+}
+
+// Value of the previous / next lane of the wave; `fill` where there is none.
+__device__ __forceinline__ float lane_prev(float src, float fill) { return dpp_move<0x138, 0xf>(fill, src); }
+__device__ __forceinline__ float lane_next(float src, float fill) { return dpp_move<0x130, 0xf>(fill, src); }
+
+__device__ __forceinline__ float read_lane(float v, int lane)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+// Inclusive scan of affine pairs over the lanes of a wave (ascending lane =
+// later in scan order). With GROUPED the wave is cut into independent groups of
+// `group` lanes (j = lane index inside its group). Lanes that have no source
+// in a step receive the identity map (1, 0). All 64 lanes must be active.
+template <bool GROUPED>
+__device__ __forceinline__ void wave_scan(float &A, float &B, int j)
+{
+#define SCANSCAM_STEP(CTRL, ROW_MASK, OFF)                      \
+    {                                                           \
+        float A1 = dpp_move<CTRL, ROW_MASK>(1.0f, A);           \
+        float B1 = dpp_move<CTRL, ROW_MASK>(0.0f, B);           \
+        if (GROUPED) {                                          \
+            const bool use = j >= (OFF);                        \
+            A1 = use ? A1 : 1.0f;                               \
+            B1 = use ? B1 : 0.0f;                               \
+        }                                                       \
+        B = __builtin_fmaf(A, B1, B);                           \
+        A = A * A1;                                             \
+    }
+    SCANSCAM_STEP(0x111, 0xf, 1)   // row_shr:1
+    SCANSCAM_STEP(0x112, 0xf, 2)   // row_shr:2
+    SCANSCAM_STEP(0x114, 0xf, 4)   // row_shr:4
+    SCANSCAM_STEP(0x118, 0xf, 8)   // row_shr:8
+    SCANSCAM_STEP(0x142, 0xa, 16)  // row_bcast:15 into rows 1 and 3
+    SCANSCAM_STEP(0x143, 0xc, 32)  // row_bcast:31 into rows 2 and 3
+#undef SCANSCAM_STEP
+}
+
+// ---------------------------------------------------------------------------
+// One wave's share of a tile: U chunks.
+//
+// Phase "load":   issue every global load of the U chunks.
+// Phase "reduce": per-lane fold + wave scan per chunk -> PA/PB, chunk totals.
+// Phase "apply":  given the carry into chunk 0, replay and store.
+// With CHAIN the U chunks are consecutive in scan order (carry flows from one
+// into the next); without it they are unrelated rows (SMALL kernel).
+// ---------------------------------------------------------------------------
+template <typename ST, int VEC, int U, bool REV, bool GROUPED, bool CHAIN>
+struct WaveTile {
+    using V = Vec<ST, VEC>;
+    using raw_t = typename V::raw_t;
+
+    // Where this lane's vector of chunk u lives.
+    int64_t off[U];  // element offset of the vector from the tensor base
+    int32_t m[U];    // vector index inside the row (element m*VEC)
+    bool valid[U];   // inside the row (and the row exists)
+
+    raw_t ra[U], rx[U], rh[REV ? U : 1];
+    float edge_a[REV ? U : 1];  // a[(m+1)*VEC] for the first lane of a group
+    float edge_h[REV ? U : 1];  // h[m*VEC - 1] for the last lane of a group
+
+    float g[U][VEC], v[U][VEC];
+    float PA[U], PB[U];
+
+    __device__ __forceinline__ void load(const ScanArgs &p, int j, int jlast)
+    {
+        const ST *a = static_cast<const ST *>(p.a);
+        const ST *x = static_cast<const ST *>(p.x);
+        const ST *h = static_cast<const ST *>(p.h);
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            ra[u] = V::zero_raw();
+            rx[u] = V::zero_raw();
+            if (valid[u]) {
+                ra[u] = V::load(a + off[u]);
+                rx[u] = V::load(x + off[u]);
+            }
+            if (REV) {
+                rh[u] = V::zero_raw();
+                if (valid[u]) rh[u] = V::load(h + off[u]);
+                edge_a[u] = 0.0f;
+                edge_h[u] = 0.0f;
+                // Neighbours that no lane of this group holds.
+                if (valid[u] && j == 0 && (m[u] + 1) * VEC < p.T) edge_a[u] = (float)a[off[u] + VEC];
+                if (valid[u] && j == jlast && m[u] > 0) edge_h[u] = (float)h[off[u] - 1];
+            }
+        }
+    }
+
+    // Builds (gate, value) per element in scan order and reduces them.
+    __device__ __forceinline__ void reduce(int j, int jlast, float (&hp)[REV ? U : 1][VEC])
+    {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            float fa[VEC], fx[VEC];
+            V::unpack(ra[u], fa);
+            V::unpack(rx[u], fx);
+            if (!REV) {
+#pragma unroll
+                for (int k = 0; k < VEC; k++) {
+                    g[u][k] = valid[u] ? fa[k] : 1.0f;
+                    v[u][k] = fx[k];  // zero-filled where invalid
+                }
+            } else {
+                float fh[VEC];
+                V::unpack(rh[u], fh);
+                // Scan order k <-> time t0 + VEC-1-k. gate = a[t+1], value = gh[t],
+                // hp = h[t-1]. Invalid lanes hold a = 0, so a neighbour past the
+                // end of the row reads as gate 0, which is what t = T-1 needs.
+                float a_next = lane_prev(fa[0], 0.0f);        // lane-1 holds vector m+1
+                float h_prev = lane_next(fh[VEC - 1], 0.0f);  // lane+1 holds vector m-1
+                a_next = (j == 0) ? edge_a[u] : a_next;
+                h_prev = (j == jlast) ? edge_h[u] : h_prev;
+#pragma unroll
+                for (int k = 0; k < VEC; k++) {
+                    const float gk = (k == 0) ? a_next : fa[(VEC - k) % VEC];
+                    g[u][k] = valid[u] ? gk : 1.0f;
+                    v[u][k] = fx[VEC - 1 - k];
+                    hp[u][k] = (k == VEC - 1) ? h_prev : fh[(VEC - 2 - k) < 0 ? 0 : (VEC - 2 - k)];
+                }
+            }
+            float A = g[u][0], B = v[u][0];
+#pragma unroll
+            for (int k = 1; k < VEC; k++) {
+                B = __builtin_fmaf(g[u][k], B, v[u][k]);
+                A = A * g[u][k];
+            }
+            wave_scan<GROUPED>(A, B, j);
+            PA[u] = A;
+            PB[u] = B;
+        }
+    }
+
+    // Aggregate of the wave's U chunks (CHAIN only): composition in scan order.
+    __device__ __forceinline__ void total(float &WA, float &WB) const
+    {
+        WA = read_lane(PA[0], 63);
+        WB = read_lane(PB[0], 63);
+#pragma unroll
+        for (int u = 1; u < U; u++) {
+            const float TA = read_lane(PA[u], 63), TB = read_lane(PB[u], 63);
+            WB = __builtin_fmaf(TA, WB, TB);
+            WA = TA * WA;
+        }
+    }
+
+    __device__ __forceinline__ void apply(const ScanArgs &p, float carry, int j,
+                                          const float (&hp)[REV ? U : 1][VEC])
+    {
+        ST *y0 = static_cast<ST *>(p.y0);
+        ST *y1 = static_cast<ST *>(p.y1);
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            // Map of everything before this lane inside the chunk.
+            float EA = lane_prev(PA[u], 1.0f);
+            float EB = lane_prev(PB[u], 0.0f);
+            if (GROUPED) {
+                EA = (j == 0) ? 1.0f : EA;
+                EB = (j == 0) ? 0.0f : EB;
+            }
+            const float c = CHAIN ? carry : 0.0f;
+            float acc = __builtin_fmaf(EA, c, EB);
+            float out[VEC];
+#pragma unroll
+            for (int k = 0; k < VEC; k++) {
+                acc = __builtin_fmaf(g[u][k], acc, v[u][k]);
+                out[k] = acc;
+            }
+            if (CHAIN && u + 1 < U)
+                carry = __builtin_fmaf(read_lane(PA[u], 63), carry, read_lane(PB[u], 63));
+            if (!REV) {
+                if (valid[u]) V::store(y0 + off[u], V::pack(out));
+            } else {
+                float gb[VEC], ga[VEC];
+#pragma unroll
+                for (int k = 0; k < VEC; k++) {
+                    gb[VEC - 1 - k] = out[k];
+                    ga[VEC - 1 - k] = out[k] * hp[u][k];
+                }
+                if (valid[u]) {
+                    V::store(y0 + off[u], V::pack(gb));
+                    V::store(y1 + off[u], V::pack(ga));
+                }
+            }
+        }
+    }
+};
+
+// ---------------------------------------------------------------------------
+// ROW kernel: `wpr` waves walk one row tile by tile; a workgroup of W waves
+// holds W / wpr rows. Tile = wpr * U chunks. Carries: FMA chunk to chunk, LDS
+// wave to wave, a register tile to tile.
+// ---------------------------------------------------------------------------
+template <typename ST, int VEC, int U, bool REV, int MAXT>
+__global__ __launch_bounds__(MAXT) void scan_row_kernel(const ScanArgs p)
+{
+    __shared__ float lds_A[2][kMaxWaves];
+    __shared__ float lds_B[2][kMaxWaves];
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int nwaves = blockDim.x / kWave;
+    const int wpr = p.wpr;
+    const int rows_per_wg = nwaves / wpr;
+    const int wr = wave % wpr;          // this wave's place among the row's waves
+    const int wbase = wave - wr;        // first wave of the row's group
+    const int64_t row = (int64_t)blockIdx.x * rows_per_wg + wave / wpr;
+    const bool row_ok = row < p.rows;
+    const int64_t row_off = row_ok ? row * (int64_t)p.T : 0;
+    const int nvp = p.nch * kWave;      // vectors per row, padded to whole chunks
+    const int tile_chunks = wpr * U;
+    const int ntiles = (p.nch + tile_chunks - 1) / tile_chunks;
+
+    WaveTile<ST, VEC, U, REV, false, true> w;
+    float hp[REV ? U : 1][VEC];
+    float row_carry = 0.0f;
+
+    for (int it = 0; it < ntiles; it++) {
+        const int chunk0 = (it * wpr + wr) * U;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int s = (chunk0 + u) * kWave + lane;  // vector index in scan order
+            const int m = REV ? nvp - 1 - s : s;
+            w.m[u] = m;
+            w.valid[u] = row_ok && m >= 0 && (int64_t)m * VEC < p.T;
+            w.off[u] = row_off + (int64_t)m * VEC;
+        }
+        w.load(p, lane, kWave - 1);
+        w.reduce(lane, kWave - 1, hp);
+
+        float carry = row_carry;
+        if (wpr > 1) {
+            float WA, WB;
+            w.total(WA, WB);
+            if (lane == 0) {
+                lds_A[it & 1][wave] = WA;
+                lds_B[it & 1][wave] = WB;
+            }
+            __syncthreads();
+            float c = row_carry;
+            for (int q = 0; q < wpr; q++) {
+                if (q == wr) carry = c;
+                c = __builtin_fmaf(lds_A[it & 1][wbase + q], c, lds_B[it & 1][wbase + q]);
+            }
+            row_carry = c;
+        } else if (ntiles > 1) {
+            float WA, WB;
+            w.total(WA, WB);
+            row_carry = __builtin_fmaf(WA, row_carry, WB);
+        }
+        w.apply(p, carry, lane, hp);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// SMALL kernel: rows no longer than one chunk. `group` lanes hold one row, a
+// wave holds U * 64 / group rows, and nothing is carried anywhere.
+// ---------------------------------------------------------------------------
+template <typename ST, int VEC, int U, bool REV, int MAXT>
+__global__ __launch_bounds__(MAXT) void scan_small_kernel(const ScanArgs p)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int G = p.group;
+    const int j = lane & (G - 1);
+    const int rows_per_chunk = kWave / G;
+    const int64_t wave_id = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+    const int64_t row0 = wave_id * (U * rows_per_chunk) + lane / G;
+
+    WaveTile<ST, VEC, U, REV, true, false> w;
+    float hp[REV ? U : 1][VEC];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const int64_t row = row0 + (int64_t)u * rows_per_chunk;
+        const int m = REV ? G - 1 - j : j;
+        w.m[u] = m;
+        w.valid[u] = row < p.rows && m * VEC < p.T;
+        w.off[u] = (w.valid[u] ? row * (int64_t)p.T : 0) + (int64_t)m * VEC;
+    }
+    w.load(p, j, G - 1);
+    w.reduce(j, G - 1, hp);
+    w.apply(p, 0.0f, j, hp);
+}
+
+// ---------------------------------------------------------------------------
+// LOOKBACK kernel: the tiles of a row are spread over workgroups. Tiles are
+// handed out by an atomic ticket, so every tile a workgroup may wait for was
+// taken by a workgroup that is already running. Ticket k works on row
+// k % rows, tile k / rows, which keeps the tiles in flight at any moment
+// spread over all rows.
+//
+// Carry protocol (wave 0 of the workgroup): publish the tile's aggregate
+// (A, B); 64 lanes inspect the 64 preceding tiles of the row at once; the
+// nearest one that has published its end value h gives the start, and the
+// aggregates of the tiles between it and this one are applied to it one FMA
+// at a time, oldest first. That is the same chain of FMAs whichever tile
+// happens to be the nearest published one, so results do not depend on timing.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ uint64_t desc_load(const uint64_t *p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void desc_store(uint64_t *p, float v)
+{
+    const uint64_t w = (1ull << 32) | (uint64_t)__builtin_bit_cast(uint32_t, v);
+    __hip_atomic_store(p, w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ bool desc_ready(uint64_t w) { return (w >> 32) != 0; }
+__device__ __forceinline__ float desc_value(uint64_t w) { return __builtin_bit_cast(float, (uint32_t)w); }
+
+// Polls of the look-back loop before a wave gives up. Tickets make every
+// awaited tile belong to a workgroup that is already running, so the limit is
+// never reached in a correct launch (a poll is a memory round trip; the limit
+// is seconds). It exists so that no wave can spin for ever: on expiry the wave
+// raises word kTimeoutWord of the workspace and carries NaN onwards.
+constexpr int kSpinLimit = 1 << 20;
+constexpr int kTimeoutWord = 1;
+
+// Returns the scan value entering tile `tile` of the row whose descriptors
+// start at `row_desc`. Called by all 64 lanes of one wave.
+__device__ __forceinline__ float lookback_carry(const uint64_t *row_desc, int tile, int lane, uint64_t *ws)
+{
+    const int look = tile - 1 - lane;  // the tile this lane watches
+    bool have_incl = look < 0;         // before the row starts the value is 0
+    bool have_agg = look < 0;
+    float incl = 0.0f, A = 1.0f, B = 0.0f;
+    for (int spin = 0; spin < kSpinLimit; spin++) {
+        if (look >= 0) {
+            const uint64_t *d = row_desc + (int64_t)look * kDescWords;
+            if (!have_incl) {
+                const uint64_t wi = desc_load(d + 2);
+                if (desc_ready(wi)) {
+                    have_incl = true;
+                    incl = desc_value(wi);
+                }
+            }
+            if (!have_agg) {
+                const uint64_t wa = desc_load(d + 0), wb = desc_load(d + 1);
+                if (desc_ready(wa) && desc_ready(wb)) {
+                    have_agg = true;
+                    A = desc_value(wa);
+                    B = desc_value(wb);
+                }
+            }
+        }
+        const uint64_t mi = __ballot(have_incl);
+        const uint64_t ma = __ballot(have_agg);
+        if (mi != 0) {
+            const int first = __builtin_ctzll(mi);  // nearest tile with a published end value
+            const uint64_t need = (first == 0) ? 0ull : ((~0ull) >> (64 - first));
+            if ((ma & need) == need) {
+                float c = read_lane(incl, first);
+                for (int q = first - 1; q >= 0; q--)
+                    c = __builtin_fmaf(read_lane(A, q), c, read_lane(B, q));
+                return c;
+            }
+        }
+        __builtin_amdgcn_s_sleep(1);
+    }
+    if (lane == 0) __hip_atomic_store(ws + kTimeoutWord, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return __builtin_nanf("");
+}
+
+template <typename ST, int VEC, int U, bool REV, int MAXT>
+__global__ __launch_bounds__(MAXT) void scan_lookback_kernel(const ScanArgs p)
+{
+    __shared__ float lds_A[kMaxWaves];
+    __shared__ float lds_B[kMaxWaves];
+    __shared__ float lds_carry;
+    __shared__ unsigned lds_ticket;
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int nwaves = blockDim.x / kWave;
+
+    if (threadIdx.x == 0)
+        lds_ticket = __hip_atomic_fetch_add(reinterpret_cast<unsigned *>(p.ws), 1u, __ATOMIC_RELAXED,
+                                            __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    const unsigned ticket = lds_ticket;
+    const int64_t row = ticket % (uint64_t)p.rows;
+    const int tile = (int)(ticket / (uint64_t)p.rows);
+    const int64_t row_off = row * (int64_t)p.T;
+    const int nvp = p.nch * kWave;
+    const int chunk0 = (tile * nwaves + wave) * U;
+
+    WaveTile<ST, VEC, U, REV, false, true> w;
+    float hp[REV ? U : 1][VEC];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const int s = (chunk0 + u) * kWave + lane;
+        const int m = REV ? nvp - 1 - s : s;
+        w.m[u] = m;
+        w.valid[u] = m >= 0 && (int64_t)m * VEC < p.T;
+        w.off[u] = row_off + (int64_t)m * VEC;
+    }
+    w.load(p, lane, kWave - 1);
+    w.reduce(lane, kWave - 1, hp);
+
+    float WA, WB;
+    w.total(WA, WB);
+    if (lane == 0) {
+        lds_A[wave] = WA;
+        lds_B[wave] = WB;
+    }
+    __syncthreads();
+
+    if (wave == 0) {
+        // Aggregate of the whole tile, waves in scan order.
+        float TA = lds_A[0], TB = lds_B[0];
+        for (int q = 1; q < nwaves; q++) {
+            TB = __builtin_fmaf(lds_A[q], TB, lds_B[q]);
+            TA = lds_A[q] * TA;
+        }
+        uint64_t *row_desc = p.ws + kDescBase + row * (int64_t)p.tiles_per_row * kDescWords;
+        uint64_t *mine = row_desc + (int64_t)tile * kDescWords;
+        float cin = 0.0f;
+        if (tile > 0) {
+            if (lane == 0) {
+                desc_store(mine + 0, TA);
+                desc_store(mine + 1, TB);
+            }
+            cin = lookback_carry(row_desc, tile, lane, p.ws);
+        }
+        if (lane == 0) {
+            desc_store(mine + 2, __builtin_fmaf(TA, cin, TB));
+            lds_carry = cin;
+        }
+    }
+    __syncthreads();
+
+    float carry = lds_carry;
+    for (int q = 0; q < wave; q++) carry = __builtin_fmaf(lds_A[q], carry, lds_B[q]);
+    w.apply(p, carry, lane, hp);
+}
+
+}  // namespace scanscam

@@ -1,0 +1,234 @@
+"""
+Binding of ``libscanscam_hip.so`` (C ABI in ``include/scanscam_hip.h``) and the
+``[rows, T]`` wrappers the autograd op calls.
+
+Takes the place of the reference's ``scanscam/cuda.py``: ``has_hip_ops`` is its
+``has_cuda_ops`` probe (``cuda.py:7-13``), and ``blocked_linear_scan_forward`` /
+``blocked_linear_scan_backward`` keep the names, argument order and behaviour of
+``cuda.py:34-40`` and ``:56-66`` (inputs made contiguous, outputs allocated with
+``torch.empty_like``, any leading dimensions flattened). PyTorch is used for
+device memory and the current stream only; all arithmetic happens in the
+library's kernels. There is no other implementation behind these functions: if
+the library is missing they raise.
+"""
+import ctypes
+import os
+from typing import Optional, Tuple
+
+import torch
+
+from .decorator import preprocess_backward_scan_args, preprocess_scan_args
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libscanscam_hip.so")
+
+MODE_AUTO, MODE_SMALL, MODE_ROW, MODE_LOOKBACK = 0, 1, 2, 3
+FORWARD, BACKWARD = 0, 1
+ABI_VERSION = 1
+
+_DTYPES = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
+
+
+class Plan(ctypes.Structure):
+    """``scanscam_plan``: an explicit launch plan; zero fields are chosen automatically."""
+
+    _fields_ = [
+        ("mode", ctypes.c_int32),
+        ("vec", ctypes.c_int32),
+        ("unroll", ctypes.c_int32),
+        ("waves", ctypes.c_int32),
+        ("waves_per_row", ctypes.c_int32),
+    ]
+
+    def __repr__(self) -> str:
+        return (
+            f"Plan(mode={self.mode}, vec={self.vec}, unroll={self.unroll}, "
+            f"waves={self.waves}, waves_per_row={self.waves_per_row})"
+        )
+
+
+def _bind(path: str) -> ctypes.CDLL:
+    lib = ctypes.CDLL(path)
+    p, i64, i32, sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t
+    plan_p = ctypes.POINTER(Plan)
+    lib.scanscam_scan_fwd.argtypes = [p, p, p, i64, i64, i32, p, sz, p]
+    lib.scanscam_scan_fwd.restype = i32
+    lib.scanscam_scan_bwd.argtypes = [p, p, p, p, p, i64, i64, i32, p, sz, p]
+    lib.scanscam_scan_bwd.restype = i32
+    lib.scanscam_workspace_bytes.argtypes = [i64, i64, i32, i32]
+    lib.scanscam_workspace_bytes.restype = sz
+    lib.scanscam_scan_fwd_plan.argtypes = [p, p, p, i64, i64, i32, p, sz, p, plan_p]
+    lib.scanscam_scan_fwd_plan.restype = i32
+    lib.scanscam_scan_bwd_plan.argtypes = [p, p, p, p, p, i64, i64, i32, p, sz, p, plan_p]
+    lib.scanscam_scan_bwd_plan.restype = i32
+    lib.scanscam_workspace_bytes_plan.argtypes = [i64, i64, i32, i32, plan_p]
+    lib.scanscam_workspace_bytes_plan.restype = sz
+    lib.scanscam_resolve_plan.argtypes = [i64, i64, i32, i32, plan_p, plan_p]
+    lib.scanscam_resolve_plan.restype = i32
+    lib.scanscam_strerror.argtypes = [i32]
+    lib.scanscam_strerror.restype = ctypes.c_char_p
+    lib.scanscam_abi_version.argtypes = []
+    lib.scanscam_abi_version.restype = i32
+    if lib.scanscam_abi_version() != ABI_VERSION:
+        raise OSError(f"{path}: ABI version {lib.scanscam_abi_version()}, this binding needs {ABI_VERSION}")
+    return lib
+
+
+_lib: Optional[ctypes.CDLL] = None
+_load_error: Optional[str] = None
+try:
+    _lib = _bind(LIB_PATH)
+except OSError as exc:  # not built, or built for another ABI
+    _load_error = str(exc)
+
+has_hip_ops = _lib is not None
+
+
+def lib() -> ctypes.CDLL:
+    """The loaded library; raises if it is not there (there is no substitute)."""
+    if _lib is None:
+        raise RuntimeError(
+            "scanscam_amd: the HIP library is not available "
+            f"({_load_error}); build it with `make -C scanscam_amd/csrc` "
+            "or `python -c 'import __graft_entry__ as g; g.build()'`"
+        )
+    return _lib
+
+
+def strerror(code: int) -> str:
+    return lib().scanscam_strerror(code).decode()
+
+
+def resolve_plan(rows: int, T: int, dtype: torch.dtype, direction: int = FORWARD,
+                 plan: Optional[Plan] = None) -> Plan:
+    """The plan the library would run for this shape (no GPU needed)."""
+    out = Plan()
+    rc = lib().scanscam_resolve_plan(rows, T, _dtype_code(dtype), direction,
+                                     ctypes.byref(plan) if plan is not None else None, ctypes.byref(out))
+    if rc != 0:
+        raise RuntimeError(f"scanscam_resolve_plan: {strerror(rc)}")
+    return out
+
+
+def workspace_bytes(rows: int, T: int, dtype: torch.dtype, direction: int = FORWARD,
+                    plan: Optional[Plan] = None) -> int:
+    if plan is None:
+        return int(lib().scanscam_workspace_bytes(rows, T, _dtype_code(dtype), direction))
+    return int(lib().scanscam_workspace_bytes_plan(rows, T, _dtype_code(dtype), direction, ctypes.byref(plan)))
+
+
+def _dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPES[dtype]
+    except KeyError:
+        raise TypeError(f"scanscam_amd: unsupported dtype {dtype}; supported: float32, bfloat16, float16") from None
+
+
+def _check_rows(*tensors: torch.Tensor) -> None:
+    first = tensors[0]
+    for t in tensors:
+        if t.device.type != "cuda":
+            raise RuntimeError(f"scanscam_amd.hip: expected a GPU tensor, got one on {t.device}")
+        if t.device != first.device:
+            raise RuntimeError("scanscam_amd.hip: tensors are on different devices")
+        if t.dtype != first.dtype:
+            raise TypeError(f"scanscam_amd.hip: tensors differ in dtype ({first.dtype} and {t.dtype})")
+        if t.shape != first.shape or t.dim() != 2:
+            raise AssertionError("scanscam_amd.hip: expected 2-D tensors of one shape")
+        if not t.is_contiguous():
+            raise RuntimeError("scanscam_amd.hip: tensors must be contiguous")
+
+
+def _workspace(rows: int, T: int, dtype: torch.dtype, direction: int, plan: Optional[Plan],
+               device: torch.device) -> Tuple[Optional[torch.Tensor], int, int]:
+    n = workspace_bytes(rows, T, dtype, direction, plan)
+    if n == 0:
+        return None, 0, 0
+    ws = torch.empty(n, dtype=torch.uint8, device=device)
+    return ws, ws.data_ptr(), n
+
+
+def scan_forward_out(gate: torch.Tensor, value: torch.Tensor, out: torch.Tensor,
+                     plan: Optional[Plan] = None) -> None:
+    """``out[r, t] = gate[r, t] * out[r, t-1] + value[r, t]`` on contiguous 2-D GPU tensors.
+
+    The raw call: what ``scanscam_ext.blocked_linear_scan(gate, value, output)``
+    is in the reference (``src/scanscam_cuda.cu:260-263``). Asynchronous on the
+    current stream.
+    """
+    L = lib()
+    _check_rows(gate, value, out)
+    rows, T = gate.shape
+    code = _dtype_code(gate.dtype)
+    if rows == 0 or T == 0:
+        return
+    with torch.cuda.device(gate.device):
+        ws, ws_ptr, ws_n = _workspace(rows, T, gate.dtype, FORWARD, plan, gate.device)
+        stream = torch.cuda.current_stream().cuda_stream
+        rc = L.scanscam_scan_fwd_plan(gate.data_ptr(), value.data_ptr(), out.data_ptr(), rows, T, code,
+                                      ws_ptr, ws_n, stream, ctypes.byref(plan) if plan is not None else None)
+    if rc != 0:
+        raise RuntimeError(f"scanscam_scan_fwd: {strerror(rc)}")
+
+
+def scan_backward_out(gate: torch.Tensor, output: torch.Tensor, out_grad: torch.Tensor,
+                      gate_grad: torch.Tensor, value_grad: torch.Tensor,
+                      plan: Optional[Plan] = None) -> None:
+    """The raw backward call (``src/scanscam_cuda.cu:427-433`` in the reference)."""
+    L = lib()
+    _check_rows(gate, output, out_grad, gate_grad, value_grad)
+    rows, T = gate.shape
+    code = _dtype_code(gate.dtype)
+    if rows == 0 or T == 0:
+        return
+    with torch.cuda.device(gate.device):
+        ws, ws_ptr, ws_n = _workspace(rows, T, gate.dtype, BACKWARD, plan, gate.device)
+        stream = torch.cuda.current_stream().cuda_stream
+        rc = L.scanscam_scan_bwd_plan(gate.data_ptr(), output.data_ptr(), out_grad.data_ptr(),
+                                      gate_grad.data_ptr(), value_grad.data_ptr(), rows, T, code,
+                                      ws_ptr, ws_n, stream, ctypes.byref(plan) if plan is not None else None)
+    if rc != 0:
+        raise RuntimeError(f"scanscam_scan_bwd: {strerror(rc)}")
+
+
+def linear_scan_forward(gate: torch.Tensor, value: torch.Tensor, plan: Optional[Plan] = None) -> torch.Tensor:
+    """Forward scan of ``[N x ... x T]`` GPU tensors with an optional explicit plan."""
+
+    @preprocess_scan_args
+    def run(x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+        x = x.contiguous()
+        y = y.contiguous()
+        out = torch.empty_like(x)
+        scan_forward_out(x, y, out, plan)
+        return out
+
+    return run(gate, value)
+
+
+def linear_scan_backward(gate: torch.Tensor, output: torch.Tensor, out_grad: torch.Tensor,
+                         plan: Optional[Plan] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Backward scan with an optional explicit plan; returns ``(gate_grad, value_grad)``."""
+
+    @preprocess_backward_scan_args
+    def run(x: torch.Tensor, y: torch.Tensor, z: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+        x = x.contiguous()
+        y = y.contiguous()
+        z = z.contiguous()
+        out_a = torch.empty_like(x)
+        out_b = torch.empty_like(x)
+        scan_backward_out(x, y, z, out_a, out_b, plan)
+        return out_a, out_b
+
+    return run(gate, output, out_grad)
+
+
+def blocked_linear_scan_forward(x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+    """Drop-in for ``scanscam.cuda.blocked_linear_scan_forward`` (``cuda.py:34-40``)."""
+    return linear_scan_forward(x, y)
+
+
+def blocked_linear_scan_backward(
+    x: torch.Tensor, y: torch.Tensor, z: torch.Tensor
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Drop-in for ``scanscam.cuda.blocked_linear_scan_backward`` (``cuda.py:56-66``)."""
+    return linear_scan_backward(x, y, z)

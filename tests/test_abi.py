@@ -1,0 +1,123 @@
+"""
+The C-ABI library loads here (no GPU needed), exports every function that
+include/scanscam_hip.h declares, and rejects bad arguments before launching
+anything. No kernel is launched in this file.
+"""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from scanscam_amd import hip
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "scanscam_hip.h")
+
+E_OK, E_INVAL, E_DTYPE, E_ALIGN, E_PLAN, E_WORKSPACE, E_LAUNCH = range(7)
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(scanscam_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_is_built_and_loads():
+    assert os.path.exists(hip.LIB_PATH), "build with `make -C scanscam_amd/csrc`"
+    assert hip.has_hip_ops
+    assert hip.lib().scanscam_abi_version() == hip.ABI_VERSION
+
+
+def test_every_declared_symbol_is_exported():
+    names = declared_functions()
+    assert "scanscam_scan_fwd" in names and "scanscam_scan_bwd" in names and len(names) == 9
+    raw = ctypes.CDLL(hip.LIB_PATH)
+    for name in names:
+        assert hasattr(raw, name), f"{name} declared in scanscam_hip.h but not exported"
+
+
+def test_header_is_plain_c():
+    import subprocess
+    import tempfile
+
+    with tempfile.TemporaryDirectory() as d:
+        src = os.path.join(d, "t.c")
+        open(src, "w").write('#include "scanscam_hip.h"\nint main(void) { scanscam_plan p = {0}; return p.mode; }\n')
+        subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), "-c", src,
+                        "-o", os.path.join(d, "t.o")], check=True)
+
+
+def test_strerror_covers_every_code():
+    seen = set()
+    for code in range(7):
+        msg = hip.strerror(code)
+        assert msg and msg not in seen
+        seen.add(msg)
+    assert "unknown" in hip.strerror(99)
+
+
+def test_plan_struct_layout_matches_header():
+    assert ctypes.sizeof(hip.Plan) == 20
+    assert [f[0] for f in hip.Plan._fields_] == ["mode", "vec", "unroll", "waves", "waves_per_row"]
+
+
+def test_argument_errors_are_reported_before_any_launch():
+    L = hip.lib()
+    fake = 0x10000  # never dereferenced: every call below must fail validation first
+    assert L.scanscam_scan_fwd(fake, fake, fake, 4, 8, 7, None, 0, None) == E_DTYPE
+    assert L.scanscam_scan_fwd(fake, fake, fake, -1, 8, 0, None, 0, None) == E_INVAL
+    assert L.scanscam_scan_fwd(fake, fake, fake, 4, 2**31, 0, None, 0, None) == E_INVAL
+    assert L.scanscam_scan_fwd(None, fake, fake, 4, 8, 0, None, 0, None) == E_INVAL
+    assert L.scanscam_scan_bwd(fake, fake, fake, None, fake, 4, 8, 0, None, 0, None) == E_INVAL
+    assert L.scanscam_scan_fwd(fake + 2, fake, fake, 4, 8, 0, None, 0, None) == E_ALIGN
+    assert L.scanscam_scan_fwd(fake + 1, fake, fake, 4, 8, 1, None, 0, None) == E_ALIGN
+    # Long rows need a workspace.
+    assert hip.workspace_bytes(4, 1 << 20, torch.float32) > 0
+    assert L.scanscam_scan_fwd(fake, fake, fake, 4, 1 << 20, 0, None, 0, None) == E_WORKSPACE
+    assert L.scanscam_scan_fwd(fake, fake, fake, 4, 1 << 20, 0, fake, 64, None) == E_WORKSPACE
+    # Bad explicit plans.
+    for bad in (hip.Plan(mode=9), hip.Plan(vec=3), hip.Plan(mode=hip.MODE_ROW, unroll=3),
+                hip.Plan(mode=hip.MODE_ROW, unroll=8, waves=8), hip.Plan(mode=hip.MODE_ROW, waves=4, waves_per_row=3),
+                hip.Plan(mode=hip.MODE_SMALL), hip.Plan(waves=17)):
+        rc = L.scanscam_scan_fwd_plan(fake, fake, fake, 4, 4096, 0, None, 0, None, ctypes.byref(bad))
+        assert rc == E_PLAN, bad
+    # vec 4 is impossible when T is not a multiple of 4 or a pointer is not 16-byte aligned.
+    v4 = hip.Plan(vec=4)
+    assert L.scanscam_scan_fwd_plan(fake, fake, fake, 4, 1025, 0, None, 0, None, ctypes.byref(v4)) == E_PLAN
+    assert L.scanscam_scan_fwd_plan(fake + 4, fake, fake, 4, 1024, 0, None, 0, None, ctypes.byref(v4)) == E_PLAN
+
+
+def test_empty_inputs_are_a_successful_noop():
+    L = hip.lib()
+    assert L.scanscam_scan_fwd(None, None, None, 0, 128, 0, None, 0, None) == E_OK
+    assert L.scanscam_scan_fwd(None, None, None, 5, 0, 0, None, 0, None) == E_OK
+    assert L.scanscam_scan_bwd(None, None, None, None, None, 0, 0, 0, None, 0, None) == E_OK
+
+
+@pytest.mark.parametrize(
+    "rows,T,dtype,mode,vec",
+    [
+        (1024, 1024, torch.float32, hip.MODE_ROW, 4),       # forward-only config
+        (16384, 4096, torch.float32, hip.MODE_ROW, 4),      # Mamba-like config
+        (64, 1 << 20, torch.float32, hip.MODE_LOOKBACK, 4), # long sequence
+        (16384, 2048, torch.bfloat16, hip.MODE_ROW, 8),     # 16-bit storage
+        (16384, 2048, torch.float16, hip.MODE_ROW, 8),
+        (131072, 64, torch.float32, hip.MODE_SMALL, 4),     # many short rows
+        (32, 1025, torch.float32, hip.MODE_ROW, 1),         # odd length: element-wise loads
+        (32, 5, torch.float32, hip.MODE_SMALL, 1),
+    ],
+)
+def test_automatic_plan_per_regime(rows, T, dtype, mode, vec):
+    for direction in (hip.FORWARD, hip.BACKWARD):
+        plan = hip.resolve_plan(rows, T, dtype, direction)
+        assert (plan.mode, plan.vec) == (mode, vec), plan
+        ws = hip.workspace_bytes(rows, T, dtype, direction)
+        assert (ws > 0) == (mode == hip.MODE_LOOKBACK)
+
+
+def test_lookback_workspace_size_formula():
+    plan = hip.Plan(mode=hip.MODE_LOOKBACK, vec=4, unroll=2, waves=2)
+    # tile = 2 waves * 2 chunks * 256 elements = 1024 elements; 5 tiles per row of 4100.
+    assert hip.workspace_bytes(3, 4100, torch.float32, hip.FORWARD, plan) == (8 + 3 * 5 * 4) * 8

@@ -1,0 +1,356 @@
+"""
+Parity of the HIP kernels (through the C ABI) with the CPU oracle on identical
+seeded inputs.
+
+Bars:
+  * fp32: max |x - ref| / max(|ref|, 1) <= 1e-5 for h, grad_a, grad_b on the
+    benchmark configurations (gates in [0, 1]); on the reference's own test
+    grid, whose gates are N(0, 1), the reference's bar
+    allclose(atol=1e-4, rtol=1e-5) (scanscam/cuda_test.py:26-34) applied to the
+    normwise error of each row;
+  * 16-bit storage: <= 1e-2 against the fp32 oracle on the upcast inputs.
+The GPU result is not expected to be bit-identical to the oracle: the kernels
+use FMAs and a parallel association order, the oracle a sequential mul + add.
+"""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from scanscam_amd import hip
+
+pytestmark = pytest.mark.gpu
+
+FP32_BAR = 1e-5
+HALF_BAR = 1e-2
+
+
+def rel_err(x, ref):
+    x = np.asarray(x, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    if x.size == 0:
+        return 0.0
+    return float(np.max(np.abs(x - ref) / np.maximum(np.abs(ref), 1.0)))
+
+
+def row_norm_err(x, ref):
+    """max over rows of max|x - ref| / max(1, max|ref|) -- scale-free per row."""
+    x = np.asarray(x, dtype=np.float64).reshape(-1, x.shape[-1])
+    ref = np.asarray(ref, dtype=np.float64).reshape(-1, ref.shape[-1])
+    if x.size == 0:
+        return 0.0
+    scale = np.maximum(np.max(np.abs(ref), axis=1), 1.0)
+    return float(np.max(np.max(np.abs(x - ref), axis=1) / scale))
+
+
+def to_np(t):
+    return t.detach().float().cpu().numpy()
+
+
+def run_fwd(gpu, a, b, plan=None):
+    return hip.linear_scan_forward(a.to(gpu), b.to(gpu), plan)
+
+
+def run_bwd(gpu, a, h, gh, plan=None):
+    return hip.linear_scan_backward(a.to(gpu), h.to(gpu), gh.to(gpu), plan)
+
+
+def seeded(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+# ---------------------------------------------------------------------------
+# The reference's own test grid (scanscam/cuda_test.py:19-126), N(0,1) gates.
+# ---------------------------------------------------------------------------
+REFERENCE_GRID = [
+    (32, 5), (16, 2, 5), (32, 64), (32, 128), (32, 256), (32, 512), (32, 513), (1, 1024), (32, 1024),
+    (32, 1025), (1, 1025), (32, 4095), (32, 4096), (32, 4097), (32, 4100), (32, 16384), (32, 16388),
+]
+
+
+@pytest.mark.parametrize("shape", REFERENCE_GRID)
+@pytest.mark.parametrize("permute", [False, True])
+def test_reference_grid(gpu, shape, permute):
+    g = seeded(100 + sum(shape))
+    a = torch.randn(shape, generator=g)
+    b = torch.randn(shape, generator=g)
+    gh = torch.randn(shape, generator=g)
+    if permute:
+        a = a.mT.contiguous().mT
+    print(f"case reference_grid shape={shape} permute={permute}", flush=True)
+    h = run_fwd(gpu, a, b)
+    assert h.shape == a.shape and h.dtype == a.dtype
+    want = oracle.fwd(a.numpy(), b.numpy())
+    assert row_norm_err(to_np(h), want) <= 1e-4
+    # Backward as a pure function of (gate, output, out_grad), as the reference tests it.
+    hs = torch.from_numpy(want)
+    if permute:
+        hs = hs.mT.contiguous().mT
+    ga, gb = run_bwd(gpu, a, hs, gh)
+    wga, wgb = oracle.bwd(a.numpy(), hs.numpy(), gh.numpy())
+    assert row_norm_err(to_np(gb), wgb) <= 1e-4
+    assert row_norm_err(to_np(ga), wga) <= 1e-4
+
+
+# ---------------------------------------------------------------------------
+# The five benchmark configurations at full size.
+# ---------------------------------------------------------------------------
+def config_inputs(n):
+    torch.manual_seed(0)
+    if n == 1:
+        shape = (4, 256, 1024)
+        a, b = torch.rand(shape), torch.randn(shape)
+    elif n == 2:
+        shape = (8, 2048, 4096)
+        a, b = torch.sigmoid(torch.randn(shape)), torch.randn(shape)
+    elif n == 3:
+        shape = (1, 64, 1 << 20)
+        a, b = 0.9 + 0.1 * torch.rand(shape), torch.randn(shape)
+    elif n == 4:
+        shape = (16, 1024, 2048)
+        a, b = torch.sigmoid(2 + torch.randn(shape)), 0.5 * torch.randn(shape)
+    elif n == 5:
+        shape = (256, 512, 64)
+        a, b = torch.rand(shape), torch.randn(shape)
+    gh = torch.randn(shape)
+    return a, b, gh
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 5])
+def test_benchmark_config_fp32(gpu, n):
+    a, b, gh = config_inputs(n)
+    print(f"case config{n} shape={tuple(a.shape)}", flush=True)
+    h = run_fwd(gpu, a, b)
+    want_h = oracle.fwd(a.numpy(), b.numpy())
+    e_h = rel_err(to_np(h), want_h)
+    # The backward pass is fed the oracle's h, so its error is its own.
+    hs = torch.from_numpy(want_h)
+    ga, gb = run_bwd(gpu, a, hs, gh)
+    wga, wgb = oracle.bwd(a.numpy(), want_h, gh.numpy())
+    e_ga, e_gb = rel_err(to_np(ga), wga), rel_err(to_np(gb), wgb)
+    # Reassociation report: both against the recurrence carried in float64.
+    h64 = oracle.fwd_acc64(a.numpy(), b.numpy())
+    print(f"config{n}: rel err h={e_h:.3e} ga={e_ga:.3e} gb={e_gb:.3e}; vs fp64 chain: "
+          f"gpu={rel_err(to_np(h), h64):.3e} cpu_fp32={rel_err(want_h, h64):.3e}", flush=True)
+    assert e_h <= FP32_BAR and e_ga <= FP32_BAR and e_gb <= FP32_BAR
+    del h64
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_benchmark_config_16bit(gpu, dtype):
+    a, b, gh = (x.to(dtype) for x in config_inputs(4))
+    print(f"case config4 dtype={dtype}", flush=True)
+    h = run_fwd(gpu, a, b)
+    assert h.dtype == dtype
+    want_h = oracle.fwd(a.float().numpy(), b.float().numpy())
+    assert rel_err(to_np(h), want_h) <= HALF_BAR
+    # Feed both sides the same 16-bit saved output, so that its storage rounding
+    # is not charged to the backward kernel.
+    hs = h.cpu()
+    ga, gb = run_bwd(gpu, a, hs, gh)
+    wga, wgb = oracle.bwd(a.float().numpy(), hs.float().numpy(), gh.float().numpy())
+    assert rel_err(to_np(gb), wgb) <= HALF_BAR
+    assert rel_err(to_np(ga), wga) <= HALF_BAR
+
+
+# ---------------------------------------------------------------------------
+# Every kernel family / vector width / unroll / workgroup shape, forced on
+# small inputs with ragged rows and lengths.
+# ---------------------------------------------------------------------------
+def plans_for(dtype):
+    full = 4 if dtype == torch.float32 else 8
+    out = []
+    for vec in (full, 1):
+        unrolls = (1, 2, 4, 8) if vec == full else (1, 4)
+        for unroll in unrolls:
+            max_waves = 16 if unroll <= 2 else 8 if unroll == 4 else 4
+            for waves in sorted({1, 4, max_waves}):
+                for wpr in sorted({1, 2, waves} & {1, 2, 4, 8, 16}):
+                    if waves % wpr == 0:
+                        out.append(hip.Plan(mode=hip.MODE_ROW, vec=vec, unroll=unroll, waves=waves, waves_per_row=wpr))
+                out.append(hip.Plan(mode=hip.MODE_LOOKBACK, vec=vec, unroll=unroll, waves=waves))
+    return out
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_forced_plans_row_and_lookback(gpu, dtype):
+    full = 4 if dtype == torch.float32 else 8
+    bar = FP32_BAR if dtype == torch.float32 else HALF_BAR
+    g = seeded(7)
+    cases = {}
+    for rows, T in [(5, 8 * full * 37), (3, 64 * full * 5 + full), (1, 64 * full * 33), (7, 1037), (2, 64 * full)]:
+        a = torch.rand((rows, T), generator=g).to(dtype)
+        b = torch.randn((rows, T), generator=g).to(dtype)
+        gh = torch.randn((rows, T), generator=g).to(dtype)
+        h = oracle.fwd(a.float().numpy(), b.float().numpy())
+        hs = torch.from_numpy(h).to(dtype)
+        ga, gb = oracle.bwd(a.float().numpy(), hs.float().numpy(), gh.float().numpy())
+        cases[(rows, T)] = (a.to(gpu), b.to(gpu), gh.to(gpu), hs.to(gpu), h, ga, gb)
+    n = 0
+    for plan in plans_for(dtype):
+        for (rows, T), (a, b, gh, hs, h, ga, gb) in cases.items():
+            if plan.vec != 1 and T % full != 0:
+                continue
+            print(f"case forced {dtype} rows={rows} T={T} {plan}", flush=True)
+            got_h = hip.linear_scan_forward(a, b, plan)
+            got_ga, got_gb = hip.linear_scan_backward(a, hs, gh, plan)
+            assert rel_err(to_np(got_h), h) <= bar, (plan, rows, T)
+            assert rel_err(to_np(got_gb), gb) <= bar, (plan, rows, T)
+            assert rel_err(to_np(got_ga), ga) <= bar, (plan, rows, T)
+            n += 1
+    assert n > 100
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_forced_plans_small(gpu, dtype):
+    full = 4 if dtype == torch.float32 else 8
+    bar = FP32_BAR if dtype == torch.float32 else HALF_BAR
+    g = seeded(8)
+    n = 0
+    for vec, unroll, waves in itertools.product((full, 1), (1, 2, 4, 8), (1, 4)):
+        if vec == 1 and unroll not in (1, 4):
+            continue
+        lengths = [vec * k for k in (1, 2, 3, 4, 7, 8, 16, 31, 33, 64)] if vec > 1 else [1, 2, 3, 5, 8, 17, 32, 63, 64]
+        for T in lengths:
+            for rows in (1, 37, 515):
+                plan = hip.Plan(mode=hip.MODE_SMALL, vec=vec, unroll=unroll, waves=waves)
+                a = torch.rand((rows, T), generator=g).to(dtype)
+                b = torch.randn((rows, T), generator=g).to(dtype)
+                gh = torch.randn((rows, T), generator=g).to(dtype)
+                print(f"case small {dtype} rows={rows} T={T} {plan}", flush=True)
+                h = oracle.fwd(a.float().numpy(), b.float().numpy())
+                hs = torch.from_numpy(h).to(dtype)
+                ga, gb = oracle.bwd(a.float().numpy(), hs.float().numpy(), gh.float().numpy())
+                got_h = run_fwd(gpu, a, b, plan)
+                got_ga, got_gb = run_bwd(gpu, a, hs, gh, plan)
+                assert rel_err(to_np(got_h), h) <= bar, (plan, rows, T)
+                assert rel_err(to_np(got_gb), gb) <= bar, (plan, rows, T)
+                assert rel_err(to_np(got_ga), ga) <= bar, (plan, rows, T)
+                n += 1
+    assert n > 100
+
+
+# ---------------------------------------------------------------------------
+# Edge cases and properties.
+# ---------------------------------------------------------------------------
+def test_empty_inputs(gpu):
+    for shape in [(0, 16), (4, 0), (0, 0), (2, 0, 8)]:
+        a = torch.zeros(shape, device=gpu)
+        h = hip.linear_scan_forward(a, a)
+        assert h.shape == a.shape
+        ga, gb = hip.linear_scan_backward(a, a, a)
+        assert ga.shape == a.shape and gb.shape == a.shape
+
+
+@pytest.mark.parametrize("T", [1, 2, 3, 4, 63, 64, 65, 255, 256, 257, 260])
+@pytest.mark.parametrize("rows", [1, 2, 129])
+def test_short_rows_automatic(gpu, rows, T):
+    g = seeded(rows * 1000 + T)
+    a = torch.rand((rows, T), generator=g)
+    b = torch.randn((rows, T), generator=g)
+    gh = torch.randn((rows, T), generator=g)
+    h = oracle.fwd(a.numpy(), b.numpy())
+    assert rel_err(to_np(run_fwd(gpu, a, b)), h) <= FP32_BAR
+    ga, gb = oracle.bwd(a.numpy(), h, gh.numpy())
+    got_ga, got_gb = run_bwd(gpu, a, torch.from_numpy(h), gh)
+    assert rel_err(to_np(got_gb), gb) <= FP32_BAR
+    assert rel_err(to_np(got_ga), ga) <= FP32_BAR
+
+
+def test_unaligned_base_pointers(gpu):
+    # Views that start 4 bytes into an allocation: the library must fall back to
+    # element-wise loads, not fault or misread.
+    g = seeded(21)
+    rows, T = 9, 512
+    a = torch.rand((rows, T), generator=g)
+    b = torch.randn((rows, T), generator=g)
+    gh = torch.randn((rows, T), generator=g)
+
+    def offset_copy(x):
+        return torch.empty(rows * T + 1, device=gpu)[1:].view(rows, T).copy_(x)
+
+    da, db, dgh = offset_copy(a), offset_copy(b), offset_copy(gh)
+    assert da.data_ptr() % 16 == 4
+    out = torch.empty(rows * T + 1, device=gpu)[1:].view(rows, T)
+    hip.scan_forward_out(da, db, out)
+    h = oracle.fwd(a.numpy(), b.numpy())
+    assert rel_err(to_np(out), h) <= FP32_BAR
+    oga = torch.empty(rows * T + 1, device=gpu)[1:].view(rows, T)
+    ogb = torch.empty(rows * T + 1, device=gpu)[1:].view(rows, T)
+    hip.scan_backward_out(da, out, dgh, oga, ogb)
+    ga, gb = oracle.bwd(a.numpy(), to_np(out), gh.numpy())
+    assert rel_err(to_np(ogb), gb) <= FP32_BAR and rel_err(to_np(oga), ga) <= FP32_BAR
+
+
+def test_closed_forms_at_full_size(gpu):
+    # Size-independent properties at the Mamba-like shape [8, 2048, 4096].
+    shape = (8, 2048, 4096)
+    g = torch.Generator(device=gpu).manual_seed(3)
+    b = torch.randn(shape, generator=g, device=gpu)
+    zero, one = torch.zeros_like(b), torch.ones_like(b)
+    # gate 0: h = b exactly; backward: gb = gh exactly, ga[..., 0] = 0.
+    assert torch.equal(hip.linear_scan_forward(zero, b), b)
+    ga, gb = hip.linear_scan_backward(zero, b, b)
+    assert torch.equal(gb, b)
+    assert torch.equal(ga[..., 0], torch.zeros_like(ga[..., 0]))
+    assert torch.equal(ga[..., 1:], b[..., 1:] * b[..., :-1])
+    # value 0: h = 0 exactly.
+    assert torch.equal(hip.linear_scan_forward(torch.rand_like(b), zero), zero)
+    # gate 1: running sum (compare with a float64 cumsum).
+    h = hip.linear_scan_forward(one, b)
+    want = torch.cumsum(b.double(), dim=-1)
+    assert float((h.double() - want).abs().max()) <= 2e-3
+    ga, gb = hip.linear_scan_backward(one, b, b)
+    want = torch.flip(torch.cumsum(torch.flip(b.double(), [-1]), dim=-1), [-1])
+    assert float((gb.double() - want).abs().max()) <= 2e-3
+    # Linearity in the value: scan(a, b1 + 2*b2) = scan(a, b1) + 2*scan(a, b2).
+    a = torch.rand_like(b)
+    b2 = torch.randn(shape, generator=g, device=gpu)
+    lhs = hip.linear_scan_forward(a, b + 2 * b2)
+    rhs = hip.linear_scan_forward(a, b) + 2 * hip.linear_scan_forward(a, b2)
+    assert float((lhs - rhs).abs().max()) <= 1e-4
+
+
+def test_long_rows_restart_property(gpu):
+    # Scanning [0, k) and then [k, T) from the carried state equals scanning [0, T):
+    # h[k:] = scan(a[k:], b[k:] with b[k] += a[k] * h[k-1]). Exercises the look-back
+    # chain at 2^20 +- 1 without the CPU in the loop.
+    g = torch.Generator(device=gpu).manual_seed(4)
+    for T in ((1 << 20) - 1, 1 << 20, (1 << 20) + 4):
+        a = 0.9 + 0.1 * torch.rand((3, T), generator=g, device=gpu)
+        b = torch.randn((3, T), generator=g, device=gpu)
+        full = hip.linear_scan_forward(a, b)
+        k = 300000
+        b_tail = b[:, k:].clone()
+        b_tail[:, 0] += a[:, k] * full[:, k - 1]
+        tail = hip.linear_scan_forward(a[:, k:].contiguous(), b_tail)
+        assert float((tail - full[:, k:]).abs().max()) <= 1e-4
+
+
+def test_results_do_not_depend_on_timing(gpu):
+    # Same launch twice: bit-identical, look-back included.
+    g = torch.Generator(device=gpu).manual_seed(5)
+    a = 0.9 + 0.1 * torch.rand((5, 300001), generator=g, device=gpu)
+    b = torch.randn(a.shape, generator=g, device=gpu)
+    for plan in (None, hip.Plan(mode=hip.MODE_LOOKBACK, vec=1, unroll=1, waves=1)):
+        first = hip.linear_scan_forward(a, b, plan)
+        for _ in range(3):
+            assert torch.equal(hip.linear_scan_forward(a, b, plan), first)
+        ga0, gb0 = hip.linear_scan_backward(a, first, b, plan)
+        ga1, gb1 = hip.linear_scan_backward(a, first, b, plan)
+        assert torch.equal(ga0, ga1) and torch.equal(gb0, gb1)
+
+
+def test_nonfinite_rows_do_not_leak_into_other_rows(gpu):
+    a = torch.rand(6, 1024)
+    b = torch.randn(6, 1024)
+    b[2, 100] = float("inf")
+    b[4, 7] = float("nan")
+    h = to_np(run_fwd(gpu, a, b))
+    want = oracle.fwd(a.numpy(), b.numpy())
+    for r in (0, 1, 3, 5):
+        assert np.all(np.isfinite(h[r])) and rel_err(h[r], want[r]) <= FP32_BAR
+    assert np.all(np.isfinite(h[2, :100])) and not np.any(np.isfinite(h[2, 100:110]))
+    assert np.all(np.isnan(h[4, 7:]))

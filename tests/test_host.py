@@ -1,0 +1,104 @@
+"""
+Host-side logic that needs no GPU: the flattening decorators, the
+channels-last probe, the tensor-level loop and the autograd op on CPU tensors,
+each checked against the CPU oracle (shapes of scanscam/cpu_test.py:14).
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import scanscam_amd
+from scanscam_amd import baseline, decorator, hip, op
+
+GRID = [(32, 5), (16, 2, 5), (32, 64), (1, 257), (3, 2, 2, 9)]
+
+
+@pytest.mark.parametrize("shape", GRID)
+@pytest.mark.parametrize("permute", [False, True])
+def test_tensor_loop_matches_oracle(shape, permute):
+    g = torch.Generator().manual_seed(11)
+    a = torch.randn(shape, generator=g)
+    b = torch.randn(shape, generator=g)
+    gh = torch.randn(shape, generator=g)
+    if permute:
+        a = a.mT.contiguous().mT  # same values, not contiguous (scanscam/cpu_test.py:21-22)
+        assert not a.is_contiguous() or a.shape[-1] == 1 or a.shape[-2] == 1
+    h = baseline.naive_linear_scan_forward(a, b)
+    assert h.shape == a.shape
+    want = oracle.fwd(a.numpy(), b.numpy())
+    assert np.allclose(h.numpy(), want, rtol=1e-5, atol=1e-4)
+    ga, gb = baseline.naive_linear_scan_backward(a, h, gh)
+    wga, wgb = oracle.bwd(a.numpy(), h.numpy(), gh.numpy())
+    assert np.allclose(ga.numpy(), wga, rtol=1e-5, atol=1e-4)
+    assert np.allclose(gb.numpy(), wgb, rtol=1e-5, atol=1e-4)
+
+
+def test_scan_autograd_on_cpu_tensors_returns_both_gradients():
+    g = torch.Generator().manual_seed(12)
+    a = torch.rand((4, 3, 20), generator=g, dtype=torch.float64, requires_grad=True)
+    b = torch.randn((4, 3, 20), generator=g, dtype=torch.float64, requires_grad=True)
+    gh = torch.randn((4, 3, 20), generator=g, dtype=torch.float64)
+    h = scanscam_amd.scan(a, b)
+    h.backward(gh)
+    wga, wgb = oracle.bwd(a.detach().numpy(), h.detach().numpy(), gh.numpy())
+    assert np.allclose(a.grad.numpy(), wga, rtol=1e-12, atol=1e-12)
+    assert np.allclose(b.grad.numpy(), wgb, rtol=1e-12, atol=1e-12)
+    assert torch.autograd.gradcheck(scanscam_amd.scan, (a, b), eps=1e-6, atol=1e-6)
+
+
+def test_decorators_check_shapes():
+    calls = []
+
+    @decorator.preprocess_scan_args
+    def f(x, y):
+        calls.append((tuple(x.shape), tuple(y.shape)))
+        return x + y
+
+    out = f(torch.zeros(2, 3, 4), torch.ones(2, 3, 4))
+    assert out.shape == (2, 3, 4) and calls == [((6, 4), (6, 4))]
+    with pytest.raises(AssertionError):
+        f(torch.zeros(2, 3), torch.zeros(3, 2))
+    with pytest.raises(AssertionError):
+        f(torch.zeros(5), torch.zeros(5))
+
+    @decorator.preprocess_backward_scan_args
+    def gfn(x, y, z):
+        return x * 2, z * 3
+
+    p, q = gfn(torch.ones(2, 3, 4), torch.ones(2, 3, 4), torch.ones(2, 3, 4))
+    assert p.shape == q.shape == (2, 3, 4) and float(q[0, 0, 0]) == 3.0
+    with pytest.raises(AssertionError):
+        gfn(torch.ones(2, 4), torch.ones(2, 4), torch.ones(2, 5))
+
+
+def test_is_transpose_contig():
+    x = torch.zeros(2, 5, 3)
+    assert not op.is_transpose_contig(x)
+    assert op.is_transpose_contig(x.mT)
+    assert not op.is_transpose_contig(torch.zeros(5, 3).mT)       # 2-D never qualifies
+    assert not op.is_transpose_contig(torch.zeros(2, 2, 5, 3).mT)  # nor 4-D
+    assert scanscam_amd.is_transpose_contig is op.is_transpose_contig
+
+
+def test_gpu_entry_points_reject_cpu_tensors_and_unknown_dtypes():
+    x = torch.zeros(2, 8)
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        hip.blocked_linear_scan_forward(x, x)
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        hip.blocked_linear_scan_backward(x, x, x)
+    with pytest.raises(TypeError):
+        hip.resolve_plan(4, 8, torch.float64)
+
+
+def test_package_never_imports_the_oracle():
+    import os
+    import re
+
+    root = os.path.dirname(os.path.abspath(scanscam_amd.__file__))
+    for dirpath, _, files in os.walk(root):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert not re.search(r"^\s*(import|from)\s+oracle\b", text, flags=re.M), f
+                assert "scan_oracle" not in text, f

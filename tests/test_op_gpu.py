@@ -1,0 +1,103 @@
+"""
+The autograd op end to end on the GPU: scan(gate, value) and .backward(),
+N-D and non-contiguous inputs, channels-last views, and the dispatch rule that
+a GPU tensor is only ever scanned by the HIP kernels.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import scanscam_amd
+from scanscam_amd import hip, op
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_err(x, ref):
+    x, ref = np.asarray(x, np.float64), np.asarray(ref, np.float64)
+    return float(np.max(np.abs(x - ref) / np.maximum(np.abs(ref), 1.0)))
+
+
+@pytest.mark.parametrize("shape", [(4, 256), (3, 5, 1024), (2, 3, 4, 68), (1, 8192)])
+def test_scan_forward_backward_matches_oracle(gpu, shape):
+    g = torch.Generator().manual_seed(31 + len(shape))
+    a = torch.rand(shape, generator=g)
+    b = torch.randn(shape, generator=g)
+    gh = torch.randn(shape, generator=g)
+    da = a.to(gpu).requires_grad_()
+    db = b.to(gpu).requires_grad_()
+    h = scanscam_amd.scan(da, db)
+    assert h.shape == da.shape and h.device == da.device and h.requires_grad
+    h.backward(gh.to(gpu))
+    want_h = oracle.fwd(a.numpy(), b.numpy())
+    assert rel_err(h.detach().cpu().numpy(), want_h) <= 1e-5
+    wga, wgb = oracle.bwd(a.numpy(), h.detach().cpu().numpy(), gh.numpy())
+    assert rel_err(da.grad.cpu().numpy(), wga) <= 1e-5
+    assert rel_err(db.grad.cpu().numpy(), wgb) <= 1e-5
+
+
+def test_scan_gradients_match_finite_differences(gpu):
+    # Directional derivative of sum(h * w) in float32 with a coarse step.
+    g = torch.Generator().manual_seed(41)
+    a = torch.rand((3, 40), generator=g).to(gpu).requires_grad_()
+    b = torch.randn((3, 40), generator=g).to(gpu).requires_grad_()
+    w = torch.randn((3, 40), generator=g).to(gpu)
+    da = torch.randn((3, 40), generator=g).to(gpu)
+    db = torch.randn((3, 40), generator=g).to(gpu)
+    (scanscam_amd.scan(a, b) * w).sum().backward()
+    analytic = float((a.grad * da).sum() + (b.grad * db).sum())
+    eps = 1e-3
+    with torch.no_grad():
+        up = (scanscam_amd.scan(a + eps * da, b + eps * db).double() * w).sum()
+        dn = (scanscam_amd.scan(a - eps * da, b - eps * db).double() * w).sum()
+    numeric = float((up - dn) / (2 * eps))
+    assert abs(analytic - numeric) <= 2e-2 * max(1.0, abs(numeric))
+
+
+def test_channels_last_and_noncontiguous_inputs(gpu):
+    g = torch.Generator().manual_seed(51)
+    base_a = torch.rand((3, 200, 24), generator=g)   # stored [B, T, C]
+    base_b = torch.randn((3, 200, 24), generator=g)
+    a, b = base_a.mT, base_b.mT                      # logical [B, C, T]
+    assert op.is_transpose_contig(a)
+    da = a.to(gpu)
+    da = da.mT.contiguous().mT  # keep the channels-last strides on the device
+    db = b.to(gpu).mT.contiguous().mT
+    assert op.is_transpose_contig(da) and op.is_transpose_contig(db)
+    da.requires_grad_()
+    db.requires_grad_()
+    h = scanscam_amd.scan(da, db)
+    want = oracle.fwd(a.contiguous().numpy(), b.contiguous().numpy())
+    assert rel_err(h.detach().cpu().numpy(), want) <= 1e-5
+    gh = torch.randn((3, 24, 200), generator=g)
+    h.backward(gh.to(gpu))
+    wga, wgb = oracle.bwd(a.contiguous().numpy(), h.detach().cpu().numpy(), gh.numpy())
+    assert rel_err(da.grad.cpu().numpy(), wga) <= 1e-5
+    assert rel_err(db.grad.cpu().numpy(), wgb) <= 1e-5
+
+
+def test_wrapper_names_of_the_reference(gpu):
+    a = torch.rand(4, 128, device=gpu)
+    b = torch.randn(4, 128, device=gpu)
+    h = hip.blocked_linear_scan_forward(a, b)
+    ga, gb = hip.blocked_linear_scan_backward(a, h, b)
+    assert h.shape == ga.shape == gb.shape == (4, 128)
+    with pytest.raises(AssertionError):
+        hip.blocked_linear_scan_forward(a, b[:, :64])
+    with pytest.raises(TypeError):
+        hip.blocked_linear_scan_forward(a.double(), b.double())
+
+
+def test_runs_on_the_current_stream(gpu):
+    s = torch.cuda.Stream(device=gpu)
+    a = torch.rand(64, 4096, device=gpu)
+    b = torch.randn(64, 4096, device=gpu)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s):
+        h = scanscam_amd.scan(a, b)
+        total = h.sum()
+    s.synchronize()
+    want = oracle.fwd(a.cpu().numpy(), b.cpu().numpy())
+    assert rel_err(h.cpu().numpy(), want) <= 1e-5
+    assert np.isfinite(float(total))
