@@ -27,7 +27,10 @@ def _check_same_shape(*tensors: torch.Tensor) -> torch.Size:
 
 
 def _as_rows(t: torch.Tensor) -> torch.Tensor:
-    return t.reshape(-1, t.shape[-1])
+    rows = 1
+    for d in t.shape[:-1]:
+        rows *= d
+    return t.reshape(rows, t.shape[-1])  # explicit row count: also valid when T == 0
 
 
 def preprocess_scan_args(fn: ScanFn) -> ScanFn:
