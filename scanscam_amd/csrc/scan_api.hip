@@ -4,9 +4,12 @@
 
 #include "scan_launch.hpp"
 
+#include <stdlib.h>
+
 namespace {
 
-using scanscam::kDescBase;
+using scanscam::kCounterStride;
+using scanscam::kMaxCounters;
 using scanscam::kDescWords;
 using scanscam::kModeLookback;
 using scanscam::kModeRow;
@@ -54,6 +57,7 @@ struct Resolved {
     Launch l;
     int nch;
     int tiles_per_row;
+    int counters;
     size_t ws_bytes;
 };
 
@@ -80,6 +84,7 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
     const int nch = (int)nch64;
     out->nch = nch;
     out->tiles_per_row = 0;
+    out->counters = 1;
     out->ws_bytes = 0;
     if (rows == 0 || T == 0) return SCANSCAM_OK;
 
@@ -124,13 +129,23 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
         const int rows_per_wg = l.waves / l.wpr;
         l.grid = (rows + rows_per_wg - 1) / rows_per_wg;
     } else if (l.mode == kModeLookback) {
+        // Tiles of 32 chunks (8192 fp32 elements): fewer, larger tiles keep the
+        // carry chain short relative to the time a tile spends on its data.
         l.unroll = u.unroll ? u.unroll : 4;
-        l.waves = u.waves ? u.waves : 4;
+        l.waves = u.waves ? u.waves : 8;
         const int tile_chunks = l.waves * l.unroll;
         out->tiles_per_row = (nch + tile_chunks - 1) / tile_chunks;
-        l.grid = rows * (int64_t)out->tiles_per_row;
+        // One ticket counter per row up to kMaxCounters; when rows do not divide
+        // evenly every counter gets the grid share of the fullest one.
+        out->counters = (int)(rows < kMaxCounters ? rows : kMaxCounters);
+#ifdef SCANSCAM_EXPERIMENT
+        if (const char *e = getenv("SCANSCAM_COUNTERS")) out->counters = atoi(e) < rows ? atoi(e) : (int)rows;
+#endif
+        const int64_t rows_per_counter = (rows + out->counters - 1) / out->counters;
+        const int64_t tiles = rows * (int64_t)out->tiles_per_row;
+        l.grid = (int64_t)out->counters * rows_per_counter * out->tiles_per_row;
         if (l.grid >= (int64_t(1) << 31)) return SCANSCAM_EINVAL;
-        out->ws_bytes = (size_t)(kDescBase + l.grid * kDescWords) * sizeof(uint64_t);
+        out->ws_bytes = (size_t)((int64_t)out->counters * kCounterStride + tiles * kDescWords) * sizeof(uint64_t);
     } else {
         return SCANSCAM_EPLAN;
     }
@@ -177,6 +192,8 @@ int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y
     args.wpr = r.l.wpr;
     args.group = r.l.group;
     args.tiles_per_row = r.tiles_per_row;
+    args.counters = r.counters;
+    args.desc_base = r.counters * kCounterStride;
     args.ws = nullptr;
 
     hipStream_t s = static_cast<hipStream_t>(stream);

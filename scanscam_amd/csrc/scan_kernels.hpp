@@ -40,6 +40,9 @@
 #ifndef SCANSCAM_NT_STORE
 #define SCANSCAM_NT_STORE 1
 #endif
+#ifndef SCANSCAM_TICKET_BY_BLOCKIDX
+#define SCANSCAM_TICKET_BY_BLOCKIDX 0
+#endif
 
 namespace scanscam {
 
@@ -61,17 +64,25 @@ struct ScanArgs {
     int32_t wpr;            // ROW: waves cooperating on one row
     int32_t group;          // SMALL: lanes per row (power of two, <= 64)
     int32_t tiles_per_row;  // LOOKBACK: tiles per row
-    uint64_t *ws;           // LOOKBACK: ticket counter + tile descriptors
+    int32_t counters;       // LOOKBACK: number of ticket counters (row r uses counter r % counters)
+    int32_t desc_base;      // LOOKBACK: first descriptor word of the workspace
+    uint64_t *ws;           // LOOKBACK: ticket counters + tile descriptors
 };
 
-// Look-back workspace layout, in 64-bit words. Word 0 is the ticket counter,
-// word 1 is raised if a look-back wait ever expired (results are then NaN);
-// each tile owns kDescWords words from kDescBase on:
+// Look-back workspace layout, in 64-bit words. Ticket counter c is word
+// c * kCounterStride (one counter per 128-byte line, so that counters do not
+// serialise on one another); word 1 is raised if a look-back wait ever expired
+// (results are then NaN); each tile owns kDescWords words from
+// counters * kCounterStride on:
 //   [0] {1, bits(A)}  [1] {1, bits(B)}   the tile's own aggregate
 //   [2] {1, bits(h)}                     the scan value at the tile's end
 // The upper half is a ready flag; the workspace is zeroed before each launch,
 // so every word is self-validating and no fence is needed around it.
-constexpr int kDescBase = 8;
+#ifndef SCANSCAM_CTR_STRIDE
+#define SCANSCAM_CTR_STRIDE 16
+#endif
+constexpr int kCounterStride = SCANSCAM_CTR_STRIDE;
+constexpr int kMaxCounters = 256;
 constexpr int kDescWords = 4;
 
 // ---------------------------------------------------------------------------
@@ -423,10 +434,12 @@ __global__ __launch_bounds__(MAXT) void scan_small_kernel(const ScanArgs p)
 
 // ---------------------------------------------------------------------------
 // LOOKBACK kernel: the tiles of a row are spread over workgroups. Tiles are
-// handed out by an atomic ticket, so every tile a workgroup may wait for was
-// taken by a workgroup that is already running. Ticket k works on row
-// k % rows, tile k / rows, which keeps the tiles in flight at any moment
-// spread over all rows.
+// handed out by atomic tickets, so every tile a workgroup may wait for was
+// taken by a workgroup that is already running. A single counter would
+// serialise the whole grid on one address, so there are up to kMaxCounters of
+// them, each serving the rows r with r % counters == c: ticket k of a counter
+// works on its (k % rows_here)-th row, tile k / rows_here, which keeps the
+// tiles in flight at any moment spread over all rows.
 //
 // Carry protocol (wave 0 of the workgroup): publish the tile's aggregate
 // (A, B); 64 lanes inspect the 64 preceding tiles of the row at once; the
@@ -512,13 +525,23 @@ __global__ __launch_bounds__(MAXT) void scan_lookback_kernel(const ScanArgs p)
     const int wave = threadIdx.x / kWave;
     const int nwaves = blockDim.x / kWave;
 
+    // Counter c serves the rows r with r % counters == c; its tickets walk those
+    // rows round-robin, tile by tile.
+    const int nctr = p.counters;
+    const int ctr = blockIdx.x % nctr;
+#if SCANSCAM_TICKET_BY_BLOCKIDX
+    if (threadIdx.x == 0) lds_ticket = blockIdx.x / nctr;
+#else
     if (threadIdx.x == 0)
-        lds_ticket = __hip_atomic_fetch_add(reinterpret_cast<unsigned *>(p.ws), 1u, __ATOMIC_RELAXED,
-                                            __HIP_MEMORY_SCOPE_AGENT);
+        lds_ticket = __hip_atomic_fetch_add(reinterpret_cast<unsigned *>(p.ws + (int64_t)ctr * kCounterStride), 1u,
+                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#endif
     __syncthreads();
     const unsigned ticket = lds_ticket;
-    const int64_t row = ticket % (uint64_t)p.rows;
-    const int tile = (int)(ticket / (uint64_t)p.rows);
+    const int64_t rows_here = (p.rows - ctr + nctr - 1) / nctr;
+    if ((int64_t)ticket >= rows_here * p.tiles_per_row) return;  // surplus workgroup of an uneven split
+    const int64_t row = ctr + (int64_t)nctr * (ticket % (uint64_t)rows_here);
+    const int tile = (int)(ticket / (uint64_t)rows_here);
     const int64_t row_off = row * (int64_t)p.T;
     const int nvp = p.nch * kWave;
     const int chunk0 = (tile * nwaves + wave) * U;
@@ -551,7 +574,7 @@ __global__ __launch_bounds__(MAXT) void scan_lookback_kernel(const ScanArgs p)
             TB = __builtin_fmaf(lds_A[q], TB, lds_B[q]);
             TA = lds_A[q] * TA;
         }
-        uint64_t *row_desc = p.ws + kDescBase + row * (int64_t)p.tiles_per_row * kDescWords;
+        uint64_t *row_desc = p.ws + p.desc_base + row * (int64_t)p.tiles_per_row * kDescWords;
         uint64_t *mine = row_desc + (int64_t)tile * kDescWords;
         float cin = 0.0f;
         if (tile > 0) {

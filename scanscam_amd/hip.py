@@ -20,7 +20,8 @@ import torch
 from .decorator import preprocess_backward_scan_args, preprocess_scan_args
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libscanscam_hip.so")
+# SCANSCAM_HIP_LIB points at another build of the same ABI (tuning builds).
+LIB_PATH = os.environ.get("SCANSCAM_HIP_LIB") or os.path.join(_HERE, "libscanscam_hip.so")
 
 MODE_AUTO, MODE_SMALL, MODE_ROW, MODE_LOOKBACK = 0, 1, 2, 3
 FORWARD, BACKWARD = 0, 1

@@ -119,5 +119,6 @@ def test_automatic_plan_per_regime(rows, T, dtype, mode, vec):
 
 def test_lookback_workspace_size_formula():
     plan = hip.Plan(mode=hip.MODE_LOOKBACK, vec=4, unroll=2, waves=2)
-    # tile = 2 waves * 2 chunks * 256 elements = 1024 elements; 5 tiles per row of 4100.
-    assert hip.workspace_bytes(3, 4100, torch.float32, hip.FORWARD, plan) == (8 + 3 * 5 * 4) * 8
+    # tile = 2 waves * 2 chunks * 256 elements = 1024 elements; 5 tiles per row of 4100;
+    # one ticket counter (a 16-word line) per row, 4 words per tile descriptor.
+    assert hip.workspace_bytes(3, 4100, torch.float32, hip.FORWARD, plan) == (3 * 16 + 3 * 5 * 4) * 8
