@@ -10,7 +10,9 @@ namespace {
 
 using scanscam::kCounterStride;
 using scanscam::kMaxCounters;
-using scanscam::kDescWords;
+using scanscam::kSuper;
+using scanscam::kSuperWords;
+using scanscam::kTileWords;
 using scanscam::kModeLookback;
 using scanscam::kModeRow;
 using scanscam::kModeSmall;
@@ -58,6 +60,7 @@ struct Resolved {
     int nch;
     int tiles_per_row;
     int counters;
+    int64_t super_base;  // word offset of the super-tile descriptors
     size_t ws_bytes;
 };
 
@@ -85,6 +88,7 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
     out->nch = nch;
     out->tiles_per_row = 0;
     out->counters = 1;
+    out->super_base = 0;
     out->ws_bytes = 0;
     if (rows == 0 || T == 0) return SCANSCAM_OK;
 
@@ -145,7 +149,9 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
         const int64_t tiles = rows * (int64_t)out->tiles_per_row;
         l.grid = (int64_t)out->counters * rows_per_counter * out->tiles_per_row;
         if (l.grid >= (int64_t(1) << 31)) return SCANSCAM_EINVAL;
-        out->ws_bytes = (size_t)((int64_t)out->counters * kCounterStride + tiles * kDescWords) * sizeof(uint64_t);
+        const int64_t supers = rows * (int64_t)((out->tiles_per_row + kSuper - 1) / kSuper);
+        out->super_base = (int64_t)out->counters * kCounterStride + tiles * kTileWords;
+        out->ws_bytes = (size_t)(out->super_base + supers * kSuperWords) * sizeof(uint64_t);
     } else {
         return SCANSCAM_EPLAN;
     }
@@ -194,6 +200,7 @@ int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y
     args.tiles_per_row = r.tiles_per_row;
     args.counters = r.counters;
     args.desc_base = r.counters * kCounterStride;
+    args.super_base = r.super_base;
     args.ws = nullptr;
 
     hipStream_t s = static_cast<hipStream_t>(stream);

@@ -40,6 +40,9 @@
 #ifndef SCANSCAM_NT_STORE
 #define SCANSCAM_NT_STORE 1
 #endif
+#ifndef SCANSCAM_XCD_REMAP
+#define SCANSCAM_XCD_REMAP 0
+#endif
 #ifndef SCANSCAM_TICKET_BY_BLOCKIDX
 #define SCANSCAM_TICKET_BY_BLOCKIDX 0
 #endif
@@ -65,25 +68,24 @@ struct ScanArgs {
     int32_t group;          // SMALL: lanes per row (power of two, <= 64)
     int32_t tiles_per_row;  // LOOKBACK: tiles per row
     int32_t counters;       // LOOKBACK: number of ticket counters (row r uses counter r % counters)
-    int32_t desc_base;      // LOOKBACK: first descriptor word of the workspace
+    int32_t desc_base;      // LOOKBACK: first tile-descriptor word of the workspace
+    int64_t super_base;     // LOOKBACK: first super-tile-descriptor word of the workspace
     uint64_t *ws;           // LOOKBACK: ticket counters + tile descriptors
 };
 
 // Look-back workspace layout, in 64-bit words. Ticket counter c is word
 // c * kCounterStride (one counter per 128-byte line, so that counters do not
 // serialise on one another); word 1 is raised if a look-back wait ever expired
-// (results are then NaN); each tile owns kDescWords words from
-// counters * kCounterStride on:
-//   [0] {1, bits(A)}  [1] {1, bits(B)}   the tile's own aggregate
-//   [2] {1, bits(h)}                     the scan value at the tile's end
-// The upper half is a ready flag; the workspace is zeroed before each launch,
-// so every word is self-validating and no fence is needed around it.
+// (results are then NaN). Then come kTileWords words per tile (its aggregate)
+// and kSuperWords words per super-tile of 64 tiles (its aggregate and its end
+// value). Each word is {1, bits(float)}: the upper half is a ready flag and the
+// workspace is zeroed before each launch, so every word is self-validating and
+// no fence is needed around it.
 #ifndef SCANSCAM_CTR_STRIDE
 #define SCANSCAM_CTR_STRIDE 16
 #endif
 constexpr int kCounterStride = SCANSCAM_CTR_STRIDE;
 constexpr int kMaxCounters = 256;
-constexpr int kDescWords = 4;
 
 // ---------------------------------------------------------------------------
 // Storage types: float, __bf16, _Float16. All arithmetic is fp32.
@@ -231,9 +233,13 @@ struct WaveTile {
                 if (valid[u]) rh[u] = V::load(h + off[u]);
                 edge_a[u] = 0.0f;
                 edge_h[u] = 0.0f;
-                // Neighbours that no lane of this group holds.
-                if (valid[u] && j == 0 && (m[u] + 1) * VEC < p.T) edge_a[u] = (float)a[off[u] + VEC];
-                if (valid[u] && j == jlast && m[u] > 0) edge_h[u] = (float)h[off[u] - 1];
+                // Neighbours that no lane of this group holds. With CHAIN the chunks of a
+                // wave are adjacent, so only the wave's outer borders need memory: the
+                // inner ones are taken from the neighbouring chunk's registers in reduce().
+                const bool need_a = !CHAIN || u == 0;
+                const bool need_h = !CHAIN || u == U - 1;
+                if (need_a && valid[u] && j == 0 && (m[u] + 1) * VEC < p.T) edge_a[u] = (float)a[off[u] + VEC];
+                if (need_h && valid[u] && j == jlast && m[u] > 0) edge_h[u] = (float)h[off[u] - 1];
             }
         }
     }
@@ -241,6 +247,19 @@ struct WaveTile {
     // Builds (gate, value) per element in scan order and reduces them.
     __device__ __forceinline__ void reduce(int j, int jlast, float (&hp)[REV ? U : 1][VEC])
     {
+        // Backward: a[first element] and h[last element] of every chunk's vectors,
+        // for the lanes at the borders between the chunks of this wave.
+        float first_a[REV ? U : 1], last_h[REV ? U : 1];
+        if (REV && CHAIN) {
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                float t[VEC];
+                V::unpack(ra[u], t);
+                first_a[u] = t[0];
+                V::unpack(rh[u], t);
+                last_h[u] = t[VEC - 1];
+            }
+        }
 #pragma unroll
         for (int u = 0; u < U; u++) {
             float fa[VEC], fx[VEC];
@@ -260,8 +279,11 @@ struct WaveTile {
                 // end of the row reads as gate 0, which is what t = T-1 needs.
                 float a_next = lane_prev(fa[0], 0.0f);        // lane-1 holds vector m+1
                 float h_prev = lane_next(fh[VEC - 1], 0.0f);  // lane+1 holds vector m-1
-                a_next = (j == 0) ? edge_a[u] : a_next;
-                h_prev = (j == jlast) ? edge_h[u] : h_prev;
+                float border_a = edge_a[u], border_h = edge_h[u];
+                if (CHAIN && u > 0) border_a = read_lane(first_a[u - 1], kWave - 1);
+                if (CHAIN && u + 1 < U) border_h = read_lane(last_h[u + 1], 0);
+                a_next = (j == 0) ? border_a : a_next;
+                h_prev = (j == jlast) ? border_h : h_prev;
 #pragma unroll
                 for (int k = 0; k < VEC; k++) {
                     const float gk = (k == 0) ? a_next : fa[(VEC - k) % VEC];
@@ -355,7 +377,14 @@ __global__ __launch_bounds__(MAXT) void scan_row_kernel(const ScanArgs p)
     const int rows_per_wg = nwaves / wpr;
     const int wr = wave % wpr;          // this wave's place among the row's waves
     const int wbase = wave - wr;        // first wave of the row's group
-    const int64_t row = (int64_t)blockIdx.x * rows_per_wg + wave / wpr;
+#if SCANSCAM_XCD_REMAP
+    // Workgroups go round-robin to the 8 XCDs: give each XCD one contiguous eighth of the rows.
+    const unsigned nb = gridDim.x;
+    const unsigned bid = (nb % 8 == 0) ? (blockIdx.x % 8) * (nb / 8) + blockIdx.x / 8 : blockIdx.x;
+#else
+    const unsigned bid = blockIdx.x;
+#endif
+    const int64_t row = (int64_t)bid * rows_per_wg + wave / wpr;
     const bool row_ok = row < p.rows;
     const int64_t row_off = row_ok ? row * (int64_t)p.T : 0;
     const int nvp = p.nch * kWave;      // vectors per row, padded to whole chunks
@@ -441,13 +470,29 @@ __global__ __launch_bounds__(MAXT) void scan_small_kernel(const ScanArgs p)
 // works on its (k % rows_here)-th row, tile k / rows_here, which keeps the
 // tiles in flight at any moment spread over all rows.
 //
-// Carry protocol (wave 0 of the workgroup): publish the tile's aggregate
-// (A, B); 64 lanes inspect the 64 preceding tiles of the row at once; the
-// nearest one that has published its end value h gives the start, and the
-// aggregates of the tiles between it and this one are applied to it one FMA
-// at a time, oldest first. That is the same chain of FMAs whichever tile
-// happens to be the nearest published one, so results do not depend on timing.
+// Carry protocol, two levels, run by wave 0 of the workgroup. 64 consecutive
+// tiles of a row form a super-tile. Let (A_q, B_q) be the aggregate of tile q
+// of super-tile m, (SA_m, SB_m) the composition of all 64 of them and S_m the
+// scan value entering the super-tile (S_0 = 0).
+//   tile level   tile j publishes (A_j, B_j), collects those of tiles 0..j-1 of
+//                its own super-tile (one per lane), and scans them with the
+//                wave ladder: its carry-in is P_{j-1}(S_m). Tile 63 thereby
+//                also has (SA_m, SB_m), and publishes it at once.
+//   super level  64 lanes inspect the 64 preceding super-tiles; the nearest
+//                one with a published end value SI_s = fma(SA_s, S_s, SB_s)
+//                starts a chain of FMAs through the aggregates of the
+//                super-tiles after it, oldest first, which ends in S_m. Tile 63
+//                then publishes SI_m.
+// Nothing waits for a value that itself waited for a predecessor's carry
+// except along the SI chain, which advances 64 tiles per step and can skip
+// over up to 64 super-tiles whose aggregates are known. Every value has one
+// defining expression (S_{m+1} = fma(SA_m, S_m, SB_m), fixed ladder inside a
+// super-tile), so results do not depend on timing.
 // ---------------------------------------------------------------------------
+constexpr int kSuper = 64;       // tiles per super-tile (one per lane)
+constexpr int kTileWords = 2;    // {1, bits(A)}, {1, bits(B)}
+constexpr int kSuperWords = 4;   // {1, bits(SA)}, {1, bits(SB)}, {1, bits(SI)}, unused
+
 __device__ __forceinline__ uint64_t desc_load(const uint64_t *p)
 {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -468,49 +513,98 @@ __device__ __forceinline__ float desc_value(uint64_t w) { return __builtin_bit_c
 constexpr int kSpinLimit = 1 << 20;
 constexpr int kTimeoutWord = 1;
 
-// Returns the scan value entering tile `tile` of the row whose descriptors
-// start at `row_desc`. Called by all 64 lanes of one wave.
-__device__ __forceinline__ float lookback_carry(const uint64_t *row_desc, int tile, int lane, uint64_t *ws)
+// Returns the scan value entering tile `tile` of row `row`, whose own aggregate
+// is (TA, TB). Called by all 64 lanes of one wave; `tile` must be wave-uniform.
+__device__ __forceinline__ float lookback_carry(const ScanArgs &p, int64_t row, int tile, float TA, float TB,
+                                                int lane)
 {
-    const int look = tile - 1 - lane;  // the tile this lane watches
-    bool have_incl = look < 0;         // before the row starts the value is 0
-    bool have_agg = look < 0;
-    float incl = 0.0f, A = 1.0f, B = 0.0f;
+    const int tpr = p.tiles_per_row;
+    const int spr = (tpr + kSuper - 1) / kSuper;
+    const int j = tile % kSuper, m = tile / kSuper;
+    uint64_t *trow = p.ws + p.desc_base + row * (int64_t)tpr * kTileWords;
+    uint64_t *srow = p.ws + p.super_base + row * (int64_t)spr * kSuperWords;
+    const bool closes = (j == kSuper - 1) && (m + 1 < spr);  // a later super-tile needs (SA, SB, SI)
+
+    if (lane == 0 && j < kSuper - 1 && tile + 1 < tpr) {
+        desc_store(trow + (int64_t)tile * kTileWords + 0, TA);
+        desc_store(trow + (int64_t)tile * kTileWords + 1, TB);
+    }
+
+    // Lane q < j collects tile q of this super-tile; lane j holds this tile; the rest the identity.
+    bool have_t = lane >= j;
+    float A = (lane == j) ? TA : 1.0f, B = (lane == j) ? TB : 0.0f;
+    // Lane k watches super-tile m-1-k; before the row starts the value is 0.
+    const int sidx = m - 1 - lane;
+    bool have_si = sidx < 0, have_sa = sidx < 0;
+    float SI = 0.0f, SA = 1.0f, SB = 0.0f;
+
+    bool tiles_done = false, super_done = false;
+    float PA = 1.0f, PB = 0.0f, S = 0.0f;
     for (int spin = 0; spin < kSpinLimit; spin++) {
-        if (look >= 0) {
-            const uint64_t *d = row_desc + (int64_t)look * kDescWords;
-            if (!have_incl) {
+        if (!have_t) {
+            const uint64_t *d = trow + (int64_t)(m * kSuper + lane) * kTileWords;
+            const uint64_t wa = desc_load(d + 0), wb = desc_load(d + 1);
+            if (desc_ready(wa) && desc_ready(wb)) {
+                have_t = true;
+                A = desc_value(wa);
+                B = desc_value(wb);
+            }
+        }
+        if (!have_si || !have_sa) {
+            const uint64_t *d = srow + (int64_t)sidx * kSuperWords;
+            if (!have_si) {
                 const uint64_t wi = desc_load(d + 2);
                 if (desc_ready(wi)) {
-                    have_incl = true;
-                    incl = desc_value(wi);
+                    have_si = true;
+                    SI = desc_value(wi);
                 }
             }
-            if (!have_agg) {
+            if (!have_sa) {
                 const uint64_t wa = desc_load(d + 0), wb = desc_load(d + 1);
                 if (desc_ready(wa) && desc_ready(wb)) {
-                    have_agg = true;
-                    A = desc_value(wa);
-                    B = desc_value(wb);
+                    have_sa = true;
+                    SA = desc_value(wa);
+                    SB = desc_value(wb);
                 }
             }
         }
-        const uint64_t mi = __ballot(have_incl);
-        const uint64_t ma = __ballot(have_agg);
-        if (mi != 0) {
-            const int first = __builtin_ctzll(mi);  // nearest tile with a published end value
-            const uint64_t need = (first == 0) ? 0ull : ((~0ull) >> (64 - first));
-            if ((ma & need) == need) {
-                float c = read_lane(incl, first);
-                for (int q = first - 1; q >= 0; q--)
-                    c = __builtin_fmaf(read_lane(A, q), c, read_lane(B, q));
-                return c;
+        if (!tiles_done && __ballot(have_t) == ~0ull) {
+            tiles_done = true;
+            PA = A;
+            PB = B;
+            wave_scan<false>(PA, PB, lane);
+            if (closes) {
+                const float sa = read_lane(PA, kSuper - 1), sb = read_lane(PB, kSuper - 1);
+                if (lane == 0) {
+                    desc_store(srow + (int64_t)m * kSuperWords + 0, sa);
+                    desc_store(srow + (int64_t)m * kSuperWords + 1, sb);
+                }
             }
         }
+        if (!super_done) {
+            const uint64_t mi = __ballot(have_si);
+            const uint64_t ma = __ballot(have_sa);
+            if (mi != 0) {
+                const int first = __builtin_ctzll(mi);  // nearest super-tile with a published end value
+                const uint64_t need = (first == 0) ? 0ull : ((~0ull) >> (64 - first));
+                if ((ma & need) == need) {
+                    S = read_lane(SI, first);
+                    for (int q = first - 1; q >= 0; q--) S = __builtin_fmaf(read_lane(SA, q), S, read_lane(SB, q));
+                    super_done = true;
+                }
+            }
+        }
+        if (tiles_done && super_done) break;
         __builtin_amdgcn_s_sleep(1);
     }
-    if (lane == 0) __hip_atomic_store(ws + kTimeoutWord, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return __builtin_nanf("");
+    if (!(tiles_done && super_done)) {
+        if (lane == 0) __hip_atomic_store(p.ws + kTimeoutWord, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        S = __builtin_nanf("");
+    }
+    if (closes && lane == 0)
+        desc_store(srow + (int64_t)m * kSuperWords + 2,
+                   __builtin_fmaf(read_lane(PA, kSuper - 1), S, read_lane(PB, kSuper - 1)));
+    return j > 0 ? __builtin_fmaf(read_lane(PA, j - 1), S, read_lane(PB, j - 1)) : S;
 }
 
 template <typename ST, int VEC, int U, bool REV, int MAXT>
@@ -537,7 +631,7 @@ __global__ __launch_bounds__(MAXT) void scan_lookback_kernel(const ScanArgs p)
                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #endif
     __syncthreads();
-    const unsigned ticket = lds_ticket;
+    const unsigned ticket = __builtin_amdgcn_readfirstlane(lds_ticket);
     const int64_t rows_here = (p.rows - ctr + nctr - 1) / nctr;
     if ((int64_t)ticket >= rows_here * p.tiles_per_row) return;  // surplus workgroup of an uneven split
     const int64_t row = ctr + (int64_t)nctr * (ticket % (uint64_t)rows_here);
@@ -574,20 +668,9 @@ __global__ __launch_bounds__(MAXT) void scan_lookback_kernel(const ScanArgs p)
             TB = __builtin_fmaf(lds_A[q], TB, lds_B[q]);
             TA = lds_A[q] * TA;
         }
-        uint64_t *row_desc = p.ws + p.desc_base + row * (int64_t)p.tiles_per_row * kDescWords;
-        uint64_t *mine = row_desc + (int64_t)tile * kDescWords;
         float cin = 0.0f;
-        if (tile > 0) {
-            if (lane == 0) {
-                desc_store(mine + 0, TA);
-                desc_store(mine + 1, TB);
-            }
-            cin = lookback_carry(row_desc, tile, lane, p.ws);
-        }
-        if (lane == 0) {
-            desc_store(mine + 2, __builtin_fmaf(TA, cin, TB));
-            lds_carry = cin;
-        }
+        if (p.tiles_per_row > 1) cin = lookback_carry(p, row, tile, TA, TB, lane);
+        if (lane == 0) lds_carry = cin;
     }
     __syncthreads();
 

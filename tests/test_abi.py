@@ -120,5 +120,5 @@ def test_automatic_plan_per_regime(rows, T, dtype, mode, vec):
 def test_lookback_workspace_size_formula():
     plan = hip.Plan(mode=hip.MODE_LOOKBACK, vec=4, unroll=2, waves=2)
     # tile = 2 waves * 2 chunks * 256 elements = 1024 elements; 5 tiles per row of 4100;
-    # one ticket counter (a 16-word line) per row, 4 words per tile descriptor.
-    assert hip.workspace_bytes(3, 4100, torch.float32, hip.FORWARD, plan) == (3 * 16 + 3 * 5 * 4) * 8
+    # one ticket counter (a 16-word line) per row, 2 words per tile, 4 per super-tile of 64 tiles.
+    assert hip.workspace_bytes(3, 4100, torch.float32, hip.FORWARD, plan) == (3 * 16 + 3 * 5 * 2 + 3 * 1 * 4) * 8
