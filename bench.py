@@ -20,7 +20,8 @@ Prints ONE JSON line. Besides the contract fields it carries
                 restatement in oracle/);
   configs       forward and forward+backward GB/s of the other four synthetic
                 configurations (buffer sets rotated so that the 256 MB
-                Infinity Cache cannot serve them).
+                Infinity Cache cannot serve them; timed as batches of
+                back-to-back launches, gaps included).
 """
 import argparse
 import json
@@ -34,6 +35,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per launch at configs[1] from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by what the same
+# counters read for a copy kernel of known size (profiles/scan_row_f32_fwd_bwd_8x2048x4096_pmc_traffic.txt).
+MEASURED_TRAFFIC = {"fwd": 805.38e6, "bwd": 1366.63e6}
 METRIC = "scan HBM GB/s and % of MI355X peak, fwd and fwd+bwd, fp32 [B,C,T]"
 FWD_BYTES = {4: 12, 2: 6}
 BWD_BYTES = {4: 20, 2: 10}
@@ -87,29 +91,53 @@ class DeviceSet:
 def time_kernels(sets, steps, warmup, hip, torch):
     """Runs (forward; backward) `steps` times, rotating over `sets`.
 
-    Returns (wall seconds per step, mean fwd kernel ms, mean bwd kernel ms),
-    the kernel times from HIP events recorded on the launch stream around each
-    launch.
+    Returns (wall seconds per step, mean fwd kernel ms, mean bwd kernel ms,
+    min fwd ms, min bwd ms); the kernel times come from HIP events recorded on
+    the launch stream around every launch.
     """
+    calls = [(hip.prepare_forward(s.a, s.b, s.h), hip.prepare_backward(s.a, s.h, s.gh, s.ga, s.gb)) for s in sets]
     for i in range(warmup):
-        s = sets[i % len(sets)]
-        hip.scan_forward_out(s.a, s.b, s.h)
-        hip.scan_backward_out(s.a, s.h, s.gh, s.ga, s.gb)
+        f, b = calls[i % len(calls)]
+        f()
+        b()
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(steps):
-        s = sets[i % len(sets)]
+        f, b = calls[i % len(calls)]
         ev[i][0].record()
-        hip.scan_forward_out(s.a, s.b, s.h)
+        f()
         ev[i][1].record()
-        hip.scan_backward_out(s.a, s.h, s.gh, s.ga, s.gb)
+        b()
         ev[i][2].record()
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / steps
     fwd = [e[0].elapsed_time(e[1]) for e in ev]
     bwd = [e[1].elapsed_time(e[2]) for e in ev]
     return wall, statistics.fmean(fwd), statistics.fmean(bwd), min(fwd), min(bwd)
+
+
+def time_batches(sets, launches, warmup, hip, torch):
+    """Mean ms per launch of each direction over `launches` back-to-back launches.
+
+    For kernels of a few microseconds, where an event pair around every launch
+    would cost as much as the launch: two events bracket the whole batch, so the
+    figure includes the gaps between launches.
+    """
+    calls = [(hip.prepare_forward(s.a, s.b, s.h), hip.prepare_backward(s.a, s.h, s.gh, s.ga, s.gb)) for s in sets]
+    out = []
+    for d in (0, 1):
+        for i in range(warmup):
+            calls[i % len(calls)][d]()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for i in range(launches):
+            calls[i % len(calls)][d]()
+        e1.record()
+        torch.cuda.synchronize()
+        out.append(e0.elapsed_time(e1) / launches)
+    return out[0], out[1]
 
 
 def cpu_baseline(a, b, gh, reps):
@@ -230,7 +258,7 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(bwd_gbps / HBM_PEAK_GBPS, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC["bwd"],
             "bytes_per_launch": BWD_BYTES[4] * n,
             "avg_ms": round(bwd_ms, 4),
             "min_ms": round(bwd_min, 4),
@@ -242,7 +270,7 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(fwd_gbps / HBM_PEAK_GBPS, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC["fwd"],
             "bytes_per_launch": FWD_BYTES[4] * n,
             "avg_ms": round(fwd_ms, 4),
             "min_ms": round(fwd_min, 4),
@@ -262,8 +290,7 @@ def main():
             per_set = 6 * cn * esize
             nsets = max(1, min(64, -(-(1 << 30) // per_set)))
             csets = [first] + [first.clone(torch) for _ in range(nsets - 1)]
-            steps = max(args.steps, 2 * nsets)
-            w, f_ms, b_ms, _, _ = time_kernels(csets, steps, max(args.warmup, nsets), hip, torch)
+            f_ms, b_ms = time_batches(csets, max(4 * args.steps, 4 * nsets), max(args.warmup, nsets), hip, torch)
             rows, T = first.a.shape
             others[key] = {
                 "shape": list(ca.shape),
