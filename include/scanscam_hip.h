@@ -110,6 +110,24 @@ size_t scanscam_workspace_bytes_plan(int64_t rows, int64_t T, int dtype, int dir
                                      const scanscam_plan *plan);
 
 /*
+ * Channels-last storage: every tensor is a dense [batch, T, C] array (C
+ * fastest) scanned along T -- the layout of a [batch, C, T] tensor whose last
+ * two dimensions were transposed. Same arithmetic as the calls above.
+ * Replace transposed_linear_scan(gate, value, output, channelsPerBlock),
+ * src/scanscam_cuda.cu:556-582, and transposed_linear_scan_backward(gate,
+ * output, outGrad, gateGradOut, valueGradOut, channelsPerBlock), :687-723. The
+ * reference's trailing tuning argument has its counterpart in `plan` (NULL =
+ * automatic): vec = channels per lane (16/sizeof(storage) or 1), unroll = time
+ * steps per wave per tile (2, 4, 8 for the full vector; 4, 8, 16 for vec 1),
+ * waves = waves per workgroup (1..16); mode and waves_per_row are ignored.
+ * No workspace is needed.
+ */
+int scanscam_scan_fwd_cl(const void *a, const void *b, void *h, int64_t batch, int64_t T, int64_t C, int dtype,
+                         void *stream, const scanscam_plan *plan);
+int scanscam_scan_bwd_cl(const void *a, const void *h, const void *gh, void *ga, void *gb, int64_t batch,
+                         int64_t T, int64_t C, int dtype, void *stream, const scanscam_plan *plan);
+
+/*
  * Writes the plan the automatic choice resolves to for this shape (assuming
  * 16-byte aligned pointers) into *out. Returns 0 or an error code.
  */

@@ -223,6 +223,92 @@ int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y
     return e == hipSuccess ? SCANSCAM_OK : SCANSCAM_ELAUNCH;
 }
 
+// Channels-last: choice of vector width, steps per wave and waves per workgroup.
+int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, int dtype, bool aligned16,
+               scanscam::ClLaunch *l)
+{
+    const int esize = elem_size(dtype);
+    const int full = 16 / esize;
+    scanscam_plan u = {0, 0, 0, 0, 0};
+    if (user) u = *user;
+    const bool vec_possible = aligned16 && (C % full == 0);
+    auto groups = [&](int vec) { return (C + (int64_t)kWave * vec - 1) / ((int64_t)kWave * vec); };
+    if (u.vec) {
+        l->vec = u.vec;
+    } else if (!vec_possible) {
+        l->vec = 1;
+    } else {
+        // A workgroup owns 64*vec channels of one batch element for all of T: prefer the
+        // 16-byte vector unless that leaves most of the GPU without a workgroup.
+        l->vec = (batch * groups(full) >= 256 || groups(1) == groups(full)) ? full : 1;
+    }
+    if (l->vec != 1 && l->vec != full) return SCANSCAM_EPLAN;
+    if (l->vec == full && full != 1 && !vec_possible) return SCANSCAM_EPLAN;
+
+    l->steps = u.unroll ? u.unroll : (l->vec == 1 ? 8 : 4);
+    const bool steps_ok = (l->vec == full) ? (l->steps == 2 || l->steps == 4 || l->steps == 8)
+                                           : (l->steps == 4 || l->steps == 8 || l->steps == 16);
+    if (!steps_ok) return SCANSCAM_EPLAN;
+
+    // LDS: 2 buffers x (A, B) x [waves][vec][64] floats, kept within 64 KiB.
+    const int max_by_lds = 64 / l->vec;
+    const int max_by_threads = scanscam::cl_max_threads(l->vec, l->steps) / kWave;
+    int max_waves = scanscam::kMaxWaves;
+    if (max_waves > max_by_lds) max_waves = max_by_lds;
+    if (max_waves > max_by_threads) max_waves = max_by_threads;
+    if (u.waves) {
+        l->waves = u.waves;
+    } else {
+        const int64_t segments = (T + l->steps - 1) / l->steps;  // no more waves than segments of time
+        l->waves = segments < max_waves ? pow2_ceil(segments) : max_waves;
+        if (l->waves > max_waves) l->waves = max_waves;
+    }
+    if (l->waves < 1 || l->waves > max_waves) return SCANSCAM_EPLAN;
+    l->grid = batch * groups(l->vec);
+    if (l->grid >= (int64_t(1) << 31)) return SCANSCAM_EINVAL;
+    l->lds_bytes = (size_t)4 * l->waves * l->vec * kWave * sizeof(float);
+    return SCANSCAM_OK;
+}
+
+int run_cl(bool rev, const void *a, const void *x, const void *h, void *y0, void *y1, int64_t batch, int64_t T,
+           int64_t C, int dtype, void *stream, const scanscam_plan *plan)
+{
+    const int esize = elem_size(dtype);
+    if (esize == 0) return SCANSCAM_EDTYPE;
+    if (batch < 0 || T < 0 || C < 0 || T >= kMaxT || C >= kMaxT) return SCANSCAM_EINVAL;
+    if (batch == 0 || T == 0 || C == 0) return SCANSCAM_OK;
+    if (!a || !x || !y0 || (rev && (!h || !y1))) return SCANSCAM_EINVAL;
+
+    const void *ptrs[5] = {a, x, y0, rev ? h : a, rev ? y1 : y0};
+    bool aligned16 = true;
+    for (const void *p : ptrs) {
+        if (!aligned_to(p, (size_t)esize)) return SCANSCAM_EALIGN;
+        aligned16 = aligned16 && aligned_to(p, 16);
+    }
+    scanscam::ClLaunch l;
+    const int rc = resolve_cl(plan, batch, T, C, dtype, aligned16, &l);
+    if (rc != SCANSCAM_OK) return rc;
+
+    scanscam::ClArgs args;
+    args.a = a;
+    args.x = x;
+    args.h = rev ? h : a;  // never read in the forward pass
+    args.y0 = y0;
+    args.y1 = rev ? y1 : y0;
+    args.batch = batch;
+    args.T = (int32_t)T;
+    args.C = (int32_t)C;
+
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipError_t e = hipErrorInvalidValue;
+    switch (dtype) {
+    case SCANSCAM_F32: e = scanscam::launch_scan_cl<float>(args, l, rev, s); break;
+    case SCANSCAM_BF16: e = scanscam::launch_scan_cl<__bf16>(args, l, rev, s); break;
+    case SCANSCAM_F16: e = scanscam::launch_scan_cl<_Float16>(args, l, rev, s); break;
+    }
+    return e == hipSuccess ? SCANSCAM_OK : SCANSCAM_ELAUNCH;
+}
+
 size_t workspace_for(int64_t rows, int64_t T, int dtype, const scanscam_plan *plan)
 {
     // The caller's pointers are not known yet: cover both the 16-byte aligned
@@ -275,6 +361,18 @@ size_t scanscam_workspace_bytes_plan(int64_t rows, int64_t T, int dtype, int dir
 {
     (void)direction;
     return workspace_for(rows, T, dtype, plan);
+}
+
+int scanscam_scan_fwd_cl(const void *a, const void *b, void *h, int64_t batch, int64_t T, int64_t C, int dtype,
+                         void *stream, const scanscam_plan *plan)
+{
+    return run_cl(false, a, b, nullptr, h, nullptr, batch, T, C, dtype, stream, plan);
+}
+
+int scanscam_scan_bwd_cl(const void *a, const void *h, const void *gh, void *ga, void *gb, int64_t batch,
+                         int64_t T, int64_t C, int dtype, void *stream, const scanscam_plan *plan)
+{
+    return run_cl(true, a, gh, h, gb, ga, batch, T, C, dtype, stream, plan);
 }
 
 int scanscam_resolve_plan(int64_t rows, int64_t T, int dtype, int direction, const scanscam_plan *plan,

@@ -3,4 +3,5 @@
 
 namespace scanscam {
 SCANSCAM_DEFINE_LAUNCH(_Float16)
+SCANSCAM_DEFINE_CL_LAUNCH(_Float16)
 }  // namespace scanscam

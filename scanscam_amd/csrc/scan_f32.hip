@@ -3,4 +3,5 @@
 
 namespace scanscam {
 SCANSCAM_DEFINE_LAUNCH(float)
+SCANSCAM_DEFINE_CL_LAUNCH(float)
 }  // namespace scanscam

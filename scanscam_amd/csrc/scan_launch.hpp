@@ -1,6 +1,7 @@
 // Host-side launch plumbing shared by the per-dtype translation units.
 #pragma once
 
+#include "scan_cl_kernels.hpp"
 #include "scan_kernels.hpp"
 
 namespace scanscam {
@@ -55,6 +56,43 @@ hipError_t launch_scan(const ScanArgs &args, const Launch &l, bool rev, hipStrea
         SCANSCAM_LAUNCH_CASE(ST, 1, 1)                                                               \
         SCANSCAM_LAUNCH_CASE(ST, 1, 4)                                                               \
         return hipErrorInvalidValue;                                                                 \
+    }
+
+// Channels-last launches. `steps` = time steps per wave per tile (S).
+struct ClLaunch {
+    int vec;
+    int steps;
+    int waves;
+    int64_t grid;
+    size_t lds_bytes;
+};
+
+constexpr int cl_max_threads(int vec, int steps) { return (vec > 1 && steps >= 8) ? 512 : 1024; }
+
+template <typename ST>
+hipError_t launch_scan_cl(const ClArgs &args, const ClLaunch &l, bool rev, hipStream_t stream);
+
+#define SCANSCAM_CL_CASE(ST, VEC, S)                                                                   \
+    if (l.vec == (VEC) && l.steps == (S)) {                                                            \
+        constexpr int MAXT = cl_max_threads(VEC, S);                                                   \
+        if (rev) hipLaunchKernelGGL((scan_cl_kernel<ST, VEC, S, true, MAXT>), grid, block, l.lds_bytes, stream, args);  \
+        else     hipLaunchKernelGGL((scan_cl_kernel<ST, VEC, S, false, MAXT>), grid, block, l.lds_bytes, stream, args); \
+        return hipGetLastError();                                                                      \
+    }
+
+#define SCANSCAM_DEFINE_CL_LAUNCH(ST)                                                                  \
+    template <>                                                                                        \
+    hipError_t launch_scan_cl<ST>(const ClArgs &args, const ClLaunch &l, bool rev, hipStream_t stream) \
+    {                                                                                                  \
+        constexpr int FULL = 16 / (int)sizeof(ST);                                                     \
+        const dim3 grid((unsigned)l.grid), block((unsigned)(l.waves * kWave));                         \
+        SCANSCAM_CL_CASE(ST, FULL, 2)                                                                  \
+        SCANSCAM_CL_CASE(ST, FULL, 4)                                                                  \
+        SCANSCAM_CL_CASE(ST, FULL, 8)                                                                  \
+        SCANSCAM_CL_CASE(ST, 1, 4)                                                                     \
+        SCANSCAM_CL_CASE(ST, 1, 8)                                                                     \
+        SCANSCAM_CL_CASE(ST, 1, 16)                                                                    \
+        return hipErrorInvalidValue;                                                                   \
     }
 
 }  // namespace scanscam

@@ -65,6 +65,10 @@ def _bind(path: str) -> ctypes.CDLL:
     lib.scanscam_scan_bwd_plan.restype = i32
     lib.scanscam_workspace_bytes_plan.argtypes = [i64, i64, i32, i32, plan_p]
     lib.scanscam_workspace_bytes_plan.restype = sz
+    lib.scanscam_scan_fwd_cl.argtypes = [p, p, p, i64, i64, i64, i32, p, plan_p]
+    lib.scanscam_scan_fwd_cl.restype = i32
+    lib.scanscam_scan_bwd_cl.argtypes = [p, p, p, p, p, i64, i64, i64, i32, p, plan_p]
+    lib.scanscam_scan_bwd_cl.restype = i32
     lib.scanscam_resolve_plan.argtypes = [i64, i64, i32, i32, plan_p, plan_p]
     lib.scanscam_resolve_plan.restype = i32
     lib.scanscam_strerror.argtypes = [i32]
@@ -291,3 +295,60 @@ def blocked_linear_scan_backward(
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """Drop-in for ``scanscam.cuda.blocked_linear_scan_backward`` (``cuda.py:56-66``)."""
     return linear_scan_backward(x, y, z)
+
+
+def _check_channels_last(*tensors: torch.Tensor) -> None:
+    first = tensors[0]
+    for t in tensors:
+        if t.shape != first.shape or t.dim() != 3:
+            raise AssertionError("scanscam_amd.hip: expected 3-D [batch, T, C] tensors of one shape")
+        if not t.is_contiguous():
+            raise AssertionError("scanscam_amd.hip: channels-last tensors must be contiguous as [batch, T, C]")
+        if t.device.type != "cuda" or t.device != first.device:
+            raise RuntimeError(f"scanscam_amd.hip: expected GPU tensors on one device, got {t.device}")
+        if t.dtype != first.dtype:
+            raise TypeError(f"scanscam_amd.hip: tensors differ in dtype ({first.dtype} and {t.dtype})")
+
+
+def transposed_linear_scan_forward(x: torch.Tensor, y: torch.Tensor, channels_per_block: int = 32,
+                                   plan: Optional[Plan] = None) -> torch.Tensor:
+    """Scan along T of contiguous ``[batch, T, C]`` tensors; returns ``[batch, T, C]``.
+
+    Drop-in for ``scanscam.cuda.transposed_linear_scan_forward`` (``cuda.py:69-80``).
+    ``channels_per_block`` tunes the reference's kernel and has no meaning here;
+    it is accepted and ignored (``plan`` is this library's tuning hook).
+    """
+    L = lib()
+    _check_channels_last(x, y)
+    out = torch.empty_like(x)
+    batch, T, C = x.shape
+    if x.numel() == 0:
+        return out
+    with torch.cuda.device(x.device):
+        rc = L.scanscam_scan_fwd_cl(x.data_ptr(), y.data_ptr(), out.data_ptr(), batch, T, C, _dtype_code(x.dtype),
+                                    torch.cuda.current_stream().cuda_stream,
+                                    ctypes.byref(plan) if plan is not None else None)
+    if rc != 0:
+        raise RuntimeError(f"scanscam_scan_fwd_cl: {strerror(rc)}")
+    return out
+
+
+def transposed_linear_scan_backward(x: torch.Tensor, y: torch.Tensor, z: torch.Tensor, channels_per_block: int = 32,
+                                    plan: Optional[Plan] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``(gate_grad, value_grad)`` for contiguous ``[batch, T, C]`` gate ``x``, output ``y``, output grad ``z``.
+
+    Drop-in for ``scanscam.cuda.transposed_linear_scan_backward`` (``cuda.py:81-95``).
+    """
+    L = lib()
+    _check_channels_last(x, y, z)
+    out_a, out_b = torch.empty_like(x), torch.empty_like(x)
+    batch, T, C = x.shape
+    if x.numel() == 0:
+        return out_a, out_b
+    with torch.cuda.device(x.device):
+        rc = L.scanscam_scan_bwd_cl(x.data_ptr(), y.data_ptr(), z.data_ptr(), out_a.data_ptr(), out_b.data_ptr(),
+                                    batch, T, C, _dtype_code(x.dtype), torch.cuda.current_stream().cuda_stream,
+                                    ctypes.byref(plan) if plan is not None else None)
+    if rc != 0:
+        raise RuntimeError(f"scanscam_scan_bwd_cl: {strerror(rc)}")
+    return out_a, out_b

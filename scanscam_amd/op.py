@@ -45,9 +45,13 @@ class Scan(torch.autograd.Function):
     def forward(ctx: Any, gate: torch.Tensor, value: torch.Tensor) -> torch.Tensor:
         if _on_gpu(gate):
             # Raises if the HIP library is missing: a GPU tensor is never
-            # quietly scanned any other way. Channels-last inputs are made
-            # row-contiguous by the wrapper for now.
-            output = hip.blocked_linear_scan_forward(gate, value)
+            # quietly scanned any other way.
+            if is_transpose_contig(gate) and is_transpose_contig(value):
+                # Stored [B, T, C]: scanned in place by the channels-last kernels
+                # (op.py:28-29 of the reference); the result keeps that layout.
+                output = hip.transposed_linear_scan_forward(gate.mT, value.mT).mT
+            else:
+                output = hip.blocked_linear_scan_forward(gate, value)
         else:
             output = naive_linear_scan_forward(gate, value)
         ctx.save_for_backward(gate, output)
@@ -57,5 +61,9 @@ class Scan(torch.autograd.Function):
     def backward(ctx: Any, output_grad: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
         gate, output = ctx.saved_tensors
         if _on_gpu(output_grad):
+            if is_transpose_contig(gate) and is_transpose_contig(output):
+                # What op.py:45-49 of the reference means to do (its call has one argument too many).
+                grads = hip.transposed_linear_scan_backward(gate.mT, output.mT, output_grad.mT.contiguous())
+                return tuple(g.mT for g in grads)
             return hip.blocked_linear_scan_backward(gate, output, output_grad)
         return naive_linear_scan_backward(gate, output, output_grad)

@@ -1,0 +1,129 @@
+"""
+Parity of the channels-last kernels ([batch, T, C] storage, scanned along T)
+with the CPU oracle, through the C ABI. Shapes and the N(0,1) gates follow the
+reference's tests of its transposed kernels (scanscam/cuda_test.py:129-163); the
+oracle sees the same values as contiguous [batch, C, T] arrays.
+"""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from scanscam_amd import hip
+
+pytestmark = pytest.mark.gpu
+
+REFERENCE_SHAPES = [(8, 4096, 512), (512, 4096, 8), (3, 107, 197), (3, 293, 283), (5, 6113, 107)]
+
+
+def row_norm_err(x, ref):
+    x = np.asarray(x, np.float64).reshape(-1, x.shape[-1])
+    ref = np.asarray(ref, np.float64).reshape(-1, ref.shape[-1])
+    scale = np.maximum(np.max(np.abs(ref), axis=1), 1.0)
+    return float(np.max(np.max(np.abs(x - ref), axis=1) / scale))
+
+
+def rel_err(x, ref, floor=None):
+    x, ref = np.asarray(x, np.float64), np.asarray(ref, np.float64)
+    den = np.maximum(np.abs(ref), 1.0)
+    if floor is not None:
+        den = np.maximum(den, floor)
+    return float(np.max(np.abs(x - ref) / den))
+
+
+def prev_abs(h):
+    h = np.abs(np.asarray(h, np.float64))
+    out = np.zeros_like(h)
+    out[..., 1:] = h[..., :-1]
+    return out
+
+
+def as_rows(t):
+    """[batch, T, C] torch tensor -> contiguous [batch, C, T] float32 numpy array."""
+    return t.detach().float().cpu().mT.contiguous().numpy()
+
+
+@pytest.mark.parametrize("shape", REFERENCE_SHAPES)
+@pytest.mark.parametrize("channels_per_block", [1, 32])
+def test_reference_shapes(gpu, shape, channels_per_block):
+    g = torch.Generator().manual_seed(sum(shape))
+    x = torch.randn(shape, generator=g)
+    y = torch.randn(shape, generator=g)
+    gh = torch.randn(shape, generator=g)
+    print(f"case channels_last shape={shape}", flush=True)
+    out = hip.transposed_linear_scan_forward(x.to(gpu), y.to(gpu), channels_per_block)
+    assert out.shape == x.shape and out.is_contiguous()
+    want = oracle.fwd(as_rows(x), as_rows(y))
+    assert row_norm_err(as_rows(out), want) <= 1e-4
+    hs = torch.from_numpy(want).mT.contiguous()  # the oracle's output, stored [batch, T, C]
+    ga, gb = hip.transposed_linear_scan_backward(x.to(gpu), hs.to(gpu), gh.to(gpu), channels_per_block)
+    wga, wgb = oracle.bwd(as_rows(x), want, as_rows(gh))
+    assert row_norm_err(as_rows(gb), wgb) <= 1e-4
+    assert row_norm_err(as_rows(ga), wga) <= 1e-4
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_forced_plans(gpu, dtype):
+    full = 4 if dtype == torch.float32 else 8
+    bar = 1e-5 if dtype == torch.float32 else 1e-2
+    g = torch.Generator().manual_seed(17)
+    cases = []
+    for shape in [(3, 301, 64 * full + full), (2, 77, 3 * full), (1, 1500, 256), (2, 5, 130), (4, 64, 33)]:
+        a = torch.rand(shape, generator=g).to(dtype)
+        b = torch.randn(shape, generator=g).to(dtype)
+        gh = torch.randn(shape, generator=g).to(dtype)
+        h = oracle.fwd(as_rows(a), as_rows(b))
+        hs = torch.from_numpy(h).mT.contiguous().to(dtype)
+        ga, gb = oracle.bwd(as_rows(a), as_rows(hs), as_rows(gh))
+        cases.append((shape, a.to(gpu), b.to(gpu), gh.to(gpu), hs.to(gpu), h, ga, gb, prev_abs(as_rows(hs))))
+    n = 0
+    for vec in (full, 1):
+        for steps in ((2, 4, 8) if vec == full else (4, 8, 16)):
+            max_waves = min(16, 64 // vec, (512 if (vec > 1 and steps >= 8) else 1024) // 64)
+            for waves in sorted({1, 3, max_waves}):
+                plan = hip.Plan(vec=vec, unroll=steps, waves=waves)
+                for shape, a, b, gh, hs, h, ga, gb, hp in cases:
+                    if vec != 1 and shape[-1] % full != 0:
+                        continue
+                    print(f"case cl forced {dtype} shape={shape} {plan}", flush=True)
+                    got_h = hip.transposed_linear_scan_forward(a, b, plan=plan)
+                    got_ga, got_gb = hip.transposed_linear_scan_backward(a, hs, gh, plan=plan)
+                    assert rel_err(as_rows(got_h), h) <= bar, (plan, shape)
+                    assert rel_err(as_rows(got_gb), gb) <= bar, (plan, shape)
+                    assert rel_err(as_rows(got_ga), ga, hp) <= bar, (plan, shape)
+                    n += 1
+    assert n > 40
+
+
+def test_matches_row_layout_kernels(gpu):
+    # Same data through both layouts: the two kernel families must agree closely
+    # (each is within 1e-5 of the oracle; they differ only in association order).
+    g = torch.Generator(device=gpu).manual_seed(9)
+    x = torch.rand((4, 2048, 1024), generator=g, device=gpu)
+    y = torch.randn((4, 2048, 1024), generator=g, device=gpu)
+    cl = hip.transposed_linear_scan_forward(x, y)
+    rows = hip.blocked_linear_scan_forward(x.mT.contiguous(), y.mT.contiguous())
+    assert float((cl.mT - rows).abs().max()) <= 2e-5
+    ga, gb = hip.transposed_linear_scan_backward(x, cl, y)
+    rga, rgb = hip.blocked_linear_scan_backward(x.mT.contiguous(), cl.mT.contiguous(), y.mT.contiguous())
+    assert float((gb.mT - rgb).abs().max()) <= 2e-5
+    assert float((ga.mT - rga).abs().max() / rga.abs().max().clamp(min=1)) <= 2e-5
+
+
+def test_empty_and_argument_checks(gpu):
+    for shape in [(0, 4, 8), (2, 0, 8), (2, 4, 0)]:
+        z = torch.zeros(shape, device=gpu)
+        assert hip.transposed_linear_scan_forward(z, z).shape == z.shape
+        ga, gb = hip.transposed_linear_scan_backward(z, z, z)
+        assert ga.shape == z.shape and gb.shape == z.shape
+    x = torch.zeros(2, 8, 16, device=gpu)
+    with pytest.raises(AssertionError):
+        hip.transposed_linear_scan_forward(x, x[:, :4])
+    with pytest.raises(AssertionError):
+        hip.transposed_linear_scan_forward(x.mT, x.mT)  # not contiguous as [batch, T, C]
+    with pytest.raises(AssertionError):
+        hip.transposed_linear_scan_forward(x[0], x[0])  # not 3-D
+    with pytest.raises(RuntimeError):
+        hip.transposed_linear_scan_forward(x, x, plan=hip.Plan(vec=4, unroll=3))
