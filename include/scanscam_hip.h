@@ -29,11 +29,13 @@
 extern "C" {
 #endif
 
-/* Storage types. Arithmetic is always fp32. */
+/* Storage types. Arithmetic is fp32 for the first three and fp64 for SCANSCAM_F64
+ * (the reference dispatches float and double, src/scanscam_cpu.hpp:43, src/scanscam_cuda.cu:288). */
 enum {
     SCANSCAM_F32 = 0,
-    SCANSCAM_BF16 = 1, /* no counterpart in the reference (float/double only, src/scanscam_cpu.hpp:43) */
-    SCANSCAM_F16 = 2
+    SCANSCAM_BF16 = 1, /* no counterpart in the reference */
+    SCANSCAM_F16 = 2,  /* no counterpart in the reference */
+    SCANSCAM_F64 = 3
 };
 
 enum { SCANSCAM_FORWARD = 0, SCANSCAM_BACKWARD = 1 };

@@ -11,8 +11,6 @@ namespace {
 using scanscam::kCounterStride;
 using scanscam::kMaxCounters;
 using scanscam::kSuper;
-using scanscam::kSuperWords;
-using scanscam::kTileWords;
 using scanscam::kModeLookback;
 using scanscam::kModeRow;
 using scanscam::kModeSmall;
@@ -36,9 +34,16 @@ int elem_size(int dtype)
     case SCANSCAM_F32: return 4;
     case SCANSCAM_BF16:
     case SCANSCAM_F16: return 2;
+    case SCANSCAM_F64: return 8;
     default: return 0;
     }
 }
+
+// 64-bit words per value published in the look-back workspace (one per 32-bit half).
+int value_words(int dtype) { return dtype == SCANSCAM_F64 ? 2 : 1; }
+
+// Bytes of the arithmetic type behind a storage type.
+int compute_size(int dtype) { return dtype == SCANSCAM_F64 ? 8 : 4; }
 
 bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
 
@@ -150,8 +155,9 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
         l.grid = (int64_t)out->counters * rows_per_counter * out->tiles_per_row;
         if (l.grid >= (int64_t(1) << 31)) return SCANSCAM_EINVAL;
         const int64_t supers = rows * (int64_t)((out->tiles_per_row + kSuper - 1) / kSuper);
-        out->super_base = (int64_t)out->counters * kCounterStride + tiles * kTileWords;
-        out->ws_bytes = (size_t)(out->super_base + supers * kSuperWords) * sizeof(uint64_t);
+        const int vw = value_words(dtype);
+        out->super_base = (int64_t)out->counters * kCounterStride + tiles * 2 * vw;
+        out->ws_bytes = (size_t)(out->super_base + supers * 4 * vw) * sizeof(uint64_t);
     } else {
         return SCANSCAM_EPLAN;
     }
@@ -219,6 +225,7 @@ int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y
     case SCANSCAM_F32: e = scanscam::launch_scan<float>(args, r.l, rev, s); break;
     case SCANSCAM_BF16: e = scanscam::launch_scan<__bf16>(args, r.l, rev, s); break;
     case SCANSCAM_F16: e = scanscam::launch_scan<_Float16>(args, r.l, rev, s); break;
+    case SCANSCAM_F64: e = scanscam::launch_scan<double>(args, r.l, rev, s); break;
     }
     return e == hipSuccess ? SCANSCAM_OK : SCANSCAM_ELAUNCH;
 }
@@ -250,8 +257,9 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
                                            : (l->steps == 4 || l->steps == 8 || l->steps == 16);
     if (!steps_ok) return SCANSCAM_EPLAN;
 
-    // LDS: 2 buffers x (A, B) x [waves][vec][64] floats, kept within 64 KiB.
-    const int max_by_lds = 64 / l->vec;
+    // LDS: 2 buffers x (A, B) x [waves][vec][64] values, kept within 64 KiB.
+    const int csize = compute_size(dtype);
+    const int max_by_lds = (64 * 1024) / (4 * l->vec * kWave * csize);
     const int max_by_threads = scanscam::cl_max_threads(l->vec, l->steps) / kWave;
     int max_waves = scanscam::kMaxWaves;
     if (max_waves > max_by_lds) max_waves = max_by_lds;
@@ -266,7 +274,7 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     if (l->waves < 1 || l->waves > max_waves) return SCANSCAM_EPLAN;
     l->grid = batch * groups(l->vec);
     if (l->grid >= (int64_t(1) << 31)) return SCANSCAM_EINVAL;
-    l->lds_bytes = (size_t)4 * l->waves * l->vec * kWave * sizeof(float);
+    l->lds_bytes = (size_t)4 * l->waves * l->vec * kWave * csize;
     return SCANSCAM_OK;
 }
 
@@ -305,6 +313,7 @@ int run_cl(bool rev, const void *a, const void *x, const void *h, void *y0, void
     case SCANSCAM_F32: e = scanscam::launch_scan_cl<float>(args, l, rev, s); break;
     case SCANSCAM_BF16: e = scanscam::launch_scan_cl<__bf16>(args, l, rev, s); break;
     case SCANSCAM_F16: e = scanscam::launch_scan_cl<_Float16>(args, l, rev, s); break;
+    case SCANSCAM_F64: e = scanscam::launch_scan_cl<double>(args, l, rev, s); break;
     }
     return e == hipSuccess ? SCANSCAM_OK : SCANSCAM_ELAUNCH;
 }

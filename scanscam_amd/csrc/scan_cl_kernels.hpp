@@ -34,13 +34,15 @@ struct ClArgs {
     int32_t C;
 };
 
-// Dynamic LDS: two buffers (tiles alternate) of A and B, each [W][VEC][64] floats.
+// Dynamic LDS: two buffers (tiles alternate) of A and B, each [W][VEC][64] values.
 template <typename ST, int VEC, int S, bool REV, int MAXT>
 __global__ __launch_bounds__(MAXT) void scan_cl_kernel(const ClArgs p)
 {
     using V = Vec<ST, VEC>;
     using raw_t = typename V::raw_t;
-    extern __shared__ float lds[];
+    using CT = typename ComputeOf<ST>::type;
+    extern __shared__ double lds_raw[];  // 8-byte aligned for either arithmetic type
+    CT *lds = reinterpret_cast<CT *>(lds_raw);
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
@@ -60,13 +62,13 @@ __global__ __launch_bounds__(MAXT) void scan_cl_kernel(const ClArgs p)
     const int tile_steps = W * S;
     const int ntiles = (T + tile_steps - 1) / tile_steps;
     const int plane = W * VEC * kWave;  // floats per LDS array
-    float carry[VEC];
+    CT carry[VEC];
 #pragma unroll
-    for (int k = 0; k < VEC; k++) carry[k] = 0.0f;
+    for (int k = 0; k < VEC; k++) carry[k] = CT(0);
 
     for (int it = 0; it < ntiles; it++) {
-        float *lds_A = lds + (it & 1) * 2 * plane;
-        float *lds_B = lds_A + plane;
+        CT *lds_A = lds + (it & 1) * 2 * plane;
+        CT *lds_B = lds_A + plane;
         const int tau0 = it * tile_steps + wave * S;  // position in scan order
 
         raw_t ra[S], rx[S], rh[REV ? S : 1];
@@ -93,28 +95,28 @@ __global__ __launch_bounds__(MAXT) void scan_cl_kernel(const ClArgs p)
             }
         }
 
-        float g[S][VEC], v[S][VEC];
-        float A[VEC], B[VEC];
+        CT g[S][VEC], v[S][VEC];
+        CT A[VEC], B[VEC];
 #pragma unroll
         for (int k = 0; k < VEC; k++) {
-            A[k] = 1.0f;
-            B[k] = 0.0f;
+            A[k] = CT(1);
+            B[k] = CT(0);
         }
 #pragma unroll
         for (int s = 0; s < S; s++) {
-            float fa[VEC], fx[VEC];
+            CT fa[VEC], fx[VEC];
             V::unpack(ra[s], fa);
             V::unpack(rx[s], fx);
 #pragma unroll
             for (int k = 0; k < VEC; k++) {
-                g[s][k] = ok[s] ? fa[k] : 1.0f;
+                g[s][k] = ok[s] ? fa[k] : CT(1);
                 v[s][k] = fx[k];  // zero where not ok
-                B[k] = __builtin_fmaf(g[s][k], B[k], v[s][k]);
+                B[k] = fma_(g[s][k], B[k], v[s][k]);
                 A[k] = A[k] * g[s][k];
             }
         }
 
-        float mine[VEC];
+        CT mine[VEC];
         if (W > 1) {
 #pragma unroll
             for (int k = 0; k < VEC; k++) {
@@ -122,7 +124,7 @@ __global__ __launch_bounds__(MAXT) void scan_cl_kernel(const ClArgs p)
                 lds_B[(wave * VEC + k) * kWave + lane] = B[k];
             }
             __syncthreads();
-            float c[VEC];
+            CT c[VEC];
 #pragma unroll
             for (int k = 0; k < VEC; k++) {
                 c[k] = carry[k];
@@ -132,7 +134,7 @@ __global__ __launch_bounds__(MAXT) void scan_cl_kernel(const ClArgs p)
 #pragma unroll
                 for (int k = 0; k < VEC; k++) {
                     if (q == wave) mine[k] = c[k];
-                    c[k] = __builtin_fmaf(lds_A[(q * VEC + k) * kWave + lane], c[k], lds_B[(q * VEC + k) * kWave + lane]);
+                    c[k] = fma_(lds_A[(q * VEC + k) * kWave + lane], c[k], lds_B[(q * VEC + k) * kWave + lane]);
                 }
             }
 #pragma unroll
@@ -141,7 +143,7 @@ __global__ __launch_bounds__(MAXT) void scan_cl_kernel(const ClArgs p)
 #pragma unroll
             for (int k = 0; k < VEC; k++) {
                 mine[k] = carry[k];
-                carry[k] = __builtin_fmaf(A[k], carry[k], B[k]);
+                carry[k] = fma_(A[k], carry[k], B[k]);
             }
         }
 
@@ -149,16 +151,16 @@ __global__ __launch_bounds__(MAXT) void scan_cl_kernel(const ClArgs p)
         for (int s = 0; s < S; s++) {
             const int tau = tau0 + s;
             const int t = REV ? T - 1 - tau : tau;
-            float out[VEC];
+            CT out[VEC];
 #pragma unroll
             for (int k = 0; k < VEC; k++) {
-                mine[k] = __builtin_fmaf(g[s][k], mine[k], v[s][k]);
+                mine[k] = fma_(g[s][k], mine[k], v[s][k]);
                 out[k] = mine[k];
             }
             if (!REV) {
                 if (ok[s]) V::store(y0 + (int64_t)t * C, V::pack(out));
             } else {
-                float fh[VEC], ga[VEC];
+                CT fh[VEC], ga[VEC];
                 V::unpack(rh[s], fh);
 #pragma unroll
                 for (int k = 0; k < VEC; k++) ga[k] = out[k] * fh[k];

@@ -76,9 +76,10 @@ struct ScanArgs {
 // Look-back workspace layout, in 64-bit words. Ticket counter c is word
 // c * kCounterStride (one counter per 128-byte line, so that counters do not
 // serialise on one another); word 1 is raised if a look-back wait ever expired
-// (results are then NaN). Then come kTileWords words per tile (its aggregate)
-// and kSuperWords words per super-tile of 64 tiles (its aggregate and its end
-// value). Each word is {1, bits(float)}: the upper half is a ready flag and the
+// (results are then NaN). Then come 2 published values per tile (its aggregate)
+// and 4 slots per super-tile of 64 tiles (its aggregate and its end value). A
+// value is one word {1, bits(float)} for fp32 arithmetic and two words, one per
+// 32-bit half, for fp64: the upper half of every word is a ready flag and the
 // workspace is zeroed before each launch, so every word is self-validating and
 // no fence is needed around it.
 #ifndef SCANSCAM_CTR_STRIDE
@@ -88,7 +89,7 @@ constexpr int kCounterStride = SCANSCAM_CTR_STRIDE;
 constexpr int kMaxCounters = 256;
 
 // ---------------------------------------------------------------------------
-// Storage types: float, __bf16, _Float16. All arithmetic is fp32.
+// Storage types: float, __bf16, _Float16 (arithmetic in fp32) and double (fp64).
 // ---------------------------------------------------------------------------
 template <int BYTES> struct RawT;
 template <> struct RawT<16> { typedef uint32_t type __attribute__((ext_vector_type(4))); };
@@ -97,6 +98,13 @@ template <> struct RawT<4> { typedef uint32_t type; };
 template <> struct RawT<2> { typedef uint16_t type; };
 
 template <typename ST, int VEC> struct Elems { ST e[VEC]; };
+
+// Arithmetic type of a storage type: fp32 for float and the 16-bit types, fp64 for double.
+template <typename ST> struct ComputeOf { using type = float; };
+template <> struct ComputeOf<double> { using type = double; };
+
+__device__ __forceinline__ float fma_(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+__device__ __forceinline__ double fma_(double a, double b, double c) { return __builtin_fma(a, b, c); }
 
 template <typename ST, int VEC> struct Vec {
     using raw_t = typename RawT<sizeof(ST) * VEC>::type;
@@ -126,13 +134,13 @@ template <typename ST, int VEC> struct Vec {
         *q = r;
 #endif
     }
-    static __device__ __forceinline__ void unpack(raw_t r, float (&f)[VEC])
+    template <typename CT> static __device__ __forceinline__ void unpack(raw_t r, CT (&f)[VEC])
     {
         Elems<ST, VEC> e = __builtin_bit_cast(Elems<ST, VEC>, r);
 #pragma unroll
-        for (int k = 0; k < VEC; k++) f[k] = (float)e.e[k];
+        for (int k = 0; k < VEC; k++) f[k] = (CT)e.e[k];
     }
-    static __device__ __forceinline__ raw_t pack(const float (&f)[VEC])
+    template <typename CT> static __device__ __forceinline__ raw_t pack(const CT (&f)[VEC])
     {
         Elems<ST, VEC> e;
 #pragma unroll
@@ -152,32 +160,52 @@ __device__ __forceinline__ float dpp_move(float old, float src)
                                            CTRL, ROW_MASK, 0xf, false));
 }
 
+struct Halves { int lo, hi; };
+
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ double dpp_move(double old, double src)
+{
+    const Halves o = __builtin_bit_cast(Halves, old), s = __builtin_bit_cast(Halves, src);
+    Halves r;
+    r.lo = __builtin_amdgcn_update_dpp(o.lo, s.lo, CTRL, ROW_MASK, 0xf, false);
+    r.hi = __builtin_amdgcn_update_dpp(o.hi, s.hi, CTRL, ROW_MASK, 0xf, false);
+    return __builtin_bit_cast(double, r);
+}
+
 // Value of the previous / next lane of the wave; `fill` where there is none.
-__device__ __forceinline__ float lane_prev(float src, float fill) { return dpp_move<0x138, 0xf>(fill, src); }
-__device__ __forceinline__ float lane_next(float src, float fill) { return dpp_move<0x130, 0xf>(fill, src); }
+template <typename CT> __device__ __forceinline__ CT lane_prev(CT src, CT fill) { return dpp_move<0x138, 0xf>(fill, src); }
+template <typename CT> __device__ __forceinline__ CT lane_next(CT src, CT fill) { return dpp_move<0x130, 0xf>(fill, src); }
 
 __device__ __forceinline__ float read_lane(float v, int lane)
 {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+__device__ __forceinline__ double read_lane(double v, int lane)
+{
+    const Halves s = __builtin_bit_cast(Halves, v);
+    Halves r;
+    r.lo = __builtin_amdgcn_readlane(s.lo, lane);
+    r.hi = __builtin_amdgcn_readlane(s.hi, lane);
+    return __builtin_bit_cast(double, r);
 }
 
 // Inclusive scan of affine pairs over the lanes of a wave (ascending lane =
 // later in scan order). With GROUPED the wave is cut into independent groups of
 // `group` lanes (j = lane index inside its group). Lanes that have no source
 // in a step receive the identity map (1, 0). All 64 lanes must be active.
-template <bool GROUPED>
-__device__ __forceinline__ void wave_scan(float &A, float &B, int j)
+template <bool GROUPED, typename CT>
+__device__ __forceinline__ void wave_scan(CT &A, CT &B, int j)
 {
 #define SCANSCAM_STEP(CTRL, ROW_MASK, OFF)                      \
     {                                                           \
-        float A1 = dpp_move<CTRL, ROW_MASK>(1.0f, A);           \
-        float B1 = dpp_move<CTRL, ROW_MASK>(0.0f, B);           \
+        CT A1 = dpp_move<CTRL, ROW_MASK>(CT(1), A);            \
+        CT B1 = dpp_move<CTRL, ROW_MASK>(CT(0), B);            \
         if (GROUPED) {                                          \
             const bool use = j >= (OFF);                        \
-            A1 = use ? A1 : 1.0f;                               \
-            B1 = use ? B1 : 0.0f;                               \
+            A1 = use ? A1 : CT(1);                              \
+            B1 = use ? B1 : CT(0);                              \
         }                                                       \
-        B = __builtin_fmaf(A, B1, B);                           \
+        B = fma_(A, B1, B);                                     \
         A = A * A1;                                             \
     }
     SCANSCAM_STEP(0x111, 0xf, 1)   // row_shr:1
@@ -202,6 +230,7 @@ template <typename ST, int VEC, int U, bool REV, bool GROUPED, bool CHAIN>
 struct WaveTile {
     using V = Vec<ST, VEC>;
     using raw_t = typename V::raw_t;
+    using CT = typename ComputeOf<ST>::type;
 
     // Where this lane's vector of chunk u lives.
     int64_t off[U];  // element offset of the vector from the tensor base
@@ -209,11 +238,11 @@ struct WaveTile {
     bool valid[U];   // inside the row (and the row exists)
 
     raw_t ra[U], rx[U], rh[REV ? U : 1];
-    float edge_a[REV ? U : 1];  // a[(m+1)*VEC] for the first lane of a group
-    float edge_h[REV ? U : 1];  // h[m*VEC - 1] for the last lane of a group
+    CT edge_a[REV ? U : 1];  // a[(m+1)*VEC] for the first lane of a group
+    CT edge_h[REV ? U : 1];  // h[m*VEC - 1] for the last lane of a group
 
-    float g[U][VEC], v[U][VEC];
-    float PA[U], PB[U];
+    CT g[U][VEC], v[U][VEC];
+    CT PA[U], PB[U];
 
     __device__ __forceinline__ void load(const ScanArgs &p, int j, int jlast)
     {
@@ -231,29 +260,29 @@ struct WaveTile {
             if (REV) {
                 rh[u] = V::zero_raw();
                 if (valid[u]) rh[u] = V::load(h + off[u]);
-                edge_a[u] = 0.0f;
-                edge_h[u] = 0.0f;
+                edge_a[u] = CT(0);
+                edge_h[u] = CT(0);
                 // Neighbours that no lane of this group holds. With CHAIN the chunks of a
                 // wave are adjacent, so only the wave's outer borders need memory: the
                 // inner ones are taken from the neighbouring chunk's registers in reduce().
                 const bool need_a = !CHAIN || u == 0;
                 const bool need_h = !CHAIN || u == U - 1;
-                if (need_a && valid[u] && j == 0 && (m[u] + 1) * VEC < p.T) edge_a[u] = (float)a[off[u] + VEC];
-                if (need_h && valid[u] && j == jlast && m[u] > 0) edge_h[u] = (float)h[off[u] - 1];
+                if (need_a && valid[u] && j == 0 && (m[u] + 1) * VEC < p.T) edge_a[u] = (CT)a[off[u] + VEC];
+                if (need_h && valid[u] && j == jlast && m[u] > 0) edge_h[u] = (CT)h[off[u] - 1];
             }
         }
     }
 
     // Builds (gate, value) per element in scan order and reduces them.
-    __device__ __forceinline__ void reduce(int j, int jlast, float (&hp)[REV ? U : 1][VEC])
+    __device__ __forceinline__ void reduce(int j, int jlast, CT (&hp)[REV ? U : 1][VEC])
     {
         // Backward: a[first element] and h[last element] of every chunk's vectors,
         // for the lanes at the borders between the chunks of this wave.
-        float first_a[REV ? U : 1], last_h[REV ? U : 1];
+        CT first_a[REV ? U : 1], last_h[REV ? U : 1];
         if (REV && CHAIN) {
 #pragma unroll
             for (int u = 0; u < U; u++) {
-                float t[VEC];
+                CT t[VEC];
                 V::unpack(ra[u], t);
                 first_a[u] = t[0];
                 V::unpack(rh[u], t);
@@ -262,89 +291,89 @@ struct WaveTile {
         }
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            float fa[VEC], fx[VEC];
+            CT fa[VEC], fx[VEC];
             V::unpack(ra[u], fa);
             V::unpack(rx[u], fx);
             if (!REV) {
 #pragma unroll
                 for (int k = 0; k < VEC; k++) {
-                    g[u][k] = valid[u] ? fa[k] : 1.0f;
+                    g[u][k] = valid[u] ? fa[k] : CT(1);
                     v[u][k] = fx[k];  // zero-filled where invalid
                 }
             } else {
-                float fh[VEC];
+                CT fh[VEC];
                 V::unpack(rh[u], fh);
                 // Scan order k <-> time t0 + VEC-1-k. gate = a[t+1], value = gh[t],
                 // hp = h[t-1]. Invalid lanes hold a = 0, so a neighbour past the
                 // end of the row reads as gate 0, which is what t = T-1 needs.
-                float a_next = lane_prev(fa[0], 0.0f);        // lane-1 holds vector m+1
-                float h_prev = lane_next(fh[VEC - 1], 0.0f);  // lane+1 holds vector m-1
-                float border_a = edge_a[u], border_h = edge_h[u];
+                CT a_next = lane_prev(fa[0], CT(0));        // lane-1 holds vector m+1
+                CT h_prev = lane_next(fh[VEC - 1], CT(0));  // lane+1 holds vector m-1
+                CT border_a = edge_a[u], border_h = edge_h[u];
                 if (CHAIN && u > 0) border_a = read_lane(first_a[u - 1], kWave - 1);
                 if (CHAIN && u + 1 < U) border_h = read_lane(last_h[u + 1], 0);
                 a_next = (j == 0) ? border_a : a_next;
                 h_prev = (j == jlast) ? border_h : h_prev;
 #pragma unroll
                 for (int k = 0; k < VEC; k++) {
-                    const float gk = (k == 0) ? a_next : fa[(VEC - k) % VEC];
-                    g[u][k] = valid[u] ? gk : 1.0f;
+                    const CT gk = (k == 0) ? a_next : fa[(VEC - k) % VEC];
+                    g[u][k] = valid[u] ? gk : CT(1);
                     v[u][k] = fx[VEC - 1 - k];
                     hp[u][k] = (k == VEC - 1) ? h_prev : fh[(VEC - 2 - k) < 0 ? 0 : (VEC - 2 - k)];
                 }
             }
-            float A = g[u][0], B = v[u][0];
+            CT A = g[u][0], B = v[u][0];
 #pragma unroll
             for (int k = 1; k < VEC; k++) {
-                B = __builtin_fmaf(g[u][k], B, v[u][k]);
+                B = fma_(g[u][k], B, v[u][k]);
                 A = A * g[u][k];
             }
-            wave_scan<GROUPED>(A, B, j);
+            wave_scan<GROUPED, CT>(A, B, j);
             PA[u] = A;
             PB[u] = B;
         }
     }
 
     // Aggregate of the wave's U chunks (CHAIN only): composition in scan order.
-    __device__ __forceinline__ void total(float &WA, float &WB) const
+    __device__ __forceinline__ void total(CT &WA, CT &WB) const
     {
         WA = read_lane(PA[0], 63);
         WB = read_lane(PB[0], 63);
 #pragma unroll
         for (int u = 1; u < U; u++) {
-            const float TA = read_lane(PA[u], 63), TB = read_lane(PB[u], 63);
-            WB = __builtin_fmaf(TA, WB, TB);
+            const CT TA = read_lane(PA[u], 63), TB = read_lane(PB[u], 63);
+            WB = fma_(TA, WB, TB);
             WA = TA * WA;
         }
     }
 
-    __device__ __forceinline__ void apply(const ScanArgs &p, float carry, int j,
-                                          const float (&hp)[REV ? U : 1][VEC])
+    __device__ __forceinline__ void apply(const ScanArgs &p, CT carry, int j,
+                                          const CT (&hp)[REV ? U : 1][VEC])
     {
         ST *y0 = static_cast<ST *>(p.y0);
         ST *y1 = static_cast<ST *>(p.y1);
 #pragma unroll
         for (int u = 0; u < U; u++) {
             // Map of everything before this lane inside the chunk.
-            float EA = lane_prev(PA[u], 1.0f);
-            float EB = lane_prev(PB[u], 0.0f);
+            CT EA = lane_prev(PA[u], CT(1));
+            CT EB = lane_prev(PB[u], CT(0));
             if (GROUPED) {
-                EA = (j == 0) ? 1.0f : EA;
-                EB = (j == 0) ? 0.0f : EB;
+                EA = (j == 0) ? CT(1) : EA;
+                EB = (j == 0) ? CT(0) : EB;
             }
-            const float c = CHAIN ? carry : 0.0f;
-            float acc = __builtin_fmaf(EA, c, EB);
-            float out[VEC];
+            const CT c = CHAIN ? carry : CT(0);
+            CT acc = fma_(EA, c, EB);
+            CT out[VEC];
 #pragma unroll
             for (int k = 0; k < VEC; k++) {
-                acc = __builtin_fmaf(g[u][k], acc, v[u][k]);
+                acc = fma_(g[u][k], acc, v[u][k]);
                 out[k] = acc;
             }
             if (CHAIN && u + 1 < U)
-                carry = __builtin_fmaf(read_lane(PA[u], 63), carry, read_lane(PB[u], 63));
+                carry = fma_(read_lane(PA[u], 63), carry, read_lane(PB[u], 63));
             if (!REV) {
                 if (valid[u]) V::store(y0 + off[u], V::pack(out));
             } else {
-                float gb[VEC], ga[VEC];
+                CT gb[VEC], ga[VEC];
 #pragma unroll
                 for (int k = 0; k < VEC; k++) {
                     gb[VEC - 1 - k] = out[k];
@@ -367,8 +396,9 @@ struct WaveTile {
 template <typename ST, int VEC, int U, bool REV, int MAXT>
 __global__ __launch_bounds__(MAXT) void scan_row_kernel(const ScanArgs p)
 {
-    __shared__ float lds_A[2][kMaxWaves];
-    __shared__ float lds_B[2][kMaxWaves];
+    using CT = typename ComputeOf<ST>::type;
+    __shared__ CT lds_A[2][kMaxWaves];
+    __shared__ CT lds_B[2][kMaxWaves];
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
@@ -392,8 +422,8 @@ __global__ __launch_bounds__(MAXT) void scan_row_kernel(const ScanArgs p)
     const int ntiles = (p.nch + tile_chunks - 1) / tile_chunks;
 
     WaveTile<ST, VEC, U, REV, false, true> w;
-    float hp[REV ? U : 1][VEC];
-    float row_carry = 0.0f;
+    CT hp[REV ? U : 1][VEC];
+    CT row_carry = CT(0);
 
     for (int it = 0; it < ntiles; it++) {
         const int chunk0 = (it * wpr + wr) * U;
@@ -408,25 +438,25 @@ __global__ __launch_bounds__(MAXT) void scan_row_kernel(const ScanArgs p)
         w.load(p, lane, kWave - 1);
         w.reduce(lane, kWave - 1, hp);
 
-        float carry = row_carry;
+        CT carry = row_carry;
         if (wpr > 1) {
-            float WA, WB;
+            CT WA, WB;
             w.total(WA, WB);
             if (lane == 0) {
                 lds_A[it & 1][wave] = WA;
                 lds_B[it & 1][wave] = WB;
             }
             __syncthreads();
-            float c = row_carry;
+            CT c = row_carry;
             for (int q = 0; q < wpr; q++) {
                 if (q == wr) carry = c;
-                c = __builtin_fmaf(lds_A[it & 1][wbase + q], c, lds_B[it & 1][wbase + q]);
+                c = fma_(lds_A[it & 1][wbase + q], c, lds_B[it & 1][wbase + q]);
             }
             row_carry = c;
         } else if (ntiles > 1) {
-            float WA, WB;
+            CT WA, WB;
             w.total(WA, WB);
-            row_carry = __builtin_fmaf(WA, row_carry, WB);
+            row_carry = fma_(WA, row_carry, WB);
         }
         w.apply(p, carry, lane, hp);
     }
@@ -439,6 +469,7 @@ __global__ __launch_bounds__(MAXT) void scan_row_kernel(const ScanArgs p)
 template <typename ST, int VEC, int U, bool REV, int MAXT>
 __global__ __launch_bounds__(MAXT) void scan_small_kernel(const ScanArgs p)
 {
+    using CT = typename ComputeOf<ST>::type;
     const int lane = threadIdx.x & (kWave - 1);
     const int G = p.group;
     const int j = lane & (G - 1);
@@ -447,7 +478,7 @@ __global__ __launch_bounds__(MAXT) void scan_small_kernel(const ScanArgs p)
     const int64_t row0 = wave_id * (U * rows_per_chunk) + lane / G;
 
     WaveTile<ST, VEC, U, REV, true, false> w;
-    float hp[REV ? U : 1][VEC];
+    CT hp[REV ? U : 1][VEC];
 #pragma unroll
     for (int u = 0; u < U; u++) {
         const int64_t row = row0 + (int64_t)u * rows_per_chunk;
@@ -458,7 +489,7 @@ __global__ __launch_bounds__(MAXT) void scan_small_kernel(const ScanArgs p)
     }
     w.load(p, j, G - 1);
     w.reduce(j, G - 1, hp);
-    w.apply(p, 0.0f, j, hp);
+    w.apply(p, CT(0), j, hp);
 }
 
 // ---------------------------------------------------------------------------
@@ -489,21 +520,43 @@ __global__ __launch_bounds__(MAXT) void scan_small_kernel(const ScanArgs p)
 // defining expression (S_{m+1} = fma(SA_m, S_m, SB_m), fixed ladder inside a
 // super-tile), so results do not depend on timing.
 // ---------------------------------------------------------------------------
-constexpr int kSuper = 64;       // tiles per super-tile (one per lane)
-constexpr int kTileWords = 2;    // {1, bits(A)}, {1, bits(B)}
-constexpr int kSuperWords = 4;   // {1, bits(SA)}, {1, bits(SB)}, {1, bits(SI)}, unused
+constexpr int kSuper = 64;  // tiles per super-tile (one per lane)
 
-__device__ __forceinline__ uint64_t desc_load(const uint64_t *p)
-{
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void desc_store(uint64_t *p, float v)
-{
-    const uint64_t w = (1ull << 32) | (uint64_t)__builtin_bit_cast(uint32_t, v);
-    __hip_atomic_store(p, w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ bool desc_ready(uint64_t w) { return (w >> 32) != 0; }
-__device__ __forceinline__ float desc_value(uint64_t w) { return __builtin_bit_cast(float, (uint32_t)w); }
+// A published value: each 32-bit half of it sits in the low half of its own
+// 64-bit word, whose high half is the ready flag (1). One word for fp32
+// arithmetic, two for fp64. A tile owns 2 values (A, B), a super-tile 4 slots
+// (SA, SB, SI, unused).
+template <typename CT> struct Desc;
+template <> struct Desc<float> {
+    static constexpr int W = 1;
+    static __device__ __forceinline__ void store(uint64_t *p, float v)
+    {
+        const uint64_t w = (1ull << 32) | (uint64_t)__builtin_bit_cast(uint32_t, v);
+        __hip_atomic_store(p, w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    static __device__ __forceinline__ bool load(const uint64_t *p, float &v)
+    {
+        const uint64_t w = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        v = __builtin_bit_cast(float, (uint32_t)w);
+        return (w >> 32) != 0;
+    }
+};
+template <> struct Desc<double> {
+    static constexpr int W = 2;
+    static __device__ __forceinline__ void store(uint64_t *p, double v)
+    {
+        const uint64_t b = __builtin_bit_cast(uint64_t, v);
+        __hip_atomic_store(p + 0, (1ull << 32) | (b & 0xffffffffull), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(p + 1, (1ull << 32) | (b >> 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    static __device__ __forceinline__ bool load(const uint64_t *p, double &v)
+    {
+        const uint64_t lo = __hip_atomic_load(p + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint64_t hi = __hip_atomic_load(p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        v = __builtin_bit_cast(double, (hi << 32) | (lo & 0xffffffffull));
+        return (lo >> 32) != 0 && (hi >> 32) != 0;
+    }
+};
 
 // Polls of the look-back loop before a wave gives up. Tickets make every
 // awaited tile belong to a workgroup that is already running, so the limit is
@@ -515,56 +568,60 @@ constexpr int kTimeoutWord = 1;
 
 // Returns the scan value entering tile `tile` of row `row`, whose own aggregate
 // is (TA, TB). Called by all 64 lanes of one wave; `tile` must be wave-uniform.
-__device__ __forceinline__ float lookback_carry(const ScanArgs &p, int64_t row, int tile, float TA, float TB,
-                                                int lane)
+template <typename CT>
+__device__ __forceinline__ CT lookback_carry(const ScanArgs &p, int64_t row, int tile, CT TA, CT TB, int lane)
 {
+    using D = Desc<CT>;
+    constexpr int TW = 2 * D::W, SW = 4 * D::W;  // words per tile / per super-tile
     const int tpr = p.tiles_per_row;
     const int spr = (tpr + kSuper - 1) / kSuper;
     const int j = tile % kSuper, m = tile / kSuper;
-    uint64_t *trow = p.ws + p.desc_base + row * (int64_t)tpr * kTileWords;
-    uint64_t *srow = p.ws + p.super_base + row * (int64_t)spr * kSuperWords;
+    uint64_t *trow = p.ws + p.desc_base + row * (int64_t)tpr * TW;
+    uint64_t *srow = p.ws + p.super_base + row * (int64_t)spr * SW;
     const bool closes = (j == kSuper - 1) && (m + 1 < spr);  // a later super-tile needs (SA, SB, SI)
 
     if (lane == 0 && j < kSuper - 1 && tile + 1 < tpr) {
-        desc_store(trow + (int64_t)tile * kTileWords + 0, TA);
-        desc_store(trow + (int64_t)tile * kTileWords + 1, TB);
+        D::store(trow + (int64_t)tile * TW, TA);
+        D::store(trow + (int64_t)tile * TW + D::W, TB);
     }
 
     // Lane q < j collects tile q of this super-tile; lane j holds this tile; the rest the identity.
     bool have_t = lane >= j;
-    float A = (lane == j) ? TA : 1.0f, B = (lane == j) ? TB : 0.0f;
+    CT A = (lane == j) ? TA : CT(1), B = (lane == j) ? TB : CT(0);
     // Lane k watches super-tile m-1-k; before the row starts the value is 0.
     const int sidx = m - 1 - lane;
     bool have_si = sidx < 0, have_sa = sidx < 0;
-    float SI = 0.0f, SA = 1.0f, SB = 0.0f;
+    CT SI = CT(0), SA = CT(1), SB = CT(0);
 
     bool tiles_done = false, super_done = false;
-    float PA = 1.0f, PB = 0.0f, S = 0.0f;
+    CT PA = CT(1), PB = CT(0), S = CT(0);
     for (int spin = 0; spin < kSpinLimit; spin++) {
         if (!have_t) {
-            const uint64_t *d = trow + (int64_t)(m * kSuper + lane) * kTileWords;
-            const uint64_t wa = desc_load(d + 0), wb = desc_load(d + 1);
-            if (desc_ready(wa) && desc_ready(wb)) {
+            const uint64_t *d = trow + (int64_t)(m * kSuper + lane) * TW;
+            CT va, vb;
+            const bool ra = D::load(d, va), rb = D::load(d + D::W, vb);
+            if (ra && rb) {
                 have_t = true;
-                A = desc_value(wa);
-                B = desc_value(wb);
+                A = va;
+                B = vb;
             }
         }
         if (!have_si || !have_sa) {
-            const uint64_t *d = srow + (int64_t)sidx * kSuperWords;
+            const uint64_t *d = srow + (int64_t)sidx * SW;
             if (!have_si) {
-                const uint64_t wi = desc_load(d + 2);
-                if (desc_ready(wi)) {
+                CT vi;
+                if (D::load(d + 2 * D::W, vi)) {
                     have_si = true;
-                    SI = desc_value(wi);
+                    SI = vi;
                 }
             }
             if (!have_sa) {
-                const uint64_t wa = desc_load(d + 0), wb = desc_load(d + 1);
-                if (desc_ready(wa) && desc_ready(wb)) {
+                CT va, vb;
+                const bool ra = D::load(d, va), rb = D::load(d + D::W, vb);
+                if (ra && rb) {
                     have_sa = true;
-                    SA = desc_value(wa);
-                    SB = desc_value(wb);
+                    SA = va;
+                    SB = vb;
                 }
             }
         }
@@ -572,12 +629,12 @@ __device__ __forceinline__ float lookback_carry(const ScanArgs &p, int64_t row, 
             tiles_done = true;
             PA = A;
             PB = B;
-            wave_scan<false>(PA, PB, lane);
+            wave_scan<false, CT>(PA, PB, lane);
             if (closes) {
-                const float sa = read_lane(PA, kSuper - 1), sb = read_lane(PB, kSuper - 1);
+                const CT sa = read_lane(PA, kSuper - 1), sb = read_lane(PB, kSuper - 1);
                 if (lane == 0) {
-                    desc_store(srow + (int64_t)m * kSuperWords + 0, sa);
-                    desc_store(srow + (int64_t)m * kSuperWords + 1, sb);
+                    D::store(srow + (int64_t)m * SW, sa);
+                    D::store(srow + (int64_t)m * SW + D::W, sb);
                 }
             }
         }
@@ -589,7 +646,7 @@ __device__ __forceinline__ float lookback_carry(const ScanArgs &p, int64_t row, 
                 const uint64_t need = (first == 0) ? 0ull : ((~0ull) >> (64 - first));
                 if ((ma & need) == need) {
                     S = read_lane(SI, first);
-                    for (int q = first - 1; q >= 0; q--) S = __builtin_fmaf(read_lane(SA, q), S, read_lane(SB, q));
+                    for (int q = first - 1; q >= 0; q--) S = fma_(read_lane(SA, q), S, read_lane(SB, q));
                     super_done = true;
                 }
             }
@@ -599,20 +656,20 @@ __device__ __forceinline__ float lookback_carry(const ScanArgs &p, int64_t row, 
     }
     if (!(tiles_done && super_done)) {
         if (lane == 0) __hip_atomic_store(p.ws + kTimeoutWord, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        S = __builtin_nanf("");
+        S = CT(__builtin_nanf(""));
     }
-    if (closes && lane == 0)
-        desc_store(srow + (int64_t)m * kSuperWords + 2,
-                   __builtin_fmaf(read_lane(PA, kSuper - 1), S, read_lane(PB, kSuper - 1)));
-    return j > 0 ? __builtin_fmaf(read_lane(PA, j - 1), S, read_lane(PB, j - 1)) : S;
+    const CT end_a = read_lane(PA, kSuper - 1), end_b = read_lane(PB, kSuper - 1);
+    if (closes && lane == 0) D::store(srow + (int64_t)m * SW + 2 * D::W, fma_(end_a, S, end_b));
+    return j > 0 ? fma_(read_lane(PA, j - 1), S, read_lane(PB, j - 1)) : S;
 }
 
 template <typename ST, int VEC, int U, bool REV, int MAXT>
 __global__ __launch_bounds__(MAXT) void scan_lookback_kernel(const ScanArgs p)
 {
-    __shared__ float lds_A[kMaxWaves];
-    __shared__ float lds_B[kMaxWaves];
-    __shared__ float lds_carry;
+    using CT = typename ComputeOf<ST>::type;
+    __shared__ CT lds_A[kMaxWaves];
+    __shared__ CT lds_B[kMaxWaves];
+    __shared__ CT lds_carry;
     __shared__ unsigned lds_ticket;
 
     const int lane = threadIdx.x & (kWave - 1);
@@ -641,7 +698,7 @@ __global__ __launch_bounds__(MAXT) void scan_lookback_kernel(const ScanArgs p)
     const int chunk0 = (tile * nwaves + wave) * U;
 
     WaveTile<ST, VEC, U, REV, false, true> w;
-    float hp[REV ? U : 1][VEC];
+    CT hp[REV ? U : 1][VEC];
 #pragma unroll
     for (int u = 0; u < U; u++) {
         const int s = (chunk0 + u) * kWave + lane;
@@ -653,7 +710,7 @@ __global__ __launch_bounds__(MAXT) void scan_lookback_kernel(const ScanArgs p)
     w.load(p, lane, kWave - 1);
     w.reduce(lane, kWave - 1, hp);
 
-    float WA, WB;
+    CT WA, WB;
     w.total(WA, WB);
     if (lane == 0) {
         lds_A[wave] = WA;
@@ -663,19 +720,19 @@ __global__ __launch_bounds__(MAXT) void scan_lookback_kernel(const ScanArgs p)
 
     if (wave == 0) {
         // Aggregate of the whole tile, waves in scan order.
-        float TA = lds_A[0], TB = lds_B[0];
+        CT TA = lds_A[0], TB = lds_B[0];
         for (int q = 1; q < nwaves; q++) {
-            TB = __builtin_fmaf(lds_A[q], TB, lds_B[q]);
+            TB = fma_(lds_A[q], TB, lds_B[q]);
             TA = lds_A[q] * TA;
         }
-        float cin = 0.0f;
-        if (p.tiles_per_row > 1) cin = lookback_carry(p, row, tile, TA, TB, lane);
+        CT cin = CT(0);
+        if (p.tiles_per_row > 1) cin = lookback_carry<CT>(p, row, tile, TA, TB, lane);
         if (lane == 0) lds_carry = cin;
     }
     __syncthreads();
 
-    float carry = lds_carry;
-    for (int q = 0; q < wave; q++) carry = __builtin_fmaf(lds_A[q], carry, lds_B[q]);
+    CT carry = lds_carry;
+    for (int q = 0; q < wave; q++) carry = fma_(lds_A[q], carry, lds_B[q]);
     w.apply(p, carry, lane, hp);
 }
 

@@ -28,7 +28,7 @@ MODE_AUTO, MODE_SMALL, MODE_ROW, MODE_LOOKBACK = 0, 1, 2, 3
 FORWARD, BACKWARD = 0, 1
 ABI_VERSION = 1
 
-_DTYPES = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
+_DTYPES = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2, torch.float64: 3}
 
 
 class Plan(ctypes.Structure):
@@ -132,7 +132,7 @@ def _dtype_code(dtype: torch.dtype) -> int:
     try:
         return _DTYPES[dtype]
     except KeyError:
-        raise TypeError(f"scanscam_amd: unsupported dtype {dtype}; supported: float32, bfloat16, float16") from None
+        raise TypeError(f"scanscam_amd: unsupported dtype {dtype}; supported: float32, float64, bfloat16, float16") from None
 
 
 def _check_rows(*tensors: torch.Tensor) -> None:

@@ -41,8 +41,10 @@ def prev_abs(h):
 
 
 def as_rows(t):
-    """[batch, T, C] torch tensor -> contiguous [batch, C, T] float32 numpy array."""
-    return t.detach().float().cpu().mT.contiguous().numpy()
+    """[batch, T, C] torch tensor -> contiguous [batch, C, T] numpy array (float64 stays, else float32)."""
+    t = t.detach().cpu()
+    t = t if t.dtype == torch.float64 else t.float()
+    return t.mT.contiguous().numpy()
 
 
 @pytest.mark.parametrize("shape", REFERENCE_SHAPES)
@@ -64,16 +66,16 @@ def test_reference_shapes(gpu, shape, channels_per_block):
     assert row_norm_err(as_rows(ga), wga) <= 1e-4
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16, torch.float16])
 def test_forced_plans(gpu, dtype):
-    full = 4 if dtype == torch.float32 else 8
-    bar = 1e-5 if dtype == torch.float32 else 1e-2
+    full = 16 // torch.empty(0, dtype=dtype).element_size()
+    bar = {torch.float32: 1e-5, torch.float64: 1e-13}.get(dtype, 1e-2)
     g = torch.Generator().manual_seed(17)
     cases = []
     for shape in [(3, 301, 64 * full + full), (2, 77, 3 * full), (1, 1500, 256), (2, 5, 130), (4, 64, 33)]:
-        a = torch.rand(shape, generator=g).to(dtype)
-        b = torch.randn(shape, generator=g).to(dtype)
-        gh = torch.randn(shape, generator=g).to(dtype)
+        a = torch.rand(shape, generator=g, dtype=torch.float64).to(dtype)
+        b = torch.randn(shape, generator=g, dtype=torch.float64).to(dtype)
+        gh = torch.randn(shape, generator=g, dtype=torch.float64).to(dtype)
         h = oracle.fwd(as_rows(a), as_rows(b))
         hs = torch.from_numpy(h).mT.contiguous().to(dtype)
         ga, gb = oracle.bwd(as_rows(a), as_rows(hs), as_rows(gh))
@@ -81,7 +83,8 @@ def test_forced_plans(gpu, dtype):
     n = 0
     for vec in (full, 1):
         for steps in ((2, 4, 8) if vec == full else (4, 8, 16)):
-            max_waves = min(16, 64 // vec, (512 if (vec > 1 and steps >= 8) else 1024) // 64)
+            csize = 8 if dtype == torch.float64 else 4
+            max_waves = min(16, 65536 // (4 * vec * 64 * csize), (512 if (vec > 1 and steps >= 8) else 1024) // 64)
             for waves in sorted({1, 3, max_waves}):
                 plan = hip.Plan(vec=vec, unroll=steps, waves=waves)
                 for shape, a, b, gh, hs, h, ga, gb, hp in cases:

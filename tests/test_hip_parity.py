@@ -26,6 +26,7 @@ from scanscam_amd import hip
 pytestmark = pytest.mark.gpu
 
 FP32_BAR = 1e-5
+FP64_BAR = 1e-13
 HALF_BAR = 1e-2
 
 
@@ -65,7 +66,21 @@ def row_norm_err(x, ref):
 
 
 def to_np(t):
-    return t.detach().float().cpu().numpy()
+    t = t.detach().cpu()
+    return (t if t.dtype == torch.float64 else t.float()).numpy()
+
+
+def upcast(t):
+    """The oracle's view of a tensor: float64 stays, everything else is exactly upcast to float32."""
+    return (t if t.dtype == torch.float64 else t.float()).numpy()
+
+
+def full_vec(dtype):
+    return 16 // torch.empty(0, dtype=dtype).element_size()
+
+
+def bar_for(dtype):
+    return {torch.float32: FP32_BAR, torch.float64: FP64_BAR}.get(dtype, HALF_BAR)
 
 
 def run_fwd(gpu, a, b, plan=None):
@@ -183,7 +198,7 @@ def test_benchmark_config_16bit(gpu, dtype):
 # small inputs with ragged rows and lengths.
 # ---------------------------------------------------------------------------
 def plans_for(dtype):
-    full = 4 if dtype == torch.float32 else 8
+    full = full_vec(dtype)
     out = []
     for vec in (full, 1):
         unrolls = (1, 2, 4, 8) if vec == full else (1, 4)
@@ -197,20 +212,20 @@ def plans_for(dtype):
     return out
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16, torch.float16])
 def test_forced_plans_row_and_lookback(gpu, dtype):
-    full = 4 if dtype == torch.float32 else 8
-    bar = FP32_BAR if dtype == torch.float32 else HALF_BAR
+    full = full_vec(dtype)
+    bar = bar_for(dtype)
     g = seeded(7)
     cases = {}
     for rows, T in [(5, 8 * full * 37), (3, 64 * full * 5 + full), (1, 64 * full * 33), (7, 1037), (2, 64 * full)]:
-        a = torch.rand((rows, T), generator=g).to(dtype)
-        b = torch.randn((rows, T), generator=g).to(dtype)
-        gh = torch.randn((rows, T), generator=g).to(dtype)
-        h = oracle.fwd(a.float().numpy(), b.float().numpy())
+        a = torch.rand((rows, T), generator=g, dtype=torch.float64).to(dtype)
+        b = torch.randn((rows, T), generator=g, dtype=torch.float64).to(dtype)
+        gh = torch.randn((rows, T), generator=g, dtype=torch.float64).to(dtype)
+        h = oracle.fwd(upcast(a), upcast(b))
         hs = torch.from_numpy(h).to(dtype)
-        ga, gb = oracle.bwd(a.float().numpy(), hs.float().numpy(), gh.float().numpy())
-        cases[(rows, T)] = (a.to(gpu), b.to(gpu), gh.to(gpu), hs.to(gpu), h, ga, gb, prev_abs(hs.float().numpy()))
+        ga, gb = oracle.bwd(upcast(a), upcast(hs), upcast(gh))
+        cases[(rows, T)] = (a.to(gpu), b.to(gpu), gh.to(gpu), hs.to(gpu), h, ga, gb, prev_abs(upcast(hs)))
     n = 0
     for plan in plans_for(dtype):
         for (rows, T), (a, b, gh, hs, h, ga, gb, hp) in cases.items():
@@ -226,10 +241,10 @@ def test_forced_plans_row_and_lookback(gpu, dtype):
     assert n > 100
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16])
 def test_forced_plans_small(gpu, dtype):
-    full = 4 if dtype == torch.float32 else 8
-    bar = FP32_BAR if dtype == torch.float32 else HALF_BAR
+    full = full_vec(dtype)
+    bar = bar_for(dtype)
     g = seeded(8)
     n = 0
     for vec, unroll, waves in itertools.product((full, 1), (1, 2, 4, 8), (1, 4)):
@@ -239,18 +254,18 @@ def test_forced_plans_small(gpu, dtype):
         for T in lengths:
             for rows in (1, 37, 515):
                 plan = hip.Plan(mode=hip.MODE_SMALL, vec=vec, unroll=unroll, waves=waves)
-                a = torch.rand((rows, T), generator=g).to(dtype)
-                b = torch.randn((rows, T), generator=g).to(dtype)
-                gh = torch.randn((rows, T), generator=g).to(dtype)
+                a = torch.rand((rows, T), generator=g, dtype=torch.float64).to(dtype)
+                b = torch.randn((rows, T), generator=g, dtype=torch.float64).to(dtype)
+                gh = torch.randn((rows, T), generator=g, dtype=torch.float64).to(dtype)
                 print(f"case small {dtype} rows={rows} T={T} {plan}", flush=True)
-                h = oracle.fwd(a.float().numpy(), b.float().numpy())
+                h = oracle.fwd(upcast(a), upcast(b))
                 hs = torch.from_numpy(h).to(dtype)
-                ga, gb = oracle.bwd(a.float().numpy(), hs.float().numpy(), gh.float().numpy())
+                ga, gb = oracle.bwd(upcast(a), upcast(hs), upcast(gh))
                 got_h = run_fwd(gpu, a, b, plan)
                 got_ga, got_gb = run_bwd(gpu, a, hs, gh, plan)
                 assert rel_err(to_np(got_h), h) <= bar, (plan, rows, T)
                 assert rel_err(to_np(got_gb), gb) <= bar, (plan, rows, T)
-                assert rel_err(to_np(got_ga), ga, prev_abs(hs.float().numpy())) <= bar, (plan, rows, T)
+                assert rel_err(to_np(got_ga), ga, prev_abs(upcast(hs))) <= bar, (plan, rows, T)
                 n += 1
     assert n > 100
 
@@ -377,3 +392,20 @@ def test_nonfinite_rows_do_not_leak_into_other_rows(gpu):
         assert np.all(np.isfinite(h[r])) and rel_err(h[r], want[r]) <= FP32_BAR
     assert np.all(np.isfinite(h[2, :100])) and not np.any(np.isfinite(h[2, 100:110]))
     assert np.all(np.isnan(h[4, 7:]))
+
+
+@pytest.mark.parametrize("shape", [(32, 1025), (32, 4100), (3, 300001), (4, 64), (16, 2, 5)])
+def test_float64(gpu, shape):
+    # The reference also dispatches double (src/scanscam_cpu.hpp:43): fp64 storage and arithmetic.
+    g = seeded(300 + sum(shape))
+    a = torch.rand(shape, generator=g, dtype=torch.float64)
+    b = torch.randn(shape, generator=g, dtype=torch.float64)
+    gh = torch.randn(shape, generator=g, dtype=torch.float64)
+    h = run_fwd(gpu, a, b)
+    assert h.dtype == torch.float64
+    want = oracle.fwd(a.numpy(), b.numpy())
+    assert rel_err(to_np(h), want) <= FP64_BAR
+    ga, gb = run_bwd(gpu, a, torch.from_numpy(want), gh)
+    wga, wgb = oracle.bwd(a.numpy(), want, gh.numpy())
+    assert rel_err(to_np(gb), wgb) <= FP64_BAR
+    assert rel_err(to_np(ga), wga, prev_abs(want)) <= FP64_BAR

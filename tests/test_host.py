@@ -88,7 +88,7 @@ def test_gpu_entry_points_reject_cpu_tensors_and_unknown_dtypes():
     with pytest.raises(RuntimeError, match="GPU tensor"):
         hip.blocked_linear_scan_backward(x, x, x)
     with pytest.raises(TypeError):
-        hip.resolve_plan(4, 8, torch.float64)
+        hip.resolve_plan(4, 8, torch.int32)
 
 
 def test_package_never_imports_the_oracle():

@@ -90,7 +90,7 @@ def test_wrapper_names_of_the_reference(gpu):
     with pytest.raises(AssertionError):
         hip.blocked_linear_scan_forward(a, b[:, :64])
     with pytest.raises(TypeError):
-        hip.blocked_linear_scan_forward(a.double(), b.double())
+        hip.blocked_linear_scan_forward(a.long(), b.long())
 
 
 def test_runs_on_the_current_stream(gpu):
@@ -105,3 +105,17 @@ def test_runs_on_the_current_stream(gpu):
     want = oracle.fwd(a.cpu().numpy(), b.cpu().numpy())
     assert rel_err(h.cpu().numpy(), want) <= 1e-5
     assert np.isfinite(float(total))
+
+
+def test_float64_gradcheck_on_gpu(gpu):
+    # The reference dispatches float and double; with double storage the op passes
+    # torch.autograd.gradcheck directly on the GPU kernels.
+    g = torch.Generator().manual_seed(61)
+    a = torch.rand((2, 3, 37), generator=g, dtype=torch.float64).to(gpu).requires_grad_()
+    b = torch.randn((2, 3, 37), generator=g, dtype=torch.float64).to(gpu).requires_grad_()
+    assert torch.autograd.gradcheck(scanscam_amd.scan, (a, b), eps=1e-6, atol=1e-7)
+    # ... and through the channels-last kernels.
+    a2 = torch.rand((2, 37, 5), generator=g, dtype=torch.float64).to(gpu).mT.requires_grad_()
+    b2 = torch.randn((2, 37, 5), generator=g, dtype=torch.float64).to(gpu).mT.requires_grad_()
+    assert op.is_transpose_contig(a2)
+    assert torch.autograd.gradcheck(scanscam_amd.scan, (a2, b2), eps=1e-6, atol=1e-7)
