@@ -140,6 +140,56 @@ def time_batches(sets, launches, warmup, hip, torch):
     return out[0], out[1]
 
 
+def reference_grid(dev, args, hip, torch):
+    """The shapes the reference's own timing tests use, fp32 N(0,1) inputs.
+
+    Row layout: scanscam/cpu_test.py:51-77 and scanscam/cuda_test.py:166-247
+    ((8,256,4096), (8,256,32), (256,4096), (16384,4096)); channels-last:
+    cuda_test.py:250-308 ((8,4096,512) stored [B, T, C]). Mean microseconds per
+    launch over back-to-back launches on rotated buffer sets.
+    """
+    out = {}
+    for shape in ((8, 256, 4096), (8, 256, 32), (256, 4096), (16384, 4096)):
+        torch.manual_seed(0)
+        x, y, z = torch.randn(shape), torch.randn(shape), torch.randn(shape)
+        first = DeviceSet(x, y, z, dev, torch)
+        n = x.numel()
+        nsets = max(1, min(64, -(-(1 << 30) // (24 * n))))
+        sets = [first] + [first.clone(torch) for _ in range(nsets - 1)]
+        f_ms, b_ms = time_batches(sets, max(4 * args.steps, 4 * nsets), max(args.warmup, nsets), hip, torch)
+        out["x".join(map(str, shape))] = {
+            "fwd_us": round(f_ms * 1e3, 2), "bwd_us": round(b_ms * 1e3, 2),
+            "fwd_GBps": round(12 * n / (f_ms * 1e-3) / 1e9, 1), "bwd_GBps": round(20 * n / (b_ms * 1e-3) / 1e9, 1),
+        }
+        del sets, first
+        torch.cuda.empty_cache()
+    # Channels-last: logical [8, 512, 4096] stored [8, 4096, 512].
+    torch.manual_seed(0)
+    shape = (8, 4096, 512)
+    x, y, z = (torch.randn(shape).to(dev) for _ in range(3))
+    h = hip.transposed_linear_scan_forward(x, y)
+    n = x.numel()
+    times = []
+    for fn in (lambda: hip.transposed_linear_scan_forward(x, y),
+               lambda: hip.transposed_linear_scan_backward(x, h, z)):
+        for _ in range(args.warmup):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(args.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        times.append(e0.elapsed_time(e1) / args.steps)
+    out["channels_last_8x4096x512"] = {
+        "fwd_us": round(times[0] * 1e3, 2), "bwd_us": round(times[1] * 1e3, 2),
+        "fwd_GBps": round(12 * n / (times[0] * 1e-3) / 1e9, 1), "bwd_GBps": round(20 * n / (times[1] * 1e-3) / 1e9, 1),
+        "note": "includes the wrapper's output allocation; working set fits the Infinity Cache",
+    }
+    return out
+
+
 def cpu_baseline(a, b, gh, reps):
     """The reference's CPU loop on the same tensors, one thread."""
     import numpy as np
@@ -309,6 +359,9 @@ def main():
             del csets, first
             torch.cuda.empty_cache()
         out["configs"] = others
+
+    if not args.no_configs:
+        out["reference_grid"] = reference_grid(dev, args, hip, torch)
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(a, b, gh, reps=5)
