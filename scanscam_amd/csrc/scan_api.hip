@@ -245,14 +245,16 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     } else if (!vec_possible) {
         l->vec = 1;
     } else {
-        // A workgroup owns 64*vec channels of one batch element for all of T: prefer the
-        // 16-byte vector unless that leaves most of the GPU without a workgroup.
-        l->vec = (batch * groups(full) >= 256 || groups(1) == groups(full)) ? full : 1;
+        // A workgroup owns 64*vec channels of one batch element. Enough of them: 16-byte loads.
+        // Not enough, but enough with one channel per lane: narrower loads beat a second pass
+        // over the data. Fewer still: 16-byte loads and time split over workgroups (below).
+        l->vec = (batch * groups(full) >= 256 || batch * groups(1) < 256) ? full : 1;
     }
     if (l->vec != 1 && l->vec != full) return SCANSCAM_EPLAN;
     if (l->vec == full && full != 1 && !vec_possible) return SCANSCAM_EPLAN;
+    const bool split_auto = u.mode != kModeRow && u.mode != kModeLookback && batch * groups(l->vec) < 256;
 
-    l->steps = u.unroll ? u.unroll : (l->vec == 1 ? 8 : 4);
+    l->steps = u.unroll ? u.unroll : (l->vec == 1 || (split_auto && full <= 4) ? 8 : 4);
     const bool steps_ok = (l->vec == full) ? (l->steps == 2 || l->steps == 4 || l->steps == 8)
                                            : (l->steps == 4 || l->steps == 8 || l->steps == 16);
     if (!steps_ok) return SCANSCAM_EPLAN;
@@ -269,17 +271,41 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     } else {
         const int64_t segments = (T + l->steps - 1) / l->steps;  // no more waves than segments of time
         l->waves = segments < max_waves ? pow2_ceil(segments) : max_waves;
+        if (split_auto && l->waves > 8) l->waves = 8;  // shorter tiles: more segments to hand out
         if (l->waves > max_waves) l->waves = max_waves;
     }
     if (l->waves < 1 || l->waves > max_waves) return SCANSCAM_EPLAN;
-    l->grid = batch * groups(l->vec);
+    // Too few (batch element, channel group) pairs to fill the GPU: cut time into segments over
+    // workgroups as well. mode = SCANSCAM_MODE_ROW forces one segment, SCANSCAM_MODE_LOOKBACK
+    // forces the split (waves_per_row then gives the number of segments).
+    const int64_t rowgroups = batch * groups(l->vec);
+    const int64_t tile_steps = (int64_t)l->waves * l->steps;
+    const int64_t tiles = (T + tile_steps - 1) / tile_steps;
+    int64_t want = 1;
+    if (u.mode == kModeLookback) {
+        want = u.waves_per_row ? u.waves_per_row : 4;
+    } else if (split_auto) {
+        want = 512 / rowgroups;
+        if (want > 32) want = 32;
+        if (want < 2) want = 2;
+    }
+    if (want > tiles) want = tiles;
+    if (want < 1) want = 1;
+    const int64_t tiles_per_seg = (tiles + want - 1) / want;
+    l->seg_steps = (int)(tiles_per_seg * tile_steps);
+    l->segments = (int)((T + l->seg_steps - 1) / l->seg_steps);
+    l->grid = rowgroups * l->segments;
     if (l->grid >= (int64_t(1) << 31)) return SCANSCAM_EINVAL;
     l->lds_bytes = (size_t)4 * l->waves * l->vec * kWave * csize;
+    l->ws_bytes = 0;
+    if (l->segments > 1)
+        l->ws_bytes = (size_t)(rowgroups * kCounterStride +
+                               rowgroups * l->segments * 2 * l->vec * kWave * value_words(dtype)) * sizeof(uint64_t);
     return SCANSCAM_OK;
 }
 
 int run_cl(bool rev, const void *a, const void *x, const void *h, void *y0, void *y1, int64_t batch, int64_t T,
-           int64_t C, int dtype, void *stream, const scanscam_plan *plan)
+           int64_t C, int dtype, void *workspace, size_t workspace_bytes, void *stream, const scanscam_plan *plan)
 {
     const int esize = elem_size(dtype);
     if (esize == 0) return SCANSCAM_EDTYPE;
@@ -306,8 +332,20 @@ int run_cl(bool rev, const void *a, const void *x, const void *h, void *y0, void
     args.batch = batch;
     args.T = (int32_t)T;
     args.C = (int32_t)C;
+    args.segments = l.segments;
+    args.seg_steps = l.seg_steps;
+    args.ws = nullptr;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (l.segments > 1) {
+        if (!workspace || workspace_bytes < l.ws_bytes) return SCANSCAM_EWORKSPACE;
+        if (!aligned_to(workspace, 8)) return SCANSCAM_EALIGN;
+        args.ws = static_cast<uint64_t *>(workspace);
+        const int64_t words = (int64_t)(l.ws_bytes / sizeof(uint64_t));
+        hipLaunchKernelGGL(scan_ws_clear_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, s, args.ws,
+                           words);
+        if (hipGetLastError() != hipSuccess) return SCANSCAM_ELAUNCH;
+    }
     hipError_t e = hipErrorInvalidValue;
     switch (dtype) {
     case SCANSCAM_F32: e = scanscam::launch_scan_cl<float>(args, l, rev, s); break;
@@ -373,15 +411,29 @@ size_t scanscam_workspace_bytes_plan(int64_t rows, int64_t T, int dtype, int dir
 }
 
 int scanscam_scan_fwd_cl(const void *a, const void *b, void *h, int64_t batch, int64_t T, int64_t C, int dtype,
-                         void *stream, const scanscam_plan *plan)
+                         void *workspace, size_t workspace_bytes, void *stream, const scanscam_plan *plan)
 {
-    return run_cl(false, a, b, nullptr, h, nullptr, batch, T, C, dtype, stream, plan);
+    return run_cl(false, a, b, nullptr, h, nullptr, batch, T, C, dtype, workspace, workspace_bytes, stream, plan);
 }
 
 int scanscam_scan_bwd_cl(const void *a, const void *h, const void *gh, void *ga, void *gb, int64_t batch,
-                         int64_t T, int64_t C, int dtype, void *stream, const scanscam_plan *plan)
+                         int64_t T, int64_t C, int dtype, void *workspace, size_t workspace_bytes, void *stream,
+                         const scanscam_plan *plan)
 {
-    return run_cl(true, a, gh, h, gb, ga, batch, T, C, dtype, stream, plan);
+    return run_cl(true, a, gh, h, gb, ga, batch, T, C, dtype, workspace, workspace_bytes, stream, plan);
+}
+
+size_t scanscam_workspace_bytes_cl(int64_t batch, int64_t T, int64_t C, int dtype, int direction,
+                                   const scanscam_plan *plan)
+{
+    (void)direction;
+    if (elem_size(dtype) == 0 || batch <= 0 || T <= 0 || C <= 0 || T >= kMaxT || C >= kMaxT) return 0;
+    size_t need = 0;
+    for (int al = 0; al < 2; al++) {
+        scanscam::ClLaunch l;
+        if (resolve_cl(plan, batch, T, C, dtype, al != 0, &l) == SCANSCAM_OK && l.ws_bytes > need) need = l.ws_bytes;
+    }
+    return need;
 }
 
 int scanscam_resolve_plan(int64_t rows, int64_t T, int dtype, int direction, const scanscam_plan *plan,

@@ -125,6 +125,8 @@ template <typename ST, int VEC> struct Vec {
         return *q;
 #endif
     }
+    // For data that is read a second time soon: left to the caches' normal policy.
+    static __device__ __forceinline__ raw_t load_cached(const ST *p) { return *reinterpret_cast<const raw_t *>(p); }
     static __device__ __forceinline__ void store(ST *p, raw_t r)
     {
         raw_t *q = reinterpret_cast<raw_t *>(p);

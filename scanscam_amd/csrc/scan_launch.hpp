@@ -63,8 +63,11 @@ struct ClLaunch {
     int vec;
     int steps;
     int waves;
+    int segments;   // > 1: time is also split over workgroups (scan_cl_split_kernel)
+    int seg_steps;
     int64_t grid;
     size_t lds_bytes;
+    size_t ws_bytes;
 };
 
 constexpr int cl_max_threads(int vec, int steps) { return (vec > 1 && steps >= 8) ? 512 : 1024; }
@@ -75,8 +78,13 @@ hipError_t launch_scan_cl(const ClArgs &args, const ClLaunch &l, bool rev, hipSt
 #define SCANSCAM_CL_CASE(ST, VEC, S)                                                                   \
     if (l.vec == (VEC) && l.steps == (S)) {                                                            \
         constexpr int MAXT = cl_max_threads(VEC, S);                                                   \
-        if (rev) hipLaunchKernelGGL((scan_cl_kernel<ST, VEC, S, true, MAXT>), grid, block, l.lds_bytes, stream, args);  \
-        else     hipLaunchKernelGGL((scan_cl_kernel<ST, VEC, S, false, MAXT>), grid, block, l.lds_bytes, stream, args); \
+        if (l.segments > 1) {                                                                          \
+            if (rev) hipLaunchKernelGGL((scan_cl_split_kernel<ST, VEC, S, true, MAXT>), grid, block, l.lds_bytes, stream, args);  \
+            else     hipLaunchKernelGGL((scan_cl_split_kernel<ST, VEC, S, false, MAXT>), grid, block, l.lds_bytes, stream, args); \
+        } else {                                                                                       \
+            if (rev) hipLaunchKernelGGL((scan_cl_kernel<ST, VEC, S, true, MAXT>), grid, block, l.lds_bytes, stream, args);  \
+            else     hipLaunchKernelGGL((scan_cl_kernel<ST, VEC, S, false, MAXT>), grid, block, l.lds_bytes, stream, args); \
+        }                                                                                              \
         return hipGetLastError();                                                                      \
     }
 

@@ -65,10 +65,12 @@ def _bind(path: str) -> ctypes.CDLL:
     lib.scanscam_scan_bwd_plan.restype = i32
     lib.scanscam_workspace_bytes_plan.argtypes = [i64, i64, i32, i32, plan_p]
     lib.scanscam_workspace_bytes_plan.restype = sz
-    lib.scanscam_scan_fwd_cl.argtypes = [p, p, p, i64, i64, i64, i32, p, plan_p]
+    lib.scanscam_scan_fwd_cl.argtypes = [p, p, p, i64, i64, i64, i32, p, sz, p, plan_p]
     lib.scanscam_scan_fwd_cl.restype = i32
-    lib.scanscam_scan_bwd_cl.argtypes = [p, p, p, p, p, i64, i64, i64, i32, p, plan_p]
+    lib.scanscam_scan_bwd_cl.argtypes = [p, p, p, p, p, i64, i64, i64, i32, p, sz, p, plan_p]
     lib.scanscam_scan_bwd_cl.restype = i32
+    lib.scanscam_workspace_bytes_cl.argtypes = [i64, i64, i64, i32, i32, plan_p]
+    lib.scanscam_workspace_bytes_cl.restype = sz
     lib.scanscam_resolve_plan.argtypes = [i64, i64, i32, i32, plan_p, plan_p]
     lib.scanscam_resolve_plan.restype = i32
     lib.scanscam_strerror.argtypes = [i32]
@@ -297,6 +299,15 @@ def blocked_linear_scan_backward(
     return linear_scan_backward(x, y, z)
 
 
+def _workspace_cl(L, batch: int, T: int, C: int, dtype: torch.dtype, direction: int, plan_ref,
+                  device: torch.device) -> Tuple[Optional[torch.Tensor], int, int]:
+    n = int(L.scanscam_workspace_bytes_cl(batch, T, C, _dtype_code(dtype), direction, plan_ref))
+    if n == 0:
+        return None, 0, 0
+    ws = torch.empty(n, dtype=torch.uint8, device=device)
+    return ws, ws.data_ptr(), n
+
+
 def _check_channels_last(*tensors: torch.Tensor) -> None:
     first = tensors[0]
     for t in tensors:
@@ -324,10 +335,11 @@ def transposed_linear_scan_forward(x: torch.Tensor, y: torch.Tensor, channels_pe
     batch, T, C = x.shape
     if x.numel() == 0:
         return out
+    plan_ref = ctypes.byref(plan) if plan is not None else None
     with torch.cuda.device(x.device):
+        ws, ws_ptr, ws_n = _workspace_cl(L, batch, T, C, x.dtype, FORWARD, plan_ref, x.device)
         rc = L.scanscam_scan_fwd_cl(x.data_ptr(), y.data_ptr(), out.data_ptr(), batch, T, C, _dtype_code(x.dtype),
-                                    torch.cuda.current_stream().cuda_stream,
-                                    ctypes.byref(plan) if plan is not None else None)
+                                    ws_ptr, ws_n, torch.cuda.current_stream().cuda_stream, plan_ref)
     if rc != 0:
         raise RuntimeError(f"scanscam_scan_fwd_cl: {strerror(rc)}")
     return out
@@ -345,10 +357,12 @@ def transposed_linear_scan_backward(x: torch.Tensor, y: torch.Tensor, z: torch.T
     batch, T, C = x.shape
     if x.numel() == 0:
         return out_a, out_b
+    plan_ref = ctypes.byref(plan) if plan is not None else None
     with torch.cuda.device(x.device):
+        ws, ws_ptr, ws_n = _workspace_cl(L, batch, T, C, x.dtype, BACKWARD, plan_ref, x.device)
         rc = L.scanscam_scan_bwd_cl(x.data_ptr(), y.data_ptr(), z.data_ptr(), out_a.data_ptr(), out_b.data_ptr(),
-                                    batch, T, C, _dtype_code(x.dtype), torch.cuda.current_stream().cuda_stream,
-                                    ctypes.byref(plan) if plan is not None else None)
+                                    batch, T, C, _dtype_code(x.dtype), ws_ptr, ws_n,
+                                    torch.cuda.current_stream().cuda_stream, plan_ref)
     if rc != 0:
         raise RuntimeError(f"scanscam_scan_bwd_cl: {strerror(rc)}")
     return out_a, out_b

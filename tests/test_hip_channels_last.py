@@ -85,8 +85,11 @@ def test_forced_plans(gpu, dtype):
         for steps in ((2, 4, 8) if vec == full else (4, 8, 16)):
             csize = 8 if dtype == torch.float64 else 4
             max_waves = min(16, 65536 // (4 * vec * 64 * csize), (512 if (vec > 1 and steps >= 8) else 1024) // 64)
-            for waves in sorted({1, 3, max_waves}):
-                plan = hip.Plan(vec=vec, unroll=steps, waves=waves)
+            shapes_plans = [hip.Plan(vec=vec, unroll=steps, waves=waves, mode=hip.MODE_ROW) for waves in sorted({1, 3, max_waves})]
+            # Time split over workgroups: 2, 3 and 7 segments (more than there are tiles is clamped).
+            shapes_plans += [hip.Plan(vec=vec, unroll=steps, waves=waves, mode=hip.MODE_LOOKBACK, waves_per_row=nseg)
+                             for waves, nseg in ((1, 7), (2, 3), (max_waves, 2))]
+            for plan in shapes_plans:
                 for shape, a, b, gh, hs, h, ga, gb, hp in cases:
                     if vec != 1 and shape[-1] % full != 0:
                         continue
@@ -97,7 +100,7 @@ def test_forced_plans(gpu, dtype):
                     assert rel_err(as_rows(got_gb), gb) <= bar, (plan, shape)
                     assert rel_err(as_rows(got_ga), ga, hp) <= bar, (plan, shape)
                     n += 1
-    assert n > 40
+    assert n > 80
 
 
 def test_matches_row_layout_kernels(gpu):
@@ -130,3 +133,20 @@ def test_empty_and_argument_checks(gpu):
         hip.transposed_linear_scan_forward(x[0], x[0])  # not 3-D
     with pytest.raises(RuntimeError):
         hip.transposed_linear_scan_forward(x, x, plan=hip.Plan(vec=4, unroll=3))
+
+
+def test_time_split_is_chosen_for_few_channels_and_is_reproducible(gpu):
+    # [8, 4096, 512]: 16 (batch element, channel group) pairs would leave most of the GPU idle,
+    # so the automatic plan cuts time into segments; results must not depend on timing.
+    g = torch.Generator(device=gpu).manual_seed(23)
+    x = torch.rand((8, 4096, 512), generator=g, device=gpu)
+    y = torch.randn((8, 4096, 512), generator=g, device=gpu)
+    assert hip.lib().scanscam_workspace_bytes_cl(8, 4096, 512, 0, 0, None) > 0
+    first = hip.transposed_linear_scan_forward(x, y)
+    whole = hip.transposed_linear_scan_forward(x, y, plan=hip.Plan(mode=hip.MODE_ROW))
+    assert float((first - whole).abs().max()) <= 2e-5
+    for _ in range(3):
+        assert torch.equal(hip.transposed_linear_scan_forward(x, y), first)
+    ga0, gb0 = hip.transposed_linear_scan_backward(x, first, y)
+    ga1, gb1 = hip.transposed_linear_scan_backward(x, first, y)
+    assert torch.equal(ga0, ga1) and torch.equal(gb0, gb1)
