@@ -1,0 +1,117 @@
+// Measurement aid, not part of the library: plain streaming kernels of known size.
+//
+//   stream_probe copy [MiB]   one kernel that reads MiB and writes MiB: what rocprofv3's FETCH_SIZE and
+//                             WRITE_SIZE counters read for a known number of bytes (their scale factors)
+//   stream_probe ceiling      scan-free kernels with the access shape of the scan kernels at
+//                             16384 rows x 4096 fp32 (one 256-thread workgroup per row, four 16-byte
+//                             non-temporal loads per lane per stream): 2 reads + 1 write like the
+//                             forward scan, 3 reads + 2 writes like the backward scan. What the memory
+//                             system gives that access shape when no scan is done at all.
+//
+//   hipcc -O3 --offload-arch=gfx950 stream_probe.hip -o stream_probe
+#include <hip/hip_runtime.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+typedef unsigned u4 __attribute__((ext_vector_type(4)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+#define CHECK(call)                                                                   \
+    do {                                                                              \
+        hipError_t e_ = (call);                                                       \
+        if (e_ != hipSuccess) {                                                       \
+            fprintf(stderr, "%s: %s\n", #call, hipGetErrorString(e_));                \
+            exit(1);                                                                  \
+        }                                                                             \
+    } while (0)
+
+__global__ __launch_bounds__(256) void copy_calib_kernel(const u4 *__restrict__ in, u4 *__restrict__ out, size_t n)
+{
+    size_t i = (size_t)blockIdx.x * 1024 + threadIdx.x;
+#pragma unroll
+    for (int k = 0; k < 4; k++, i += 256)
+        if (i < n) __builtin_nontemporal_store(__builtin_nontemporal_load(in + i), out + i);
+}
+
+// READS input streams, WRITES output streams; workgroup b covers vectors [b*1024, (b+1)*1024), wave w its
+// quarter, four consecutive 1 KiB spans per wave -- the layout of scan_row_kernel<float, 4, 4>.
+template <int READS, int WRITES>
+__global__ __launch_bounds__(256) void stream_shape_kernel(const f4 *__restrict__ a, const f4 *__restrict__ b,
+                                                           const f4 *__restrict__ c, f4 *__restrict__ o0,
+                                                           f4 *__restrict__ o1)
+{
+    const size_t base = (size_t)blockIdx.x * 1024 + (threadIdx.x / 64) * 256 + (threadIdx.x % 64);
+    f4 va[4], vb[4], vc[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        va[u] = __builtin_nontemporal_load(a + base + u * 64);
+        if (READS > 1) vb[u] = __builtin_nontemporal_load(b + base + u * 64);
+        if (READS > 2) vc[u] = __builtin_nontemporal_load(c + base + u * 64);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        f4 r = va[u];
+        if (READS > 1) r += vb[u];
+        if (READS > 2) r *= vc[u];
+        __builtin_nontemporal_store(r, o0 + base + u * 64);
+        if (WRITES > 1) __builtin_nontemporal_store(r + 1.0f, o1 + base + u * 64);
+    }
+}
+
+template <typename F> static float mean_ms(F launch, int reps)
+{
+    hipEvent_t e0, e1;
+    CHECK(hipEventCreate(&e0));
+    CHECK(hipEventCreate(&e1));
+    for (int i = 0; i < 3; i++) launch();
+    CHECK(hipEventRecord(e0, 0));
+    for (int i = 0; i < reps; i++) launch();
+    CHECK(hipEventRecord(e1, 0));
+    CHECK(hipEventSynchronize(e1));
+    float ms = 0;
+    CHECK(hipEventElapsedTime(&ms, e0, e1));
+    return ms / reps;
+}
+
+static int run_copy(size_t mib)
+{
+    const size_t bytes = mib << 20, n = bytes / 16;
+    u4 *in, *out;
+    CHECK(hipMalloc(&in, bytes));
+    CHECK(hipMalloc(&out, bytes));
+    CHECK(hipMemset(in, 1, bytes));
+    CHECK(hipMemset(out, 0, bytes));
+    const float ms = mean_ms(
+        [&] { hipLaunchKernelGGL(copy_calib_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, 0, in, out, n); }, 20);
+    printf("copy_calib: %zu MiB read + %zu MiB written per launch, %.1f us per launch, %.1f GB/s\n", mib, mib,
+           ms * 1e3, 2.0 * bytes / (ms * 1e-3) / 1e9);
+    return hipDeviceSynchronize() == hipSuccess ? 0 : 1;
+}
+
+static int run_ceiling()
+{
+    const size_t rows = 16384, T = 4096, n = rows * T, bytes = n * 4;
+    f4 *buf[5];
+    for (auto &p : buf) {
+        CHECK(hipMalloc(&p, bytes));
+        CHECK(hipMemset(p, 0, bytes));
+    }
+    const dim3 grid((unsigned)rows), block(256);
+    const float fwd = mean_ms([&] { hipLaunchKernelGGL((stream_shape_kernel<2, 1>), grid, block, 0, 0, buf[0], buf[1], buf[2], buf[3], buf[4]); }, 30);
+    const float bwd = mean_ms([&] { hipLaunchKernelGGL((stream_shape_kernel<3, 2>), grid, block, 0, 0, buf[0], buf[1], buf[2], buf[3], buf[4]); }, 30);
+    printf("stream ceiling, 16384 x 4096 fp32, one workgroup per row:\n");
+    printf("  2 reads + 1 write (forward shape):  %7.1f us  %7.1f GB/s  %4.1f %% of 8 TB/s\n", fwd * 1e3,
+           3.0 * bytes / (fwd * 1e-3) / 1e9, 3.0 * bytes / (fwd * 1e-3) / 8e12 * 100);
+    printf("  3 reads + 2 writes (backward shape): %7.1f us  %7.1f GB/s  %4.1f %% of 8 TB/s\n", bwd * 1e3,
+           5.0 * bytes / (bwd * 1e-3) / 1e9, 5.0 * bytes / (bwd * 1e-3) / 8e12 * 100);
+    return hipDeviceSynchronize() == hipSuccess ? 0 : 1;
+}
+
+int main(int argc, char **argv)
+{
+    if (argc > 1 && strcmp(argv[1], "ceiling") == 0) return run_ceiling();
+    if (argc > 1 && strcmp(argv[1], "copy") == 0) return run_copy(argc > 2 ? (size_t)atol(argv[2]) : 1024);
+    fprintf(stderr, "usage: %s copy [MiB] | ceiling\n", argv[0]);
+    return 2;
+}
