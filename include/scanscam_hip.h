@@ -66,6 +66,9 @@ enum {
  *   unroll         64-lane chunks per wave per tile: 1, 2, 4 or 8 (1 or 4 when vec == 1)
  *   waves          waves per workgroup, 1..16 (at most 8 when unroll == 4, 4 when unroll == 8)
  *   waves_per_row  ROW only: power of two dividing `waves`
+ *   spin_limit     kernels that wait for another workgroup's carry poll at most this many times
+ *                  (0 = 2^20, about a second); a wait that expires sets word 1 of the workspace to 1
+ *                  and poisons the affected outputs with NaN instead of spinning for ever
  */
 typedef struct scanscam_plan {
     int32_t mode;
@@ -73,6 +76,7 @@ typedef struct scanscam_plan {
     int32_t unroll;
     int32_t waves;
     int32_t waves_per_row;
+    int32_t spin_limit;
 } scanscam_plan;
 
 /*

@@ -77,7 +77,7 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
     if (esize == 0) return SCANSCAM_EDTYPE;
     if (rows < 0 || T < 0 || T >= kMaxT) return SCANSCAM_EINVAL;
     const int full = 16 / esize;
-    scanscam_plan u = {0, 0, 0, 0, 0};
+    scanscam_plan u = {0, 0, 0, 0, 0, 0};
     if (user) u = *user;
 
     Launch &l = out->l;
@@ -207,6 +207,7 @@ int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y
     args.counters = r.counters;
     args.desc_base = r.counters * kCounterStride;
     args.super_base = r.super_base;
+    args.spin_limit = (plan && plan->spin_limit > 0) ? plan->spin_limit : scanscam::kSpinLimit;
     args.ws = nullptr;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -236,7 +237,7 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
 {
     const int esize = elem_size(dtype);
     const int full = 16 / esize;
-    scanscam_plan u = {0, 0, 0, 0, 0};
+    scanscam_plan u = {0, 0, 0, 0, 0, 0};
     if (user) u = *user;
     const bool vec_possible = aligned16 && (C % full == 0);
     auto groups = [&](int vec) { return (C + (int64_t)kWave * vec - 1) / ((int64_t)kWave * vec); };
@@ -335,6 +336,7 @@ int run_cl(bool rev, const void *a, const void *x, const void *h, void *y0, void
     args.segments = l.segments;
     args.seg_steps = l.seg_steps;
     args.ws = nullptr;
+    args.spin_limit = (plan && plan->spin_limit > 0) ? plan->spin_limit : scanscam::kSpinLimit;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (l.segments > 1) {
@@ -449,6 +451,7 @@ int scanscam_resolve_plan(int64_t rows, int64_t T, int dtype, int direction, con
     out->unroll = r.l.unroll;
     out->waves = r.l.waves;
     out->waves_per_row = r.l.mode == kModeRow ? r.l.wpr : 0;
+    out->spin_limit = (plan && plan->spin_limit > 0) ? plan->spin_limit : scanscam::kSpinLimit;
     return SCANSCAM_OK;
 }
 

@@ -42,6 +42,7 @@ struct ClArgs {
     int32_t segments;   // split kernel: segments of time per (batch element, channel group)
     int32_t seg_steps;  // split kernel: time steps per segment (a multiple of the tile)
     uint64_t *ws;       // split kernel: ticket counters + segment aggregates
+    int32_t spin_limit; // split kernel: polls before a wait gives up
 };
 
 // One workgroup's view of its channels: pointers already offset to (batch
@@ -279,7 +280,7 @@ __global__ __launch_bounds__(MAXT) void scan_cl_split_kernel(const ClArgs p)
             const uint64_t *theirs = segs + (int64_t)q * kSegWords;
             CT pa[VEC], pb[VEC];
             bool got = false;
-            for (int spin = 0; spin < kSpinLimit && !got; spin++) {
+            for (int spin = 0; spin < p.spin_limit && !got; spin++) {
                 bool ready = true;
 #pragma unroll
                 for (int k = 0; k < VEC; k++) {

@@ -70,6 +70,7 @@ struct ScanArgs {
     int32_t counters;       // LOOKBACK: number of ticket counters (row r uses counter r % counters)
     int32_t desc_base;      // LOOKBACK: first tile-descriptor word of the workspace
     int64_t super_base;     // LOOKBACK: first super-tile-descriptor word of the workspace
+    int32_t spin_limit;     // LOOKBACK: polls before a wait gives up
     uint64_t *ws;           // LOOKBACK: ticket counters + tile descriptors
 };
 
@@ -560,11 +561,11 @@ template <> struct Desc<double> {
     }
 };
 
-// Polls of the look-back loop before a wave gives up. Tickets make every
+// Default number of polls before a waiting wave gives up. Tickets make every
 // awaited tile belong to a workgroup that is already running, so the limit is
 // never reached in a correct launch (a poll is a memory round trip; the limit
-// is seconds). It exists so that no wave can spin for ever: on expiry the wave
-// raises word kTimeoutWord of the workspace and carries NaN onwards.
+// is about a second). It exists so that no wave can spin for ever: on expiry
+// the wave raises word kTimeoutWord of the workspace and carries NaN onwards.
 constexpr int kSpinLimit = 1 << 20;
 constexpr int kTimeoutWord = 1;
 
@@ -597,7 +598,7 @@ __device__ __forceinline__ CT lookback_carry(const ScanArgs &p, int64_t row, int
 
     bool tiles_done = false, super_done = false;
     CT PA = CT(1), PB = CT(0), S = CT(0);
-    for (int spin = 0; spin < kSpinLimit; spin++) {
+    for (int spin = 0; spin < p.spin_limit; spin++) {
         if (!have_t) {
             const uint64_t *d = trow + (int64_t)(m * kSuper + lane) * TW;
             CT va, vb;

@@ -40,6 +40,7 @@ class Plan(ctypes.Structure):
         ("unroll", ctypes.c_int32),
         ("waves", ctypes.c_int32),
         ("waves_per_row", ctypes.c_int32),
+        ("spin_limit", ctypes.c_int32),
     ]
 
     def __repr__(self) -> str:

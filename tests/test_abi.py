@@ -59,8 +59,8 @@ def test_strerror_covers_every_code():
 
 
 def test_plan_struct_layout_matches_header():
-    assert ctypes.sizeof(hip.Plan) == 20
-    assert [f[0] for f in hip.Plan._fields_] == ["mode", "vec", "unroll", "waves", "waves_per_row"]
+    assert ctypes.sizeof(hip.Plan) == 24
+    assert [f[0] for f in hip.Plan._fields_] == ["mode", "vec", "unroll", "waves", "waves_per_row", "spin_limit"]
 
 
 def test_argument_errors_are_reported_before_any_launch():

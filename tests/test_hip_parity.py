@@ -409,3 +409,34 @@ def test_float64(gpu, shape):
     wga, wgb = oracle.bwd(a.numpy(), want, gh.numpy())
     assert rel_err(to_np(gb), wgb) <= FP64_BAR
     assert rel_err(to_np(ga), wga, prev_abs(want)) <= FP64_BAR
+
+
+def test_expired_wait_is_reported_and_every_wave_exits(gpu):
+    # A look-back wait that gives up must not hang: with one poll allowed the launch still
+    # completes, and either every tile found its predecessors in that one poll (results right)
+    # or word 1 of the workspace is raised and the affected outputs are NaN.
+    import ctypes
+
+    rows, T = 2, 1 << 18
+    g = torch.Generator(device=gpu).manual_seed(6)
+    a = torch.rand((rows, T), generator=g, device=gpu)
+    b = torch.randn((rows, T), generator=g, device=gpu)
+    good = hip.linear_scan_forward(a, b, hip.Plan(mode=hip.MODE_LOOKBACK, vec=4, unroll=1, waves=1))
+    plan = hip.Plan(mode=hip.MODE_LOOKBACK, vec=4, unroll=1, waves=1, spin_limit=1)
+    n = hip.workspace_bytes(rows, T, torch.float32, hip.FORWARD, plan)
+    ws = torch.empty(n, dtype=torch.uint8, device=gpu)
+    out = torch.empty_like(a)
+    rc = hip.lib().scanscam_scan_fwd_plan(a.data_ptr(), b.data_ptr(), out.data_ptr(), rows, T, 0, ws.data_ptr(), n,
+                                          torch.cuda.current_stream().cuda_stream, ctypes.byref(plan))
+    assert rc == 0
+    torch.cuda.synchronize()  # returns: no wave is left spinning
+    expired = int(ws.view(torch.int64)[1].item()) != 0
+    if expired:
+        assert bool(torch.isnan(out).any())
+        ok = ~torch.isnan(out)
+        assert torch.equal(out[ok], good[ok]) or float((out[ok] - good[ok]).abs().max()) <= 1e-4
+    else:
+        assert torch.equal(out, good)
+    # The default limit on the same input: no expiry, right answer.
+    again = hip.linear_scan_forward(a, b, hip.Plan(mode=hip.MODE_LOOKBACK, vec=4, unroll=1, waves=1))
+    assert torch.equal(again, good)
