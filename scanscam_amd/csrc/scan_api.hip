@@ -221,14 +221,40 @@ int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y
         if (hipGetLastError() != hipSuccess) return SCANSCAM_ELAUNCH;
     }
 
-    hipError_t e = hipErrorInvalidValue;
-    switch (dtype) {
-    case SCANSCAM_F32: e = scanscam::launch_scan<float>(args, r.l, rev, s); break;
-    case SCANSCAM_BF16: e = scanscam::launch_scan<__bf16>(args, r.l, rev, s); break;
-    case SCANSCAM_F16: e = scanscam::launch_scan<_Float16>(args, r.l, rev, s); break;
-    case SCANSCAM_F64: e = scanscam::launch_scan<double>(args, r.l, rev, s); break;
+    // One launch may hold at most 2^32 - 1 threads. Rows are independent, so a ROW or SMALL launch
+    // that would exceed it is issued as several launches over consecutive slabs of rows (only
+    // tensors of tens of GB get there). LOOKBACK grids are far below the limit by construction.
+    const int64_t threads = (int64_t)r.l.waves * kWave;
+    const int64_t max_grid = ((int64_t(1) << 32) - 1) / threads;
+    int64_t rows_per_wg = 1;
+    if (r.l.mode == kModeRow) rows_per_wg = r.l.waves / r.l.wpr;
+    if (r.l.mode == kModeSmall) rows_per_wg = (int64_t)r.l.waves * r.l.unroll * (kWave / r.l.group);
+    const int64_t slab_rows = (r.l.mode == kModeLookback || r.l.grid <= max_grid) ? rows : max_grid * rows_per_wg;
+
+    for (int64_t row0 = 0; row0 < rows; row0 += slab_rows) {
+        const int64_t n = rows - row0 < slab_rows ? rows - row0 : slab_rows;
+        const int64_t byte_off = row0 * T * esize;
+        ScanArgs slab = args;
+        Launch l = r.l;
+        if (slab_rows != rows) {
+            slab.a = static_cast<const char *>(a) + byte_off;
+            slab.x = static_cast<const char *>(x) + byte_off;
+            slab.h = h ? static_cast<const char *>(h) + byte_off : nullptr;
+            slab.y0 = static_cast<char *>(y0) + byte_off;
+            slab.y1 = y1 ? static_cast<char *>(y1) + byte_off : nullptr;
+            slab.rows = n;
+            l.grid = (n + rows_per_wg - 1) / rows_per_wg;
+        }
+        hipError_t e = hipErrorInvalidValue;
+        switch (dtype) {
+        case SCANSCAM_F32: e = scanscam::launch_scan<float>(slab, l, rev, s); break;
+        case SCANSCAM_BF16: e = scanscam::launch_scan<__bf16>(slab, l, rev, s); break;
+        case SCANSCAM_F16: e = scanscam::launch_scan<_Float16>(slab, l, rev, s); break;
+        case SCANSCAM_F64: e = scanscam::launch_scan<double>(slab, l, rev, s); break;
+        }
+        if (e != hipSuccess) return SCANSCAM_ELAUNCH;
     }
-    return e == hipSuccess ? SCANSCAM_OK : SCANSCAM_ELAUNCH;
+    return SCANSCAM_OK;
 }
 
 // Channels-last: choice of vector width, steps per wave and waves per workgroup.

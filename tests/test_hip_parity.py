@@ -440,3 +440,21 @@ def test_expired_wait_is_reported_and_every_wave_exits(gpu):
     # The default limit on the same input: no expiry, right answer.
     again = hip.linear_scan_forward(a, b, hip.Plan(mode=hip.MODE_LOOKBACK, vec=4, unroll=1, waves=1))
     assert torch.equal(again, good)
+
+
+def test_launch_is_split_when_a_grid_would_exceed_2_pow_32_threads(gpu):
+    # 1024-thread workgroups, one row each: 2^22 workgroups is the most one launch can hold, so
+    # 2^22 + 1000 rows must be issued as two launches over slabs of rows.
+    rows, T = (1 << 22) + 1000, 16
+    g = torch.Generator(device=gpu).manual_seed(8)
+    a = torch.rand((rows, T), generator=g, device=gpu)
+    b = torch.randn((rows, T), generator=g, device=gpu)
+    plan = hip.Plan(mode=hip.MODE_ROW, vec=4, unroll=1, waves=16, waves_per_row=16)
+    h = hip.linear_scan_forward(a, b, plan)
+    want = hip.linear_scan_forward(a, b)  # automatic plan: the small-row kernel, one launch
+    assert float((h - want).abs().max()) <= 1e-5
+    tail = slice(rows - 2000, rows)  # rows on both sides of the slab border, against the oracle
+    assert rel_err(to_np(h[tail]), oracle.fwd(to_np(a[tail]), to_np(b[tail]))) <= FP32_BAR
+    ga, gb = hip.linear_scan_backward(a, h, b, plan)
+    wga, wgb = hip.linear_scan_backward(a, h, b)
+    assert float((gb - wgb).abs().max()) <= 1e-5 and float((ga - wga).abs().max()) <= 1e-4
