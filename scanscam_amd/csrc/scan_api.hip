@@ -81,11 +81,15 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
     if (user) u = *user;
 
     Launch &l = out->l;
-    l = Launch{0, 0, 0, 0, 1, 64, 0};
-    const bool vec_possible = aligned16 && (T % full == 0);
-    l.vec = u.vec ? u.vec : (vec_possible ? full : 1);
+    l = Launch{0, 0, 0, 0, 1, 64, 0, false};
+    // The full 16-byte vector needs rows that start on 16-byte borders -- or, for rows longer than one
+    // chunk, the element-aligned ("ragged") variants of the ROW and LOOKBACK kernels.
+    const bool vec_aligned = aligned16 && (T % full == 0);
+    const bool ragged_possible = full > 1 && T > (int64_t)kWave * full && u.mode != kModeSmall;
+    l.vec = u.vec ? u.vec : ((vec_aligned || ragged_possible) ? full : 1);
     if (l.vec != 1 && l.vec != full) return SCANSCAM_EPLAN;
-    if (l.vec == full && full != 1 && !vec_possible) return SCANSCAM_EPLAN;
+    l.ragged = l.vec == full && full != 1 && !vec_aligned;
+    if (l.ragged && !ragged_possible) return SCANSCAM_EPLAN;
 
     const int64_t chunk = (int64_t)kWave * l.vec;
     const int64_t nch64 = (T + chunk - 1) / chunk;
@@ -162,6 +166,10 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
         return SCANSCAM_EPLAN;
     }
 
+    if (l.ragged) {
+        if (!u.unroll && l.unroll < 2) l.unroll = 2;  // instantiated for 2 and 4 chunks per wave
+        if (l.unroll != 2 && l.unroll != 4) return SCANSCAM_EPLAN;
+    }
     if (!unroll_ok(l.vec, full, l.unroll)) return SCANSCAM_EPLAN;
     if (l.waves < 1 || l.waves > scanscam::kMaxWaves ||
         l.waves * kWave > scanscam::max_threads_for_unroll(l.unroll))

@@ -126,6 +126,32 @@ template <typename ST, int VEC> struct Vec {
         return *q;
 #endif
     }
+    // The same accesses for a vector that is only element-aligned (rows of a length that is not a
+    // multiple of VEC start anywhere): still one 16-byte instruction, the memory pipeline splits it.
+    typedef raw_t raw_unaligned_t __attribute__((aligned(sizeof(ST))));
+    static __device__ __forceinline__ raw_t load_unaligned(const ST *p)
+    {
+        return __builtin_nontemporal_load(reinterpret_cast<const raw_unaligned_t *>(p));
+    }
+    static __device__ __forceinline__ void store_unaligned(ST *p, raw_t r)
+    {
+        __builtin_nontemporal_store(r, reinterpret_cast<raw_unaligned_t *>(p));
+    }
+    // The first n (< VEC) elements only, the rest zero: the partial vector at the end of a row.
+    static __device__ __forceinline__ raw_t load_head(const ST *p, int n)
+    {
+        Elems<ST, VEC> e;
+#pragma unroll
+        for (int k = 0; k < VEC; k++) e.e[k] = (k < n) ? p[k] : (ST)0.0f;
+        return __builtin_bit_cast(raw_t, e);
+    }
+    static __device__ __forceinline__ void store_head(ST *p, raw_t r, int n)
+    {
+        const Elems<ST, VEC> e = __builtin_bit_cast(Elems<ST, VEC>, r);
+#pragma unroll
+        for (int k = 0; k < VEC; k++)
+            if (k < n) p[k] = e.e[k];
+    }
     // For data that is read a second time soon: left to the caches' normal policy.
     static __device__ __forceinline__ raw_t load_cached(const ST *p) { return *reinterpret_cast<const raw_t *>(p); }
     static __device__ __forceinline__ void store(ST *p, raw_t r)
@@ -229,7 +255,11 @@ __device__ __forceinline__ void wave_scan(CT &A, CT &B, int j)
 // With CHAIN the U chunks are consecutive in scan order (carry flows from one
 // into the next); without it they are unrelated rows (SMALL kernel).
 // ---------------------------------------------------------------------------
-template <typename ST, int VEC, int U, bool REV, bool GROUPED, bool CHAIN>
+// With RAGGED, rows may start at any element (their length need not be a
+// multiple of VEC, bases need not be 16-byte aligned): vectors are loaded and
+// stored element-aligned, and the last vector of a row may hold fewer than VEC
+// elements (`count`), the rest being masked to the identity.
+template <typename ST, int VEC, int U, bool REV, bool GROUPED, bool CHAIN, bool RAGGED = false>
 struct WaveTile {
     using V = Vec<ST, VEC>;
     using raw_t = typename V::raw_t;
@@ -239,6 +269,23 @@ struct WaveTile {
     int64_t off[U];  // element offset of the vector from the tensor base
     int32_t m[U];    // vector index inside the row (element m*VEC)
     bool valid[U];   // inside the row (and the row exists)
+    int32_t count[RAGGED ? U : 1];  // RAGGED: elements of the vector inside the row (1..VEC)
+
+    __device__ __forceinline__ raw_t fetch(const ST *p, int u) const
+    {
+        if (!RAGGED) return V::load(p);
+        return count[u] >= VEC ? V::load_unaligned(p) : V::load_head(p, count[u]);
+    }
+    __device__ __forceinline__ void put(ST *p, raw_t r, int u) const
+    {
+        if (!RAGGED) {
+            V::store(p, r);
+        } else if (count[u] >= VEC) {
+            V::store_unaligned(p, r);
+        } else {
+            V::store_head(p, r, count[u]);
+        }
+    }
 
     raw_t ra[U], rx[U], rh[REV ? U : 1];
     CT edge_a[REV ? U : 1];  // a[(m+1)*VEC] for the first lane of a group
@@ -257,12 +304,12 @@ struct WaveTile {
             ra[u] = V::zero_raw();
             rx[u] = V::zero_raw();
             if (valid[u]) {
-                ra[u] = V::load(a + off[u]);
-                rx[u] = V::load(x + off[u]);
+                ra[u] = fetch(a + off[u], u);
+                rx[u] = fetch(x + off[u], u);
             }
             if (REV) {
                 rh[u] = V::zero_raw();
-                if (valid[u]) rh[u] = V::load(h + off[u]);
+                if (valid[u]) rh[u] = fetch(h + off[u], u);
                 edge_a[u] = CT(0);
                 edge_h[u] = CT(0);
                 // Neighbours that no lane of this group holds. With CHAIN the chunks of a
@@ -300,7 +347,8 @@ struct WaveTile {
             if (!REV) {
 #pragma unroll
                 for (int k = 0; k < VEC; k++) {
-                    g[u][k] = valid[u] ? fa[k] : CT(1);
+                    const bool in_row = RAGGED ? (valid[u] && k < count[u]) : valid[u];
+                    g[u][k] = in_row ? fa[k] : CT(1);
                     v[u][k] = fx[k];  // zero-filled where invalid
                 }
             } else {
@@ -319,7 +367,10 @@ struct WaveTile {
 #pragma unroll
                 for (int k = 0; k < VEC; k++) {
                     const CT gk = (k == 0) ? a_next : fa[(VEC - k) % VEC];
-                    g[u][k] = valid[u] ? gk : CT(1);
+                    // Scan position k is element VEC-1-k of the vector; past the row's end it is the identity
+                    // (its a and gh read as 0, so the element below it sees gate 0, as t = T-1 must).
+                    const bool in_row = RAGGED ? (valid[u] && VEC - 1 - k < count[u]) : valid[u];
+                    g[u][k] = in_row ? gk : CT(1);
                     v[u][k] = fx[VEC - 1 - k];
                     hp[u][k] = (k == VEC - 1) ? h_prev : fh[(VEC - 2 - k) < 0 ? 0 : (VEC - 2 - k)];
                 }
@@ -374,7 +425,7 @@ struct WaveTile {
             if (CHAIN && u + 1 < U)
                 carry = fma_(read_lane(PA[u], 63), carry, read_lane(PB[u], 63));
             if (!REV) {
-                if (valid[u]) V::store(y0 + off[u], V::pack(out));
+                if (valid[u]) put(y0 + off[u], V::pack(out), u);
             } else {
                 CT gb[VEC], ga[VEC];
 #pragma unroll
@@ -383,8 +434,8 @@ struct WaveTile {
                     ga[VEC - 1 - k] = out[k] * hp[u][k];
                 }
                 if (valid[u]) {
-                    V::store(y0 + off[u], V::pack(gb));
-                    V::store(y1 + off[u], V::pack(ga));
+                    put(y0 + off[u], V::pack(gb), u);
+                    put(y1 + off[u], V::pack(ga), u);
                 }
             }
         }
@@ -396,7 +447,7 @@ struct WaveTile {
 // holds W / wpr rows. Tile = wpr * U chunks. Carries: FMA chunk to chunk, LDS
 // wave to wave, a register tile to tile.
 // ---------------------------------------------------------------------------
-template <typename ST, int VEC, int U, bool REV, int MAXT>
+template <typename ST, int VEC, int U, bool REV, int MAXT, bool RAGGED = false>
 __global__ __launch_bounds__(MAXT) void scan_row_kernel(const ScanArgs p)
 {
     using CT = typename ComputeOf<ST>::type;
@@ -424,7 +475,7 @@ __global__ __launch_bounds__(MAXT) void scan_row_kernel(const ScanArgs p)
     const int tile_chunks = wpr * U;
     const int ntiles = (p.nch + tile_chunks - 1) / tile_chunks;
 
-    WaveTile<ST, VEC, U, REV, false, true> w;
+    WaveTile<ST, VEC, U, REV, false, true, RAGGED> w;
     CT hp[REV ? U : 1][VEC];
     CT row_carry = CT(0);
 
@@ -437,6 +488,7 @@ __global__ __launch_bounds__(MAXT) void scan_row_kernel(const ScanArgs p)
             w.m[u] = m;
             w.valid[u] = row_ok && m >= 0 && (int64_t)m * VEC < p.T;
             w.off[u] = row_off + (int64_t)m * VEC;
+            if (RAGGED) w.count[u] = p.T - m * VEC;
         }
         w.load(p, lane, kWave - 1);
         w.reduce(lane, kWave - 1, hp);
@@ -666,7 +718,7 @@ __device__ __forceinline__ CT lookback_carry(const ScanArgs &p, int64_t row, int
     return j > 0 ? fma_(read_lane(PA, j - 1), S, read_lane(PB, j - 1)) : S;
 }
 
-template <typename ST, int VEC, int U, bool REV, int MAXT>
+template <typename ST, int VEC, int U, bool REV, int MAXT, bool RAGGED = false>
 __global__ __launch_bounds__(MAXT) void scan_lookback_kernel(const ScanArgs p)
 {
     using CT = typename ComputeOf<ST>::type;
@@ -700,7 +752,7 @@ __global__ __launch_bounds__(MAXT) void scan_lookback_kernel(const ScanArgs p)
     const int nvp = p.nch * kWave;
     const int chunk0 = (tile * nwaves + wave) * U;
 
-    WaveTile<ST, VEC, U, REV, false, true> w;
+    WaveTile<ST, VEC, U, REV, false, true, RAGGED> w;
     CT hp[REV ? U : 1][VEC];
 #pragma unroll
     for (int u = 0; u < U; u++) {
@@ -709,6 +761,7 @@ __global__ __launch_bounds__(MAXT) void scan_lookback_kernel(const ScanArgs p)
         w.m[u] = m;
         w.valid[u] = m >= 0 && (int64_t)m * VEC < p.T;
         w.off[u] = row_off + (int64_t)m * VEC;
+        if (RAGGED) w.count[u] = p.T - m * VEC;
     }
     w.load(p, lane, kWave - 1);
     w.reduce(lane, kWave - 1, hp);

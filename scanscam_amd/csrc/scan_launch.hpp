@@ -17,6 +17,7 @@ struct Launch {
     int wpr;     // ROW: waves per row
     int group;   // SMALL: lanes per row
     int64_t grid;
+    bool ragged; // ROW / LOOKBACK with the full vector on rows that start at any element
 };
 
 // Largest workgroup (threads) a kernel with U chunks per wave is compiled for.
@@ -43,12 +44,31 @@ hipError_t launch_scan(const ScanArgs &args, const Launch &l, bool rev, hipStrea
         return hipGetLastError();                                                                    \
     }
 
+// The same for rows that are only element-aligned (ROW and LOOKBACK, full vector, U = 2 or 4).
+#define SCANSCAM_RAGGED_CASE(ST, VEC, U)                                                             \
+    if (l.ragged && l.vec == (VEC) && l.unroll == (U)) {                                             \
+        constexpr int MAXT = max_threads_for_unroll(U);                                              \
+        if (l.mode == kModeRow) {                                                                    \
+            if (rev) hipLaunchKernelGGL((scan_row_kernel<ST, VEC, U, true, MAXT, true>), grid, block, 0, stream, args);      \
+            else     hipLaunchKernelGGL((scan_row_kernel<ST, VEC, U, false, MAXT, true>), grid, block, 0, stream, args);     \
+        } else if (l.mode == kModeLookback) {                                                        \
+            if (rev) hipLaunchKernelGGL((scan_lookback_kernel<ST, VEC, U, true, MAXT, true>), grid, block, 0, stream, args); \
+            else     hipLaunchKernelGGL((scan_lookback_kernel<ST, VEC, U, false, MAXT, true>), grid, block, 0, stream, args);\
+        } else {                                                                                     \
+            return hipErrorInvalidValue;                                                             \
+        }                                                                                            \
+        return hipGetLastError();                                                                    \
+    }
+
 #define SCANSCAM_DEFINE_LAUNCH(ST)                                                                   \
     template <>                                                                                      \
     hipError_t launch_scan<ST>(const ScanArgs &args, const Launch &l, bool rev, hipStream_t stream)  \
     {                                                                                                \
         constexpr int FULL = 16 / (int)sizeof(ST);                                                   \
         const dim3 grid((unsigned)l.grid), block((unsigned)(l.waves * kWave));                       \
+        SCANSCAM_RAGGED_CASE(ST, FULL, 2)                                                            \
+        SCANSCAM_RAGGED_CASE(ST, FULL, 4)                                                            \
+        if (l.ragged) return hipErrorInvalidValue;                                                   \
         SCANSCAM_LAUNCH_CASE(ST, FULL, 1)                                                            \
         SCANSCAM_LAUNCH_CASE(ST, FULL, 2)                                                            \
         SCANSCAM_LAUNCH_CASE(ST, FULL, 4)                                                            \

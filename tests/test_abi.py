@@ -83,10 +83,13 @@ def test_argument_errors_are_reported_before_any_launch():
                 hip.Plan(mode=hip.MODE_SMALL), hip.Plan(waves=17)):
         rc = L.scanscam_scan_fwd_plan(fake, fake, fake, 4, 4096, 0, None, 0, None, ctypes.byref(bad))
         assert rc == E_PLAN, bad
-    # vec 4 is impossible when T is not a multiple of 4 or a pointer is not 16-byte aligned.
+    # Rows no longer than one chunk can use the 16-byte vector only if they start on 16-byte borders.
     v4 = hip.Plan(vec=4)
-    assert L.scanscam_scan_fwd_plan(fake, fake, fake, 4, 1025, 0, None, 0, None, ctypes.byref(v4)) == E_PLAN
-    assert L.scanscam_scan_fwd_plan(fake + 4, fake, fake, 4, 1024, 0, None, 0, None, ctypes.byref(v4)) == E_PLAN
+    assert L.scanscam_scan_fwd_plan(fake, fake, fake, 4, 5, 0, None, 0, None, ctypes.byref(v4)) == E_PLAN
+    assert L.scanscam_scan_fwd_plan(fake + 4, fake, fake, 4, 64, 0, None, 0, None, ctypes.byref(v4)) == E_PLAN
+    # ... and element-aligned long rows only with 2 or 4 chunks per wave.
+    v4u8 = hip.Plan(vec=4, unroll=8)
+    assert L.scanscam_scan_fwd_plan(fake, fake, fake, 4, 1025, 0, None, 0, None, ctypes.byref(v4u8)) == E_PLAN
 
 
 def test_empty_inputs_are_a_successful_noop():
@@ -105,7 +108,7 @@ def test_empty_inputs_are_a_successful_noop():
         (16384, 2048, torch.bfloat16, hip.MODE_ROW, 8),     # 16-bit storage
         (16384, 2048, torch.float16, hip.MODE_ROW, 8),
         (131072, 64, torch.float32, hip.MODE_SMALL, 4),     # many short rows
-        (32, 1025, torch.float32, hip.MODE_ROW, 1),         # odd length: element-wise loads
+        (32, 1025, torch.float32, hip.MODE_ROW, 4),         # odd length: element-aligned 16-byte vectors
         (32, 5, torch.float32, hip.MODE_SMALL, 1),
     ],
 )
