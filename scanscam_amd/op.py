@@ -35,6 +35,23 @@ def scan(gate: torch.Tensor, value: torch.Tensor) -> torch.Tensor:
     return Scan.apply(gate, value)
 
 
+def _is_channels_last(x: torch.Tensor) -> bool:
+    """``[..., C, T]`` stored ``[..., T, C]``: the last two dimensions are transposed in memory.
+
+    ``is_transpose_contig`` (3-D only, as in the reference) is the common case; the
+    channels-last kernels take any number of leading dimensions, flattened to one
+    batch dimension, so 2-D and N-D tensors of this layout are scanned in place too
+    instead of being copied to row-contiguous storage first.
+    """
+    return x.dim() >= 2 and not x.is_contiguous() and x.mT.is_contiguous()
+
+
+def _as_batch_t_c(x: torch.Tensor) -> torch.Tensor:
+    """The ``[batch, T, C]`` contiguous view of a channels-last ``[..., C, T]`` tensor."""
+    xt = x.mT
+    return xt.reshape(-1, xt.shape[-2], xt.shape[-1])
+
+
 def _on_gpu(t: torch.Tensor) -> bool:
     # PyTorch-ROCm reports AMD GPUs with device type "cuda".
     return t.device.type == "cuda"
@@ -46,10 +63,11 @@ class Scan(torch.autograd.Function):
         if _on_gpu(gate):
             # Raises if the HIP library is missing: a GPU tensor is never
             # quietly scanned any other way.
-            if is_transpose_contig(gate) and is_transpose_contig(value):
-                # Stored [B, T, C]: scanned in place by the channels-last kernels
+            if gate.shape == value.shape and _is_channels_last(gate) and _is_channels_last(value):
+                # Stored [..., T, C]: scanned in place by the channels-last kernels
                 # (op.py:28-29 of the reference); the result keeps that layout.
-                output = hip.transposed_linear_scan_forward(gate.mT, value.mT).mT
+                out = hip.transposed_linear_scan_forward(_as_batch_t_c(gate), _as_batch_t_c(value))
+                output = out.reshape(gate.mT.shape).mT
             else:
                 output = hip.blocked_linear_scan_forward(gate, value)
         else:
@@ -61,9 +79,10 @@ class Scan(torch.autograd.Function):
     def backward(ctx: Any, output_grad: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
         gate, output = ctx.saved_tensors
         if _on_gpu(output_grad):
-            if is_transpose_contig(gate) and is_transpose_contig(output):
+            if _is_channels_last(gate) and _is_channels_last(output):
                 # What op.py:45-49 of the reference means to do (its call has one argument too many).
-                grads = hip.transposed_linear_scan_backward(gate.mT, output.mT, output_grad.mT.contiguous())
-                return tuple(g.mT for g in grads)
+                grads = hip.transposed_linear_scan_backward(
+                    _as_batch_t_c(gate), _as_batch_t_c(output), _as_batch_t_c(output_grad.mT.contiguous().mT))
+                return tuple(g.reshape(gate.mT.shape).mT for g in grads)
             return hip.blocked_linear_scan_backward(gate, output, output_grad)
         return naive_linear_scan_backward(gate, output, output_grad)

@@ -158,3 +158,24 @@ def test_hip_graph_capture_and_replay(gpu):
             for w, x in zip(want, got):
                 assert torch.equal(w, x), f"replay {replay} differs from the eager result"
         del scratch
+
+
+@pytest.mark.parametrize("shape", [(300, 40), (2, 3, 129, 24), (7, 5)])
+def test_transposed_storage_of_any_rank_is_scanned_in_place(gpu, shape):
+    # [..., C, T] tensors whose last two dimensions are transposed in memory (the reference's
+    # permute=True cases, scanscam/cpu_test.py:21-22) go to the channels-last kernels without a copy.
+    g = torch.Generator().manual_seed(81 + len(shape))
+    a = torch.rand(shape, generator=g)
+    b = torch.randn(shape, generator=g)
+    gh = torch.randn(shape, generator=g)
+    da = a.to(gpu).mT.contiguous().mT.requires_grad_()
+    db = b.to(gpu).mT.contiguous().mT.requires_grad_()
+    assert not da.is_contiguous() and da.mT.is_contiguous()
+    h = scanscam_amd.scan(da, db)
+    assert h.shape == da.shape and h.stride() == da.stride()
+    h.backward(gh.to(gpu))
+    want = oracle.fwd(a.numpy(), b.numpy())
+    assert rel_err(h.detach().cpu().numpy(), want) <= 1e-5
+    wga, wgb = oracle.bwd(a.numpy(), h.detach().cpu().numpy(), gh.numpy())
+    assert rel_err(da.grad.cpu().numpy(), wga, h.detach().cpu().numpy()) <= 1e-5
+    assert rel_err(db.grad.cpu().numpy(), wgb) <= 1e-5
