@@ -4,8 +4,6 @@
 
 #include "scan_launch.hpp"
 
-#include <stdlib.h>
-
 namespace {
 
 using scanscam::kCounterStride;
@@ -151,9 +149,6 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
         // One ticket counter per row up to kMaxCounters; when rows do not divide
         // evenly every counter gets the grid share of the fullest one.
         out->counters = (int)(rows < kMaxCounters ? rows : kMaxCounters);
-#ifdef SCANSCAM_EXPERIMENT
-        if (const char *e = getenv("SCANSCAM_COUNTERS")) out->counters = atoi(e) < rows ? atoi(e) : (int)rows;
-#endif
         const int64_t rows_per_counter = (rows + out->counters - 1) / out->counters;
         const int64_t tiles = rows * (int64_t)out->tiles_per_row;
         l.grid = (int64_t)out->counters * rows_per_counter * out->tiles_per_row;
