@@ -1,15 +1,18 @@
 """
 Binding of ``libscanscam_hip.so`` (C ABI in ``include/scanscam_hip.h``) and the
-``[rows, T]`` wrappers the autograd op calls.
+wrappers the autograd op calls.
 
 Takes the place of the reference's ``scanscam/cuda.py``: ``has_hip_ops`` is its
-``has_cuda_ops`` probe (``cuda.py:7-13``), and ``blocked_linear_scan_forward`` /
+``has_cuda_ops`` probe (``cuda.py:7-13``); ``blocked_linear_scan_forward`` /
 ``blocked_linear_scan_backward`` keep the names, argument order and behaviour of
 ``cuda.py:34-40`` and ``:56-66`` (inputs made contiguous, outputs allocated with
-``torch.empty_like``, any leading dimensions flattened). PyTorch is used for
-device memory and the current stream only; all arithmetic happens in the
-library's kernels. There is no other implementation behind these functions: if
-the library is missing they raise.
+``torch.empty_like``, any leading dimensions flattened), and
+``transposed_linear_scan_forward`` / ``transposed_linear_scan_backward`` those
+of ``cuda.py:69-95`` (contiguous ``[batch, T, C]`` tensors). Storage types:
+float32, float64, bfloat16, float16. PyTorch is used for device memory and the
+current stream only; all arithmetic happens in the library's kernels. There is
+no other implementation behind these functions: if the library is missing they
+raise.
 """
 import ctypes
 import functools

@@ -3,8 +3,10 @@ The user-facing op: ``scan(gate, value)`` and its ``torch.autograd.Function``.
 
 Same surface as the reference's ``scanscam/op.py:9-55``: ``scan`` applies
 ``Scan``; ``Scan.forward`` saves ``(gate, output)``; ``Scan.backward`` returns
-``(grad_gate, grad_value)``. Dispatch is by device as in ``op.py:27-35``: GPU
-tensors run the HIP kernels, everything else the tensor-level loop. Two
+``(grad_gate, grad_value)``. Dispatch is by device and layout as in
+``op.py:27-35``: GPU tensors run the HIP kernels (the channels-last ones when the
+last two dimensions are transposed in memory, the row ones otherwise),
+everything else the tensor-level loop. Two
 defects of the reference are not reproduced: its backward for transposed
 inputs calls a three-argument wrapper with four arguments (``op.py:46-48``),
 and its CPU backward drops its result (``op.py:52-53``); both return the
