@@ -293,15 +293,25 @@ struct WaveTile {
         const ST *h = static_cast<const ST *>(p.h);
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            ra[u] = V::zero_raw();
-            rx[u] = V::zero_raw();
-            if (valid[u]) {
-                ra[u] = fetch(a + off[u], u);
-                rx[u] = fetch(x + off[u], u);
+            if (!RAGGED) {
+                // Unconditional: lanes outside the row read element 0 of the tensor instead and are
+                // masked in reduce(). No branch separates the loads, so all of the wave's U x streams
+                // loads are in flight before the first one is waited for.
+                const int64_t o = valid[u] ? off[u] : 0;
+                ra[u] = V::load(a + o);
+                rx[u] = V::load(x + o);
+                if (REV) rh[u] = V::load(h + o);
+            } else {
+                ra[u] = V::zero_raw();
+                rx[u] = V::zero_raw();
+                if (REV) rh[u] = V::zero_raw();
+                if (valid[u]) {
+                    ra[u] = fetch(a + off[u], u);
+                    rx[u] = fetch(x + off[u], u);
+                    if (REV) rh[u] = fetch(h + off[u], u);
+                }
             }
             if (REV) {
-                rh[u] = V::zero_raw();
-                if (valid[u]) rh[u] = fetch(h + off[u], u);
                 edge_a[u] = CT(0);
                 edge_h[u] = CT(0);
                 // Neighbours that no lane of this group holds. With CHAIN the chunks of a
@@ -326,9 +336,9 @@ struct WaveTile {
             for (int u = 0; u < U; u++) {
                 CT t[VEC];
                 V::unpack(ra[u], t);
-                first_a[u] = t[0];
+                first_a[u] = valid[u] ? t[0] : CT(0);
                 V::unpack(rh[u], t);
-                last_h[u] = t[VEC - 1];
+                last_h[u] = valid[u] ? t[VEC - 1] : CT(0);
             }
         }
 #pragma unroll
@@ -336,6 +346,11 @@ struct WaveTile {
             CT fa[VEC], fx[VEC];
             V::unpack(ra[u], fa);
             V::unpack(rx[u], fx);
+#pragma unroll
+            for (int k = 0; k < VEC; k++) {  // lanes outside the row hold a = 0, x = 0
+                fa[k] = valid[u] ? fa[k] : CT(0);
+                fx[k] = valid[u] ? fx[k] : CT(0);
+            }
             if (!REV) {
 #pragma unroll
                 for (int k = 0; k < VEC; k++) {
@@ -346,6 +361,8 @@ struct WaveTile {
             } else {
                 CT fh[VEC];
                 V::unpack(rh[u], fh);
+#pragma unroll
+                for (int k = 0; k < VEC; k++) fh[k] = valid[u] ? fh[k] : CT(0);
                 // Scan order k <-> time t0 + VEC-1-k. gate = a[t+1], value = gh[t],
                 // hp = h[t-1]. Invalid lanes hold a = 0, so a neighbour past the
                 // end of the row reads as gate 0, which is what t = T-1 needs.

@@ -2,8 +2,8 @@
 //
 //   stream_probe copy [MiB]   one kernel that reads MiB and writes MiB: what rocprofv3's FETCH_SIZE and
 //                             WRITE_SIZE counters read for a known number of bytes (their scale factors)
-//   stream_probe ceiling      scan-free kernels with the access shape of the scan kernels at
-//                             16384 rows x 4096 fp32 (one 256-thread workgroup per row, four 16-byte
+//   stream_probe ceiling [rows]  scan-free kernels with the access shape of the scan kernels at
+//                             rows (default 16384) x 4096 fp32 (one 256-thread workgroup per row, four 16-byte
 //                             non-temporal loads per lane per stream): 2 reads + 1 write like the
 //                             forward scan, 3 reads + 2 writes like the backward scan. What the memory
 //                             system gives that access shape when no scan is done at all.
@@ -89,9 +89,9 @@ static int run_copy(size_t mib)
     return hipDeviceSynchronize() == hipSuccess ? 0 : 1;
 }
 
-static int run_ceiling()
+static int run_ceiling(size_t rows)
 {
-    const size_t rows = 16384, T = 4096, n = rows * T, bytes = n * 4;
+    const size_t T = 4096, n = rows * T, bytes = n * 4;
     f4 *buf[5];
     for (auto &p : buf) {
         CHECK(hipMalloc(&p, bytes));
@@ -100,7 +100,7 @@ static int run_ceiling()
     const dim3 grid((unsigned)rows), block(256);
     const float fwd = mean_ms([&] { hipLaunchKernelGGL((stream_shape_kernel<2, 1>), grid, block, 0, 0, buf[0], buf[1], buf[2], buf[3], buf[4]); }, 30);
     const float bwd = mean_ms([&] { hipLaunchKernelGGL((stream_shape_kernel<3, 2>), grid, block, 0, 0, buf[0], buf[1], buf[2], buf[3], buf[4]); }, 30);
-    printf("stream ceiling, 16384 x 4096 fp32, one workgroup per row:\n");
+    printf("stream ceiling, %zu x 4096 fp32, one workgroup per row:\n", rows);
     printf("  2 reads + 1 write (forward shape):  %7.1f us  %7.1f GB/s  %4.1f %% of 8 TB/s\n", fwd * 1e3,
            3.0 * bytes / (fwd * 1e-3) / 1e9, 3.0 * bytes / (fwd * 1e-3) / 8e12 * 100);
     printf("  3 reads + 2 writes (backward shape): %7.1f us  %7.1f GB/s  %4.1f %% of 8 TB/s\n", bwd * 1e3,
@@ -110,8 +110,8 @@ static int run_ceiling()
 
 int main(int argc, char **argv)
 {
-    if (argc > 1 && strcmp(argv[1], "ceiling") == 0) return run_ceiling();
+    if (argc > 1 && strcmp(argv[1], "ceiling") == 0) return run_ceiling(argc > 2 ? (size_t)atol(argv[2]) : 16384);
     if (argc > 1 && strcmp(argv[1], "copy") == 0) return run_copy(argc > 2 ? (size_t)atol(argv[2]) : 1024);
-    fprintf(stderr, "usage: %s copy [MiB] | ceiling\n", argv[0]);
+    fprintf(stderr, "usage: %s copy [MiB] | ceiling [rows]\n", argv[0]);
     return 2;
 }
