@@ -140,10 +140,12 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
         const int rows_per_wg = l.waves / l.wpr;
         l.grid = (rows + rows_per_wg - 1) / rows_per_wg;
     } else if (l.mode == kModeLookback) {
-        // Tiles of 32 chunks (8192 fp32 elements): fewer, larger tiles keep the
-        // carry chain short relative to the time a tile spends on its data.
+        // Tiles of 32 chunks (8192 fp32 elements): fewer, larger tiles keep the wait for the
+        // carry short relative to the time a tile spends on its data. With very few rows the
+        // tiles in flight are neighbours in one row, which publish almost together and so wait
+        // longest for each other: 64 chunks there.
         l.unroll = u.unroll ? u.unroll : 4;
-        l.waves = u.waves ? u.waves : 8;
+        l.waves = u.waves ? u.waves : (rows <= 16 && l.unroll <= 4 ? 16 : 8);
         const int tile_chunks = l.waves * l.unroll;
         out->tiles_per_row = (nch + tile_chunks - 1) / tile_chunks;
         // One ticket counter per row up to kMaxCounters; when rows do not divide

@@ -21,7 +21,7 @@ struct Launch {
 };
 
 // Largest workgroup (threads) a kernel with U chunks per wave is compiled for.
-constexpr int max_threads_for_unroll(int unroll) { return unroll <= 2 ? 1024 : unroll <= 4 ? 512 : 256; }
+constexpr int max_threads_for_unroll(int unroll) { return unroll <= 4 ? 1024 : 256; }
 
 // One per storage type, defined in scan_f32.hip / scan_bf16.hip / scan_f16.hip.
 // Returns hipErrorInvalidValue when (vec, unroll) is not an instantiated pair.

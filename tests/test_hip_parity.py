@@ -203,7 +203,7 @@ def plans_for(dtype):
     for vec in (full, 1):
         unrolls = (1, 2, 4, 8) if vec == full else (1, 4)
         for unroll in unrolls:
-            max_waves = 16 if unroll <= 2 else 8 if unroll == 4 else 4
+            max_waves = 16 if unroll <= 4 else 4
             for waves in sorted({1, 4, max_waves}):
                 for wpr in sorted({1, 2, waves} & {1, 2, 4, 8, 16}):
                     if waves % wpr == 0:

@@ -179,3 +179,24 @@ def test_transposed_storage_of_any_rank_is_scanned_in_place(gpu, shape):
     wga, wgb = oracle.bwd(a.numpy(), h.detach().cpu().numpy(), gh.numpy())
     assert rel_err(da.grad.cpu().numpy(), wga, h.detach().cpu().numpy()) <= 1e-5
     assert rel_err(db.grad.cpu().numpy(), wgb) <= 1e-5
+
+
+def test_concurrent_launches_on_two_streams(gpu):
+    # Two long-row scans (look-back kernels, each with its own workspace) in flight at once on
+    # different streams must neither disturb each other nor stall: waits only ever target
+    # workgroups of the same launch that already hold a ticket.
+    g = torch.Generator(device=gpu).manual_seed(91)
+    xs = [(torch.rand((6, 400000), generator=g, device=gpu), torch.randn((6, 400000), generator=g, device=gpu))
+          for _ in range(2)]
+    want = [hip.blocked_linear_scan_forward(a, b) for a, b in xs]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(device=gpu) for _ in range(2)]
+    got = [None, None]
+    for rep in range(3):
+        for i, (a, b) in enumerate(xs):
+            with torch.cuda.stream(streams[i]):
+                got[i] = hip.blocked_linear_scan_forward(a, b)
+        for s in streams:
+            s.synchronize()
+        for w, x in zip(want, got):
+            assert torch.equal(w, x)
