@@ -93,27 +93,35 @@ def time_kernels(sets, steps, warmup, hip, torch):
 
     Returns (wall seconds per step, mean fwd kernel ms, mean bwd kernel ms,
     min fwd ms, min bwd ms); the kernel times come from HIP events recorded on
-    the launch stream around every launch.
+    the launch stream around the launches of a sample of the steps.
     """
     calls = [(hip.prepare_forward(s.a, s.b, s.h), hip.prepare_backward(s.a, s.h, s.gh, s.ga, s.gb)) for s in sets]
     for i in range(warmup):
         f, b = calls[i % len(calls)]
         f()
         b()
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    # Events bracket the launches of every `stride`-th step only (at least 10 steps): an event pair
+    # around every launch would put ~3 us of event packets between all kernels of the timed region.
+    stride = max(1, steps // 10)
+    ev = {i: [torch.cuda.Event(enable_timing=True) for _ in range(3)] for i in range(0, steps, stride)}
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(steps):
         f, b = calls[i % len(calls)]
-        ev[i][0].record()
-        f()
-        ev[i][1].record()
-        b()
-        ev[i][2].record()
+        e = ev.get(i)
+        if e is None:
+            f()
+            b()
+        else:
+            e[0].record()
+            f()
+            e[1].record()
+            b()
+            e[2].record()
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / steps
-    fwd = [e[0].elapsed_time(e[1]) for e in ev]
-    bwd = [e[1].elapsed_time(e[2]) for e in ev]
+    fwd = [e[0].elapsed_time(e[1]) for e in ev.values()]
+    bwd = [e[1].elapsed_time(e[2]) for e in ev.values()]
     return wall, statistics.fmean(fwd), statistics.fmean(bwd), min(fwd), min(bwd)
 
 
