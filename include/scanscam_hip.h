@@ -126,10 +126,10 @@ size_t scanscam_workspace_bytes_plan(int64_t rows, int64_t T, int dtype, int dir
  * automatic): vec = channels per lane (16/sizeof(storage) or 1), unroll = time
  * steps per wave per tile (2, 4, 8 for the full vector; 4, 8, 16 for vec 1),
  * waves = waves per workgroup (1..16). When batch * C is too small to fill the
- * GPU, time is also cut into segments over workgroups, which needs a workspace
- * (scanscam_workspace_bytes_cl, same rules as above); mode = SCANSCAM_MODE_ROW
- * forbids that split, SCANSCAM_MODE_LOOKBACK forces it with waves_per_row
- * segments (4 if zero).
+ * GPU, time is also cut into tiles over workgroups, carried by a look-back
+ * chain, which needs a workspace (scanscam_workspace_bytes_cl, same rules as
+ * above); mode = SCANSCAM_MODE_ROW forbids that split, SCANSCAM_MODE_LOOKBACK
+ * forces it.
  */
 int scanscam_scan_fwd_cl(const void *a, const void *b, void *h, int64_t batch, int64_t T, int64_t C, int dtype,
                          void *workspace, size_t workspace_bytes, void *stream, const scanscam_plan *plan);

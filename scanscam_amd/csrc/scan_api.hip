@@ -284,16 +284,24 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     }
     if (l->vec != 1 && l->vec != full) return SCANSCAM_EPLAN;
     if (l->vec == full && full != 1 && !vec_possible) return SCANSCAM_EPLAN;
-    const bool split_auto = u.mode != kModeRow && u.mode != kModeLookback && batch * groups(l->vec) < 256;
+    // Too few (batch element, channel group) pairs to fill the GPU: cut time into tiles over
+    // workgroups as well. kind 0: one workgroup walks all of T. kind 2: tiles by ticket with a
+    // look-back chain of per-channel pairs (mode = SCANSCAM_MODE_LOOKBACK forces it,
+    // SCANSCAM_MODE_ROW forbids it).
+    const int64_t rowgroups = batch * groups(l->vec);
+    l->kind = 0;
+    if (u.mode == kModeLookback || (u.mode == SCANSCAM_MODE_AUTO && rowgroups < 256)) l->kind = 2;
+    if (u.mode == kModeSmall) return SCANSCAM_EPLAN;
 
-    l->steps = u.unroll ? u.unroll : (l->vec == 1 || (split_auto && full <= 4) ? 8 : 4);
+    l->steps = u.unroll ? u.unroll : (l->vec == 1 || (l->kind != 0 && full <= 4) ? 8 : 4);
     const bool steps_ok = (l->vec == full) ? (l->steps == 2 || l->steps == 4 || l->steps == 8)
                                            : (l->steps == 4 || l->steps == 8 || l->steps == 16);
     if (!steps_ok) return SCANSCAM_EPLAN;
 
-    // LDS: 2 buffers x (A, B) x [waves][vec][64] values, kept within 64 KiB.
+    // LDS arrays of [waves][vec][64] values, kept within 64 KiB: 2 buffers x (A, B), or 7 for kind 2.
     const int csize = compute_size(dtype);
-    const int max_by_lds = (64 * 1024) / (4 * l->vec * kWave * csize);
+    const int planes = l->kind == 2 ? 7 : 4;
+    const int max_by_lds = (64 * 1024) / (planes * l->vec * kWave * csize);
     const int max_by_threads = scanscam::cl_max_threads(l->vec, l->steps) / kWave;
     int max_waves = scanscam::kMaxWaves;
     if (max_waves > max_by_lds) max_waves = max_by_lds;
@@ -303,36 +311,30 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     } else {
         const int64_t segments = (T + l->steps - 1) / l->steps;  // no more waves than segments of time
         l->waves = segments < max_waves ? pow2_ceil(segments) : max_waves;
-        if (split_auto && l->waves > 8) l->waves = 8;  // shorter tiles: more segments to hand out
-        if (l->waves > max_waves) l->waves = max_waves;
+        if (l->kind != 0 && l->waves > 8) l->waves = 8;  // shorter tiles: more of them to hand out
+        while (l->waves > max_waves) l->waves >>= 1;
     }
     if (l->waves < 1 || l->waves > max_waves) return SCANSCAM_EPLAN;
-    // Too few (batch element, channel group) pairs to fill the GPU: cut time into segments over
-    // workgroups as well. mode = SCANSCAM_MODE_ROW forces one segment, SCANSCAM_MODE_LOOKBACK
-    // forces the split (waves_per_row then gives the number of segments).
-    const int64_t rowgroups = batch * groups(l->vec);
+
     const int64_t tile_steps = (int64_t)l->waves * l->steps;
     const int64_t tiles = (T + tile_steps - 1) / tile_steps;
-    int64_t want = 1;
-    if (u.mode == kModeLookback) {
-        want = u.waves_per_row ? u.waves_per_row : 4;
-    } else if (split_auto) {
-        want = 512 / rowgroups;
-        if (want > 32) want = 32;
-        if (want < 2) want = 2;
+    const int64_t vals = (int64_t)l->vec * kWave * value_words(dtype);  // words of one [vec][64] array of values
+    l->lds_bytes = (size_t)planes * l->waves * l->vec * kWave * csize;
+    l->ws_bytes = 0;
+    l->segments = 1;
+    if (l->kind == 2) {
+        if (tiles >= (int64_t(1) << 31)) return SCANSCAM_EINVAL;
+        l->segments = (int)tiles;  // the kernel's tiles per row-group
+        const int64_t supers = (tiles + l->waves - 1) / l->waves;
+        l->ws_bytes = (size_t)(rowgroups * kCounterStride + rowgroups * tiles * 2 * vals + rowgroups * supers * 4 * vals) *
+                      sizeof(uint64_t);
     }
-    if (want > tiles) want = tiles;
-    if (want < 1) want = 1;
-    const int64_t tiles_per_seg = (tiles + want - 1) / want;
-    l->seg_steps = (int)(tiles_per_seg * tile_steps);
-    l->segments = (int)((T + l->seg_steps - 1) / l->seg_steps);
+    if (l->segments <= 1) {  // nothing to split after all
+        l->kind = 0;
+        l->ws_bytes = 0;
+    }
     l->grid = rowgroups * l->segments;
     if (l->grid >= (int64_t(1) << 31)) return SCANSCAM_EINVAL;
-    l->lds_bytes = (size_t)4 * l->waves * l->vec * kWave * csize;
-    l->ws_bytes = 0;
-    if (l->segments > 1)
-        l->ws_bytes = (size_t)(rowgroups * kCounterStride +
-                               rowgroups * l->segments * 2 * l->vec * kWave * value_words(dtype)) * sizeof(uint64_t);
     return SCANSCAM_OK;
 }
 
@@ -365,12 +367,11 @@ int run_cl(bool rev, const void *a, const void *x, const void *h, void *y0, void
     args.T = (int32_t)T;
     args.C = (int32_t)C;
     args.segments = l.segments;
-    args.seg_steps = l.seg_steps;
     args.ws = nullptr;
     args.spin_limit = (plan && plan->spin_limit > 0) ? plan->spin_limit : scanscam::kSpinLimit;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (l.segments > 1) {
+    if (l.kind != 0) {
         if (!workspace || workspace_bytes < l.ws_bytes) return SCANSCAM_EWORKSPACE;
         if (!aligned_to(workspace, 8)) return SCANSCAM_EALIGN;
         args.ws = static_cast<uint64_t *>(workspace);

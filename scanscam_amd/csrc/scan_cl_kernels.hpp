@@ -19,11 +19,9 @@
 // element, like the row layout.
 //
 // A workgroup owns 64*VEC channels of one batch element. When that gives too
-// few workgroups to fill the GPU, time is also cut into segments over
-// workgroups (scan_cl_split_kernel): every workgroup first folds its segment
-// to one pair per channel (its data stays in the memory-side cache), publishes
-// it, collects the pairs of the segments before it, and only then replays its
-// segment from the resulting carry.
+// few workgroups to fill the GPU, time is also cut into tiles over workgroups
+// (scan_cl_lookback_kernel), with a decoupled look-back chain that carries one
+// affine pair per channel from tile to tile.
 #pragma once
 
 #include "scan_kernels.hpp"
@@ -39,10 +37,9 @@ struct ClArgs {
     int64_t batch;
     int32_t T;
     int32_t C;
-    int32_t segments;   // split kernel: segments of time per (batch element, channel group)
-    int32_t seg_steps;  // split kernel: time steps per segment (a multiple of the tile)
-    uint64_t *ws;       // split kernel: ticket counters + segment aggregates
-    int32_t spin_limit; // split kernel: polls before a wait gives up
+    int32_t segments;   // look-back kernel: tiles per (batch element, channel group)
+    uint64_t *ws;       // look-back kernel: ticket counters + published pairs
+    int32_t spin_limit; // look-back kernel: polls before a wait gives up
 };
 
 // One workgroup's view of its channels: pointers already offset to (batch
@@ -53,66 +50,111 @@ template <typename ST> struct ClLane {
     bool c_ok;
 };
 
+// One wave's S consecutive time steps of a tile, for the 64*VEC channels of the workgroup.
+//   load_fold   issues all loads and folds the steps to one affine pair per channel
+//   apply       replays the steps from the scan value entering them and stores the results
+// With APPLY = false only load_fold is used, and its loads are left cacheable (the data is
+// read again later).
+template <typename ST, int VEC, int S, bool REV, bool APPLY, typename CT>
+struct ClSteps {
+    using V = Vec<ST, VEC>;
+    using raw_t = typename V::raw_t;
+
+    CT g[S][VEC], v[S][VEC];
+    raw_t rh[(REV && APPLY) ? S : 1];
+    bool ok[S], h_ok[S];
+    int tau0;  // scan position of the first step
+
+    __device__ __forceinline__ void load_fold(const ClLane<ST> &ln, int T, int C, int first_step, int limit,
+                                              CT (&A)[VEC], CT (&B)[VEC])
+    {
+        tau0 = first_step;
+        // Every load is issued unconditionally, masked lanes from offset 0 of their own column (always
+        // valid), and masked by a select afterwards: no branch separates the loads, so all of a wave's
+        // S x streams loads are in flight before the first one is waited for.
+        raw_t ra[S], rx[S];
+        bool a_ok[S];
+#pragma unroll
+        for (int s = 0; s < S; s++) {
+            const int tau = tau0 + s;
+            const int t = REV ? T - 1 - tau : tau;
+            ok[s] = ln.c_ok && tau < limit;
+            // The gate of step t is a[t] forwards and a[t+1] backwards (0 past the end); h[-1] = 0.
+            a_ok[s] = ok[s] && (!REV || t + 1 < T);
+            h_ok[s] = ok[s] && t > 0;
+            const int64_t off_x = ok[s] ? (int64_t)t * C : 0;
+            const int64_t off_a = a_ok[s] ? (int64_t)(REV ? t + 1 : t) * C : 0;
+            if (APPLY) {
+                ra[s] = V::load(ln.a + off_a);
+                rx[s] = V::load(ln.x + off_x);
+                if (REV) rh[s] = V::load(ln.h + (h_ok[s] ? (int64_t)(t - 1) * C : 0));
+            } else {
+                ra[s] = V::load_cached(ln.a + off_a);
+                rx[s] = V::load_cached(ln.x + off_x);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < VEC; k++) {
+            A[k] = CT(1);
+            B[k] = CT(0);
+        }
+#pragma unroll
+        for (int s = 0; s < S; s++) {
+            CT fa[VEC], fx[VEC];
+            V::unpack(ra[s], fa);
+            V::unpack(rx[s], fx);
+#pragma unroll
+            for (int k = 0; k < VEC; k++) {
+                g[s][k] = ok[s] ? (a_ok[s] ? fa[k] : CT(0)) : CT(1);
+                v[s][k] = ok[s] ? fx[k] : CT(0);
+                B[k] = fma_(g[s][k], B[k], v[s][k]);
+                A[k] = A[k] * g[s][k];
+            }
+        }
+    }
+
+    __device__ __forceinline__ void apply(const ClLane<ST> &ln, int T, int C, CT (&mine)[VEC])
+    {
+#pragma unroll
+        for (int s = 0; s < S; s++) {
+            const int tau = tau0 + s;
+            const int t = REV ? T - 1 - tau : tau;
+            CT out[VEC];
+#pragma unroll
+            for (int k = 0; k < VEC; k++) {
+                mine[k] = fma_(g[s][k], mine[k], v[s][k]);
+                out[k] = mine[k];
+            }
+            if (!REV) {
+                if (ok[s]) V::store(ln.y0 + (int64_t)t * C, V::pack(out));
+            } else {
+                CT fh[VEC], ga[VEC];
+                V::unpack(rh[s], fh);
+#pragma unroll
+                for (int k = 0; k < VEC; k++) ga[k] = out[k] * (h_ok[s] ? fh[k] : CT(0));
+                if (ok[s]) {
+                    V::store(ln.y0 + (int64_t)t * C, V::pack(out));
+                    V::store(ln.y1 + (int64_t)t * C, V::pack(ga));
+                }
+            }
+        }
+    }
+};
+
 // Processes the tile of W*S steps that starts at scan position tile0.
 //   APPLY = true   `run` holds the scan value entering the tile per channel; the
 //                  tile's outputs are stored and `run` advanced to its end.
 //   APPLY = false  `runA`, `run` hold the affine pair of everything folded so
 //                  far; the tile's pair is composed onto it; nothing is stored
-//                  and loads are left cacheable (the data is read again later).
+//                  (kept for callers that only need a pair; unused by the kernels here).
 // lds_A / lds_B: [W][VEC][64] values each; the caller alternates two buffers.
 template <typename ST, int VEC, int S, bool REV, bool APPLY, typename CT>
 __device__ __forceinline__ void cl_tile(const ClLane<ST> &ln, int T, int C, int tile0, int limit, int wave, int W,
                                         int lane, CT *lds_A, CT *lds_B, CT (&runA)[VEC], CT (&run)[VEC])
 {
-    using V = Vec<ST, VEC>;
-    using raw_t = typename V::raw_t;
-    const int tau0 = tile0 + wave * S;  // position in scan order
-
-    // Every load is issued unconditionally, masked lanes from offset 0 of their own column (always
-    // valid), and masked by a select afterwards: no branch separates the loads, so all of a wave's
-    // S x streams loads are in flight before the first one is waited for.
-    raw_t ra[S], rx[S], rh[(REV && APPLY) ? S : 1];
-    bool ok[S], a_ok[S], h_ok[S];
-#pragma unroll
-    for (int s = 0; s < S; s++) {
-        const int tau = tau0 + s;
-        const int t = REV ? T - 1 - tau : tau;
-        ok[s] = ln.c_ok && tau < limit;
-        // The gate of step t is a[t] forwards and a[t+1] backwards (0 past the end); h[-1] = 0.
-        a_ok[s] = ok[s] && (!REV || t + 1 < T);
-        h_ok[s] = ok[s] && t > 0;
-        const int64_t off_x = ok[s] ? (int64_t)t * C : 0;
-        const int64_t off_a = a_ok[s] ? (int64_t)(REV ? t + 1 : t) * C : 0;
-        if (APPLY) {
-            ra[s] = V::load(ln.a + off_a);
-            rx[s] = V::load(ln.x + off_x);
-            if (REV) rh[s] = V::load(ln.h + (h_ok[s] ? (int64_t)(t - 1) * C : 0));
-        } else {
-            ra[s] = V::load_cached(ln.a + off_a);
-            rx[s] = V::load_cached(ln.x + off_x);
-        }
-    }
-
-    CT g[S][VEC], v[S][VEC];
+    ClSteps<ST, VEC, S, REV, APPLY, CT> steps;
     CT A[VEC], B[VEC];
-#pragma unroll
-    for (int k = 0; k < VEC; k++) {
-        A[k] = CT(1);
-        B[k] = CT(0);
-    }
-#pragma unroll
-    for (int s = 0; s < S; s++) {
-        CT fa[VEC], fx[VEC];
-        V::unpack(ra[s], fa);
-        V::unpack(rx[s], fx);
-#pragma unroll
-        for (int k = 0; k < VEC; k++) {
-            g[s][k] = ok[s] ? (a_ok[s] ? fa[k] : CT(0)) : CT(1);
-            v[s][k] = ok[s] ? fx[k] : CT(0);
-            B[k] = fma_(g[s][k], B[k], v[s][k]);
-            A[k] = A[k] * g[s][k];
-        }
-    }
+    steps.load_fold(ln, T, C, tile0 + wave * S, limit, A, B);
 
     CT mine[VEC];
 #pragma unroll
@@ -140,31 +182,7 @@ __device__ __forceinline__ void cl_tile(const ClLane<ST> &ln, int T, int C, int 
             if (!APPLY) runA[k] = A[k] * runA[k];
         }
     }
-    if (!APPLY) return;
-
-#pragma unroll
-    for (int s = 0; s < S; s++) {
-        const int tau = tau0 + s;
-        const int t = REV ? T - 1 - tau : tau;
-        CT out[VEC];
-#pragma unroll
-        for (int k = 0; k < VEC; k++) {
-            mine[k] = fma_(g[s][k], mine[k], v[s][k]);
-            out[k] = mine[k];
-        }
-        if (!REV) {
-            if (ok[s]) V::store(ln.y0 + (int64_t)t * C, V::pack(out));
-        } else {
-            CT fh[VEC], ga[VEC];
-            V::unpack(rh[s], fh);
-#pragma unroll
-            for (int k = 0; k < VEC; k++) ga[k] = out[k] * (h_ok[s] ? fh[k] : CT(0));
-            if (ok[s]) {
-                V::store(ln.y0 + (int64_t)t * C, V::pack(out));
-                V::store(ln.y1 + (int64_t)t * C, V::pack(ga));
-            }
-        }
-    }
+    if (APPLY) steps.apply(ln, T, C, mine);
 }
 
 template <typename ST, int VEC>
@@ -210,115 +228,263 @@ __global__ __launch_bounds__(MAXT) void scan_cl_kernel(const ClArgs p)
     }
 }
 
-// Time split over workgroups. Workspace, in 64-bit words: ticket counter of
-// row-group r (= batch element x channel group) at word r * kCounterStride,
-// word 1 raised on a timed-out wait; from word rowgroups * kCounterStride on,
-// per (row-group, segment) the segment's pair per channel: A then B, each
-// [VEC][64] published values (see Desc<CT>). Zeroed before each launch.
+// ---------------------------------------------------------------------------
+// Time split over workgroups in ONE pass: decoupled look-back with one affine
+// pair per channel. A tile is W*S time steps of the workgroup's 64*VEC channels;
+// tiles of a row-group (batch element x channel group) are taken by ticket. W
+// consecutive tiles form a super-tile. The protocol is the two-level one of
+// scan_lookback_kernel with the roles of lanes and waves exchanged, because here
+// a lane is a channel: WAVE w of the workgroup fetches tile w of the current
+// super-tile (w < j) and super-tile m-1-w into LDS, polling until all 64 lanes
+// see them; then every lane folds, for its own channels and in a fixed order,
+//   S_m     from the nearest super-tile with a published end value SI and the
+//           aggregates (SA, SB) of the super-tiles after it,
+//   carry   from S_m through the aggregates of tiles 0..j-1.
+// The last tile of a super-tile publishes (SA, SB) as soon as it holds all W
+// tile aggregates, and SI = fma(SA, S_m, SB) once S_m is known.
+//
+// Workspace, in 64-bit words: ticket counter of row-group r at word
+// r * kCounterStride, word 1 raised on a timed-out wait; then per (row-group,
+// tile) its pair, A then B, each [VEC][64] published values; then per
+// (row-group, super-tile) SA, SB, SI likewise (4 slots, one unused).
+// LDS: 7 arrays of [W][VEC][64] values (wave pairs A, B; tile aggregates A, B;
+// super-tile SI, SA, SB).
+// ---------------------------------------------------------------------------
+template <typename CT, int VEC>
+__device__ __forceinline__ bool cl_fetch(const uint64_t *src, int lane, CT (&out)[VEC])
+{
+    using D = Desc<CT>;
+    bool ready = true;
+#pragma unroll
+    for (int k = 0; k < VEC; k++) ready = D::load(src + (k * kWave + lane) * D::W, out[k]) && ready;
+    return __ballot(ready) == ~0ull;  // all 64 lanes: the decision is the same for the whole wave
+}
+
+template <typename CT, int VEC>
+__device__ __forceinline__ void cl_publish(uint64_t *dst, int lane, const CT (&val)[VEC])
+{
+    using D = Desc<CT>;
+#pragma unroll
+    for (int k = 0; k < VEC; k++) D::store(dst + (k * kWave + lane) * D::W, val[k]);
+}
+
 template <typename ST, int VEC, int S, bool REV, int MAXT>
-__global__ __launch_bounds__(MAXT) void scan_cl_split_kernel(const ClArgs p)
+__global__ __launch_bounds__(MAXT) void scan_cl_lookback_kernel(const ClArgs p)
 {
     using CT = typename ComputeOf<ST>::type;
     using D = Desc<CT>;
     extern __shared__ double lds_raw[];
     CT *lds = reinterpret_cast<CT *>(lds_raw);
     __shared__ unsigned lds_ticket;
+    __shared__ int lds_flags[2][kMaxWaves];
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
     const int W = blockDim.x / kWave;
     const int groups = (p.C + kWave * VEC - 1) / (kWave * VEC);
     const int64_t rowgroups = p.batch * groups;
-    const int64_t rg = blockIdx.x % rowgroups;  // neighbouring workgroups hit different counters
+    const int64_t rg = blockIdx.x % rowgroups;
 
-    // The ticket is the segment: whoever holds segment s knows that segments 0..s-1 are running.
     if (threadIdx.x == 0)
         lds_ticket = __hip_atomic_fetch_add(reinterpret_cast<unsigned *>(p.ws + rg * kCounterStride), 1u,
                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
-    const int seg = (int)__builtin_amdgcn_readfirstlane(lds_ticket);
+    const int tile = (int)__builtin_amdgcn_readfirstlane(lds_ticket);
     const ClLane<ST> ln = cl_lane<ST, VEC>(p, rg / groups, (int)(rg % groups), lane);
 
-    const int tile_steps = W * S;
-    const int seg0 = seg * p.seg_steps;
-    const int seg_end = (seg0 + p.seg_steps < p.T) ? seg0 + p.seg_steps : p.T;
-    const int ntiles = (seg_end - seg0 + tile_steps - 1) / tile_steps;  // <= 0 for an empty trailing segment
+    const int tpr = p.segments;              // tiles per row-group
+    const int spr = (tpr + W - 1) / W;       // super-tiles per row-group
+    const int j = tile % W, m = tile / W;
     const int plane = W * VEC * kWave;
-    constexpr int kSegWords = 2 * VEC * kWave * D::W;
-    uint64_t *segs = p.ws + rowgroups * kCounterStride + rg * (int64_t)p.segments * kSegWords;
+    CT *exA = lds, *exB = lds + plane;                         // pairs of this tile's waves
+    CT *tA = lds + 2 * plane, *tB = lds + 3 * plane;           // aggregates of tiles 0..j-1 of the super-tile
+    CT *sI = lds + 4 * plane, *sA = lds + 5 * plane, *sB = lds + 6 * plane;  // super-tiles m-1, m-2, ...
+    constexpr int kVals = VEC * kWave * D::W;  // words of one [VEC][64] array of published values
+    uint64_t *tiles = p.ws + rowgroups * kCounterStride + rg * (int64_t)tpr * 2 * kVals;
+    uint64_t *supers = p.ws + rowgroups * kCounterStride + rowgroups * (int64_t)tpr * 2 * kVals +
+                       rg * (int64_t)spr * 4 * kVals;
+#define AT(arr, w, k) arr[((w) * VEC + (k)) * kWave + lane]
 
-    // Pass 1: the segment's pair per channel.
-    CT aggA[VEC], aggB[VEC];
+    ClSteps<ST, VEC, S, REV, true, CT> steps;
+    CT A[VEC], B[VEC];
+    steps.load_fold(ln, p.T, p.C, tile * W * S + wave * S, p.T, A, B);
 #pragma unroll
     for (int k = 0; k < VEC; k++) {
-        aggA[k] = CT(1);
-        aggB[k] = CT(0);
+        AT(exA, wave, k) = A[k];
+        AT(exB, wave, k) = B[k];
     }
-    for (int it = 0; it < ntiles; it++) {
-        CT *lds_A = lds + (it & 1) * 2 * plane;
-        cl_tile<ST, VEC, S, REV, false, CT>(ln, p.T, p.C, seg0 + it * tile_steps, seg_end, wave, W, lane, lds_A,
-                                            lds_A + plane, aggA, aggB);
+    __syncthreads();
+
+    // The tile's own aggregate (every wave computes it for its lanes).
+    CT TA[VEC], TB[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; k++) {
+        TA[k] = CT(1);
+        TB[k] = CT(0);
     }
-    if (wave == 0 && seg + 1 < p.segments) {
-        uint64_t *mine = segs + (int64_t)seg * kSegWords;
+    for (int q = 0; q < W; q++) {
 #pragma unroll
         for (int k = 0; k < VEC; k++) {
-            D::store(mine + (k * kWave + lane) * D::W, aggA[k]);
-            D::store(mine + ((VEC + k) * kWave + lane) * D::W, aggB[k]);
+            TB[k] = fma_(AT(exA, q, k), TB[k], AT(exB, q, k));
+            TA[k] = AT(exA, q, k) * TA[k];
         }
     }
-
-    // Carry into the segment: the pairs of segments 0..seg-1 applied to 0 in order. Wave w
-    // fetches segment w, w + W, ... into LDS; then every lane folds them for its channels.
     CT carry[VEC];
 #pragma unroll
     for (int k = 0; k < VEC; k++) carry[k] = CT(0);
-    __syncthreads();  // pass 1 is done with both LDS buffers
-    for (int first = 0; first < seg; first += W) {
-        const int q = first + wave;
-        if (q < seg) {
-            const uint64_t *theirs = segs + (int64_t)q * kSegWords;
-            CT pa[VEC], pb[VEC];
-            bool got = false;
-            for (int spin = 0; spin < p.spin_limit && !got; spin++) {
-                bool ready = true;
+
+    if (tpr > 1) {
+        const bool closes = (j == W - 1) && (m + 1 < spr);
+        if (wave == 0 && j < W - 1 && tile + 1 < tpr) {
+            cl_publish<CT, VEC>(tiles + (int64_t)tile * 2 * kVals, lane, TA);
+            cl_publish<CT, VEC>(tiles + (int64_t)tile * 2 * kVals + kVals, lane, TB);
+        }
+        // Wave w is responsible for tile w of this super-tile (if w < j) and for super-tile m-1-w.
+        bool have_t = wave >= j;
+        const int sidx = m - 1 - wave;
+        bool have_si = sidx < 0, have_sa = sidx < 0;
+        if (sidx < 0) {  // before the row-group starts: value 0, identity aggregate
+#pragma unroll
+            for (int k = 0; k < VEC; k++) {
+                AT(sI, wave, k) = CT(0);
+                AT(sA, wave, k) = CT(1);
+                AT(sB, wave, k) = CT(0);
+            }
+        }
+        bool tiles_done = false, supers_done = false, super_published = false;
+        int first = 0;
+        for (int spin = 0; spin < p.spin_limit; spin++) {
+            CT val[VEC], val2[VEC];
+            if (!have_t) {
+                const uint64_t *d = tiles + (int64_t)(m * W + wave) * 2 * kVals;
+                const bool ra = cl_fetch<CT, VEC>(d, lane, val), rb = cl_fetch<CT, VEC>(d + kVals, lane, val2);
+                if (ra && rb) {
+                    have_t = true;
+#pragma unroll
+                    for (int k = 0; k < VEC; k++) {
+                        AT(tA, wave, k) = val[k];
+                        AT(tB, wave, k) = val2[k];
+                    }
+                }
+            }
+            if (!have_si) {
+                if (cl_fetch<CT, VEC>(supers + (int64_t)sidx * 4 * kVals + 2 * kVals, lane, val)) {
+                    have_si = true;
+#pragma unroll
+                    for (int k = 0; k < VEC; k++) AT(sI, wave, k) = val[k];
+                }
+            }
+            if (!have_sa) {
+                const uint64_t *d = supers + (int64_t)sidx * 4 * kVals;
+                const bool ra = cl_fetch<CT, VEC>(d, lane, val), rb = cl_fetch<CT, VEC>(d + kVals, lane, val2);
+                if (ra && rb) {
+                    have_sa = true;
+#pragma unroll
+                    for (int k = 0; k < VEC; k++) {
+                        AT(sA, wave, k) = val[k];
+                        AT(sB, wave, k) = val2[k];
+                    }
+                }
+            }
+            if (lane == 0) lds_flags[spin & 1][wave] = (have_t ? 1 : 0) | (have_si ? 2 : 0) | (have_sa ? 4 : 0);
+            __syncthreads();
+            // The same decision in every thread of the workgroup.
+            tiles_done = true;
+            supers_done = false;
+            bool chain_ok = true;
+            for (int w = 0; w < W; w++) {
+                const int f = lds_flags[spin & 1][w];
+                tiles_done = tiles_done && (f & 1);
+                if (!supers_done && chain_ok) {
+                    if (f & 2) {
+                        supers_done = true;
+                        first = w;
+                    } else if (!(f & 4)) {
+                        chain_ok = false;
+                    }
+                }
+            }
+            if (tiles_done && closes && !super_published) {
+                // (SA, SB): the W tile aggregates composed in order, this tile's last.
+                super_published = true;
+                if (wave == 0) {
+                    CT SA[VEC], SB[VEC];
+#pragma unroll
+                    for (int k = 0; k < VEC; k++) {
+                        SA[k] = CT(1);
+                        SB[k] = CT(0);
+                    }
+                    for (int w = 0; w < W - 1; w++) {
+#pragma unroll
+                        for (int k = 0; k < VEC; k++) {
+                            SB[k] = fma_(AT(tA, w, k), SB[k], AT(tB, w, k));
+                            SA[k] = AT(tA, w, k) * SA[k];
+                        }
+                    }
+#pragma unroll
+                    for (int k = 0; k < VEC; k++) {
+                        SB[k] = fma_(TA[k], SB[k], TB[k]);
+                        SA[k] = TA[k] * SA[k];
+                    }
+                    cl_publish<CT, VEC>(supers + (int64_t)m * 4 * kVals, lane, SA);
+                    cl_publish<CT, VEC>(supers + (int64_t)m * 4 * kVals + kVals, lane, SB);
+                }
+            }
+            if (tiles_done && supers_done) break;
+            __builtin_amdgcn_s_sleep(1);
+        }
+        // S_m, then the carry into this tile, for this lane's channels.
+#pragma unroll
+        for (int k = 0; k < VEC; k++) carry[k] = AT(sI, first, k);
+        for (int q = first - 1; q >= 0; q--) {
+#pragma unroll
+            for (int k = 0; k < VEC; k++) carry[k] = fma_(AT(sA, q, k), carry[k], AT(sB, q, k));
+        }
+        if (!(tiles_done && supers_done)) {
+            if (threadIdx.x == 0)
+                __hip_atomic_store(p.ws + kTimeoutWord, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+            for (int k = 0; k < VEC; k++) carry[k] = CT(__builtin_nanf(""));
+        }
+        CT S_m[VEC];
+#pragma unroll
+        for (int k = 0; k < VEC; k++) S_m[k] = carry[k];
+        for (int w = 0; w < j; w++) {
+#pragma unroll
+            for (int k = 0; k < VEC; k++) carry[k] = fma_(AT(tA, w, k), carry[k], AT(tB, w, k));
+        }
+        if (closes && wave == 0) {
+            // SI = fma(SA, S_m, SB) with (SA, SB) recomposed exactly as published above.
+            CT SA[VEC], SB[VEC], SI[VEC];
+#pragma unroll
+            for (int k = 0; k < VEC; k++) {
+                SA[k] = CT(1);
+                SB[k] = CT(0);
+            }
+            for (int w = 0; w < W - 1; w++) {
 #pragma unroll
                 for (int k = 0; k < VEC; k++) {
-                    ready = D::load(theirs + (k * kWave + lane) * D::W, pa[k]) && ready;
-                    ready = D::load(theirs + ((VEC + k) * kWave + lane) * D::W, pb[k]) && ready;
+                    SB[k] = fma_(AT(tA, w, k), SB[k], AT(tB, w, k));
+                    SA[k] = AT(tA, w, k) * SA[k];
                 }
-                got = __ballot(ready) == ~0ull;
-                if (!got) __builtin_amdgcn_s_sleep(1);
-            }
-            if (!got) {
-                if (lane == 0)
-                    __hip_atomic_store(p.ws + kTimeoutWord, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-                for (int k = 0; k < VEC; k++) pb[k] = CT(__builtin_nanf(""));
             }
 #pragma unroll
             for (int k = 0; k < VEC; k++) {
-                lds[(wave * VEC + k) * kWave + lane] = pa[k];
-                lds[plane + (wave * VEC + k) * kWave + lane] = pb[k];
+                SB[k] = fma_(TA[k], SB[k], TB[k]);
+                SA[k] = TA[k] * SA[k];
+                SI[k] = fma_(SA[k], S_m[k], SB[k]);
             }
+            cl_publish<CT, VEC>(supers + (int64_t)m * 4 * kVals + 2 * kVals, lane, SI);
         }
-        __syncthreads();
-        const int count = (seg - first < W) ? seg - first : W;
-        for (int w = 0; w < count; w++) {
-#pragma unroll
-            for (int k = 0; k < VEC; k++)
-                carry[k] = fma_(lds[(w * VEC + k) * kWave + lane], carry[k], lds[plane + (w * VEC + k) * kWave + lane]);
-        }
-        __syncthreads();
     }
 
-    // Pass 2: replay the segment from its carry (its data is still in the memory-side cache).
-    CT unused[VEC];
-    for (int it = 0; it < ntiles; it++) {
-        CT *lds_A = lds + (it & 1) * 2 * plane;
-        cl_tile<ST, VEC, S, REV, true, CT>(ln, p.T, p.C, seg0 + it * tile_steps, seg_end, wave, W, lane, lds_A,
-                                           lds_A + plane, unused, carry);
+    // Carry into this wave's steps: through the pairs of the waves before it.
+    for (int q = 0; q < wave; q++) {
+#pragma unroll
+        for (int k = 0; k < VEC; k++) carry[k] = fma_(AT(exA, q, k), carry[k], AT(exB, q, k));
     }
+    steps.apply(ln, p.T, p.C, carry);
+#undef AT
 }
 
 }  // namespace scanscam

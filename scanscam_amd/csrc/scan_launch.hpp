@@ -83,8 +83,8 @@ struct ClLaunch {
     int vec;
     int steps;
     int waves;
-    int segments;   // > 1: time is also split over workgroups (scan_cl_split_kernel)
-    int seg_steps;
+    int kind;       // 0: a workgroup walks all of T; 2: tiles over workgroups with a look-back chain
+    int segments;   // kind 2: tiles per row-group
     int64_t grid;
     size_t lds_bytes;
     size_t ws_bytes;
@@ -98,9 +98,9 @@ hipError_t launch_scan_cl(const ClArgs &args, const ClLaunch &l, bool rev, hipSt
 #define SCANSCAM_CL_CASE(ST, VEC, S)                                                                   \
     if (l.vec == (VEC) && l.steps == (S)) {                                                            \
         constexpr int MAXT = cl_max_threads(VEC, S);                                                   \
-        if (l.segments > 1) {                                                                          \
-            if (rev) hipLaunchKernelGGL((scan_cl_split_kernel<ST, VEC, S, true, MAXT>), grid, block, l.lds_bytes, stream, args);  \
-            else     hipLaunchKernelGGL((scan_cl_split_kernel<ST, VEC, S, false, MAXT>), grid, block, l.lds_bytes, stream, args); \
+        if (l.kind == 2) {                                                                             \
+            if (rev) hipLaunchKernelGGL((scan_cl_lookback_kernel<ST, VEC, S, true, MAXT>), grid, block, l.lds_bytes, stream, args);  \
+            else     hipLaunchKernelGGL((scan_cl_lookback_kernel<ST, VEC, S, false, MAXT>), grid, block, l.lds_bytes, stream, args); \
         } else {                                                                                       \
             if (rev) hipLaunchKernelGGL((scan_cl_kernel<ST, VEC, S, true, MAXT>), grid, block, l.lds_bytes, stream, args);  \
             else     hipLaunchKernelGGL((scan_cl_kernel<ST, VEC, S, false, MAXT>), grid, block, l.lds_bytes, stream, args); \
