@@ -151,3 +151,30 @@ def test_time_split_is_chosen_for_few_channels_and_is_reproducible(gpu):
     ga0, gb0 = hip.transposed_linear_scan_backward(x, first, y)
     ga1, gb1 = hip.transposed_linear_scan_backward(x, first, y)
     assert torch.equal(ga0, ga1) and torch.equal(gb0, gb1)
+
+
+def test_expired_wait_is_reported_and_every_wave_exits(gpu):
+    # One poll allowed: the launch must still complete; either all waits succeeded in that poll or
+    # word 1 of the workspace is raised and the poisoned outputs are NaN.
+    import ctypes
+
+    B, T, C = 1, 4096, 64
+    g = torch.Generator(device=gpu).manual_seed(29)
+    x = torch.rand((B, T, C), generator=g, device=gpu)
+    y = torch.randn((B, T, C), generator=g, device=gpu)
+    good = hip.transposed_linear_scan_forward(x, y, plan=hip.Plan(mode=hip.MODE_LOOKBACK, vec=1, unroll=4, waves=2))
+    plan = hip.Plan(mode=hip.MODE_LOOKBACK, vec=1, unroll=4, waves=2, spin_limit=1)
+    L = hip.lib()
+    n = L.scanscam_workspace_bytes_cl(B, T, C, 0, 0, ctypes.byref(plan))
+    assert n > 0
+    ws = torch.empty(n, dtype=torch.uint8, device=gpu)
+    out = torch.empty_like(x)
+    rc = L.scanscam_scan_fwd_cl(x.data_ptr(), y.data_ptr(), out.data_ptr(), B, T, C, 0, ws.data_ptr(), n,
+                                torch.cuda.current_stream().cuda_stream, ctypes.byref(plan))
+    assert rc == 0
+    torch.cuda.synchronize()
+    if int(ws.view(torch.int64)[1].item()) != 0:
+        assert bool(torch.isnan(out).any())
+    else:
+        assert torch.equal(out, good)
+    assert torch.equal(hip.transposed_linear_scan_forward(x, y, plan=hip.Plan(mode=hip.MODE_LOOKBACK, vec=1, unroll=4, waves=2)), good)
