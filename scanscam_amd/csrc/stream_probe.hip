@@ -7,6 +7,9 @@
 //                             non-temporal loads per lane per stream): 2 reads + 1 write like the
 //                             forward scan, 3 reads + 2 writes like the backward scan. What the memory
 //                             system gives that access shape when no scan is done at all.
+//   stream_probe policy [rows]   the same two shapes with every combination of the sc0 / sc1 / nt cache-policy bits on
+//                             the loads or on the stores, over 8 rotated buffer sets so that no cache level can
+//                             hold an output between launches. Shows which policy the kernels should use.
 //
 //   hipcc -O3 --offload-arch=gfx950 stream_probe.hip -o stream_probe
 #include <hip/hip_runtime.h>
@@ -59,6 +62,55 @@ __global__ __launch_bounds__(256) void stream_shape_kernel(const f4 *__restrict_
     }
 }
 
+// Cache-policy variants: the builtins only reach "nt", so the instruction is written out. POLICY 0..6 =
+// nt | sc1 nt | sc0 sc1 nt | sc0 nt | sc1 | sc0 sc1 | none.
+#define PROBE_POLICY(OP, ...)                                                          \
+    switch (POLICY) {                                                                  \
+    case 0: asm volatile(OP " nt" __VA_ARGS__); break;                                 \
+    case 1: asm volatile(OP " sc1 nt" __VA_ARGS__); break;                             \
+    case 2: asm volatile(OP " sc0 sc1 nt" __VA_ARGS__); break;                         \
+    case 3: asm volatile(OP " sc0 nt" __VA_ARGS__); break;                             \
+    case 4: asm volatile(OP " sc1" __VA_ARGS__); break;                                \
+    case 5: asm volatile(OP " sc0 sc1" __VA_ARGS__); break;                            \
+    default: asm volatile(OP __VA_ARGS__); break;                                      \
+    }
+static const char *const kPolicyName[7] = {"nt", "sc1 nt", "sc0 sc1 nt", "sc0 nt", "sc1", "sc0 sc1", "(none)"};
+
+template <int POLICY> __device__ __forceinline__ f4 policy_load(const f4 *p)
+{
+    f4 r;
+    PROBE_POLICY("global_load_dwordx4 %0, %1, off", : "=v"(r) : "v"(p) : "memory")
+    return r;
+}
+template <int POLICY> __device__ __forceinline__ void policy_store(f4 *p, f4 v)
+{
+    PROBE_POLICY("global_store_dwordx4 %0, %1, off", : : "v"(p), "v"(v) : "memory")
+}
+
+template <int READS, int WRITES, int LOAD_POLICY, int STORE_POLICY>
+__global__ __launch_bounds__(256) void stream_policy_kernel(const f4 *__restrict__ a, const f4 *__restrict__ b,
+                                                            const f4 *__restrict__ c, f4 *__restrict__ o0,
+                                                            f4 *__restrict__ o1)
+{
+    const size_t base = (size_t)blockIdx.x * 1024 + (threadIdx.x / 64) * 256 + (threadIdx.x % 64);
+    f4 va[4], vb[4], vc[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        va[u] = policy_load<LOAD_POLICY>(a + base + u * 64);
+        if (READS > 1) vb[u] = policy_load<LOAD_POLICY>(b + base + u * 64);
+        if (READS > 2) vc[u] = policy_load<LOAD_POLICY>(c + base + u * 64);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the compiler does not track loads issued from asm
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        f4 r = va[u];
+        if (READS > 1) r += vb[u];
+        if (READS > 2) r *= vc[u];
+        policy_store<STORE_POLICY>(o0 + base + u * 64, r);
+        if (WRITES > 1) policy_store<STORE_POLICY>(o1 + base + u * 64, r + 1.0f);
+    }
+}
+
 template <typename F> static float mean_ms(F launch, int reps)
 {
     hipEvent_t e0, e1;
@@ -108,10 +160,58 @@ static int run_ceiling(size_t rows)
     return hipDeviceSynchronize() == hipSuccess ? 0 : 1;
 }
 
+static f4 *g_sets[8][5];
+
+template <int READS, int WRITES, int LP, int SP> static void policy_case(size_t rows)
+{
+    int i = 0;
+    const float ms = mean_ms(
+        [&] {
+            f4 **s = g_sets[i++ % 8];
+            hipLaunchKernelGGL((stream_policy_kernel<READS, WRITES, LP, SP>), dim3((unsigned)rows), dim3(256), 0, 0,
+                               s[0], s[1], s[2], s[3], s[4]);
+        },
+        32);
+    const double bytes = (double)(READS + WRITES) * rows * 4096 * 4;
+    printf("  %dR%dW  loads %-11s stores %-11s %7.1f us  %4.1f %% of 8 TB/s\n", READS, WRITES, kPolicyName[LP],
+           kPolicyName[SP], ms * 1e3, bytes / (ms * 1e-3) / 8e12 * 100);
+}
+template <int LP, int SP> static void policy_pair(size_t rows)
+{
+    policy_case<2, 1, LP, SP>(rows);
+    policy_case<3, 2, LP, SP>(rows);
+}
+
+static int run_policy(size_t rows)
+{
+    const size_t bytes = rows * 4096 * 4;
+    for (auto &set : g_sets)
+        for (auto &p : set) {
+            CHECK(hipMalloc(&p, bytes));
+            CHECK(hipMemset(p, 0, bytes));
+        }
+    printf("cache policy, %zu x 4096 fp32, one workgroup per row, 8 rotated buffer sets:\n", rows);
+    policy_pair<0, 0>(rows);
+    policy_pair<1, 0>(rows);
+    policy_pair<2, 0>(rows);
+    policy_pair<3, 0>(rows);
+    policy_pair<4, 0>(rows);
+    policy_pair<5, 0>(rows);
+    policy_pair<6, 0>(rows);
+    policy_pair<0, 1>(rows);
+    policy_pair<0, 2>(rows);
+    policy_pair<0, 3>(rows);
+    policy_pair<0, 4>(rows);
+    policy_pair<0, 5>(rows);
+    policy_pair<0, 6>(rows);
+    return hipDeviceSynchronize() == hipSuccess ? 0 : 1;
+}
+
 int main(int argc, char **argv)
 {
     if (argc > 1 && strcmp(argv[1], "ceiling") == 0) return run_ceiling(argc > 2 ? (size_t)atol(argv[2]) : 16384);
     if (argc > 1 && strcmp(argv[1], "copy") == 0) return run_copy(argc > 2 ? (size_t)atol(argv[2]) : 1024);
-    fprintf(stderr, "usage: %s copy [MiB] | ceiling [rows]\n", argv[0]);
+    if (argc > 1 && strcmp(argv[1], "policy") == 0) return run_policy(argc > 2 ? (size_t)atol(argv[2]) : 16384);
+    fprintf(stderr, "usage: %s copy [MiB] | ceiling [rows] | policy [rows]\n", argv[0]);
     return 2;
 }
