@@ -102,7 +102,9 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
     l.mode = u.mode;
     if (l.mode == SCANSCAM_MODE_AUTO) {
         if (T <= chunk) l.mode = kModeSmall;
-        else if (nch >= 64 && rows < 2048) l.mode = kModeLookback;
+        // From 256 rows on, one 16-wave workgroup per row fills the chip as well as tiles over
+        // workgroups do and needs no carry hand-off between workgroups.
+        else if (nch >= 64 && rows < 256) l.mode = kModeLookback;
         else l.mode = kModeRow;
     }
 
@@ -123,13 +125,19 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
                 l.wpr = 1;
                 l.waves = 4;
             } else if (rows < 2048 && nch >= 16) {
-                l.unroll = 1;
+                // Few rows: as many waves per row as a workgroup holds.
+                l.unroll = nch >= 64 ? 4 : 1;
                 l.wpr = 16;
                 l.waves = 16;
-            } else {
+            } else if (nch <= 16) {
                 l.unroll = (l.vec == full && nch <= 8) ? 2 : 4;
                 l.wpr = 4;
                 l.waves = 4;
+            } else {
+                // Longer rows: a workgroup tile (waves x chunks per wave) that covers the row in one
+                // step, or in as few as possible -- each further step waits for the carry of the last.
+                l.unroll = 4;
+                l.wpr = l.waves = nch <= 48 ? 8 : 16;
             }
         } else {
             if (!l.unroll) l.unroll = 4;

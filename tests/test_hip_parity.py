@@ -297,6 +297,34 @@ def test_short_rows_automatic(gpu, rows, T):
     assert rel_err(to_np(got_ga), ga, prev_abs(h)) <= FP32_BAR
 
 
+# One shape per branch of the automatic plan for rows longer than a chunk: (rows, T) -> the
+# (mode, waves per row, chunks per wave) the library reports for it.
+AUTO_REGIMES = [
+    (2048, 1280, (hip.MODE_ROW, 4, 2)),
+    (2048, 4100, (hip.MODE_ROW, 8, 4)),       # 17 chunks: one step of an 8-wave tile
+    (2048, 12501, (hip.MODE_ROW, 16, 4)),     # 49 chunks, element-aligned rows
+    (300, 4100, (hip.MODE_ROW, 16, 1)),
+    (300, 16640, (hip.MODE_ROW, 16, 4)),      # few rows, 65 chunks
+    (255, 16640, (hip.MODE_LOOKBACK, 0, 4)),
+]
+
+
+@pytest.mark.parametrize("rows,T,expect", AUTO_REGIMES)
+def test_automatic_plan_regimes(gpu, rows, T, expect):
+    plan = hip.resolve_plan(rows, T, torch.float32, hip.FORWARD)
+    assert (plan.mode, plan.waves_per_row, plan.unroll) == expect, plan
+    g = seeded(rows + T)
+    a = torch.rand((rows, T), generator=g)
+    b = torch.randn((rows, T), generator=g)
+    gh = torch.randn((rows, T), generator=g)
+    h = oracle.fwd(a.numpy(), b.numpy())
+    assert rel_err(to_np(run_fwd(gpu, a, b)), h) <= FP32_BAR
+    ga, gb = oracle.bwd(a.numpy(), h, gh.numpy())
+    got_ga, got_gb = run_bwd(gpu, a, torch.from_numpy(h), gh)
+    assert rel_err(to_np(got_gb), gb) <= FP32_BAR
+    assert rel_err(to_np(got_ga), ga, prev_abs(h)) <= FP32_BAR
+
+
 def test_unaligned_base_pointers(gpu):
     # Views that start 4 bytes into an allocation: the library must fall back to
     # element-wise loads, not fault or misread.
