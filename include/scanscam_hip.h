@@ -140,6 +140,47 @@ size_t scanscam_workspace_bytes_cl(int64_t batch, int64_t T, int64_t C, int dtyp
                                    const scanscam_plan *plan);
 
 /*
+ * Strided tensors, so that views need no copy first. The reference's wrappers
+ * call .contiguous() on every argument (scanscam/cuda.py:36-37, 60-62), which
+ * costs a full extra read and write of each tensor that is a view: a half of a
+ * fused projection (chunk along channels), a slice of a longer buffer, a gate
+ * broadcast over the batch. These calls replace that copy + kernel pair.
+ *
+ * Strides are in elements and must be >= 0; 0 is allowed for inputs (a
+ * broadcast). Outputs must not overlap themselves or any input.
+ *
+ * Row layout: the tensors are logical [n0, n1, T] arrays, unit-stride along T;
+ * element (r0, r1, t) of a tensor with strides s is at s.outer*r0 + s.row*r1 + t.
+ * Channels-last: logical [batch, T, C], unit-stride along C; element (b, t, c)
+ * is at s.outer*b + s.row*t + c, with s.row < 2^31.
+ * A NULL strides pointer means dense. Workspace: scanscam_workspace_bytes(n0*n1,
+ * T, ...) and scanscam_workspace_bytes_cl(batch, T, C, ...).
+ */
+typedef struct scanscam_strides {
+    int64_t outer;
+    int64_t row;
+} scanscam_strides;
+
+int scanscam_scan_fwd_strided(const void *a, const void *b, void *h, const scanscam_strides *sa,
+                              const scanscam_strides *sb, const scanscam_strides *sh, int64_t n0, int64_t n1,
+                              int64_t T, int dtype, void *workspace, size_t workspace_bytes, void *stream,
+                              const scanscam_plan *plan);
+int scanscam_scan_bwd_strided(const void *a, const void *h, const void *gh, void *ga, void *gb,
+                              const scanscam_strides *sa, const scanscam_strides *sh, const scanscam_strides *sgh,
+                              const scanscam_strides *sga, const scanscam_strides *sgb, int64_t n0, int64_t n1,
+                              int64_t T, int dtype, void *workspace, size_t workspace_bytes, void *stream,
+                              const scanscam_plan *plan);
+int scanscam_scan_fwd_cl_strided(const void *a, const void *b, void *h, const scanscam_strides *sa,
+                                 const scanscam_strides *sb, const scanscam_strides *sh, int64_t batch, int64_t T,
+                                 int64_t C, int dtype, void *workspace, size_t workspace_bytes, void *stream,
+                                 const scanscam_plan *plan);
+int scanscam_scan_bwd_cl_strided(const void *a, const void *h, const void *gh, void *ga, void *gb,
+                                 const scanscam_strides *sa, const scanscam_strides *sh,
+                                 const scanscam_strides *sgh, const scanscam_strides *sga,
+                                 const scanscam_strides *sgb, int64_t batch, int64_t T, int64_t C, int dtype,
+                                 void *workspace, size_t workspace_bytes, void *stream, const scanscam_plan *plan);
+
+/*
  * Writes the plan the automatic choice resolves to for this shape (assuming
  * 16-byte aligned pointers) into *out. Returns 0 or an error code.
  */

@@ -79,7 +79,7 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
     if (user) u = *user;
 
     Launch &l = out->l;
-    l = Launch{0, 0, 0, 0, 1, 64, 0, false};
+    l = Launch{0, 0, 0, 0, 1, 64, 0, false, 1};
     // The full 16-byte vector needs rows that start on 16-byte borders -- or, for rows longer than one
     // chunk, the element-aligned ("ragged") variants of the ROW and LOOKBACK kernels.
     const bool vec_aligned = aligned16 && (T % full == 0);
@@ -185,20 +185,67 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
 
 bool aligned_to(const void *p, size_t n) { return (reinterpret_cast<uintptr_t>(p) % n) == 0; }
 
-int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y1, int64_t rows, int64_t T,
-        int dtype, void *workspace, size_t workspace_bytes, void *stream, const scanscam_plan *plan)
+const scanscam_strides *const kDense[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
+
+// Tensor order everywhere below: a, x, h, y0, y1 (x = b forwards, gh backwards; y0 = h forwards,
+// gb backwards; h and y1 = ga exist only backwards). st[k] == nullptr means dense.
+int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y1,
+        const scanscam_strides *const st[5], int64_t n0, int64_t n1, int64_t T, int dtype, void *workspace,
+        size_t workspace_bytes, void *stream, const scanscam_plan *plan)
 {
     const int esize = elem_size(dtype);
     if (esize == 0) return SCANSCAM_EDTYPE;
-    if (rows < 0 || T < 0 || T >= kMaxT) return SCANSCAM_EINVAL;
-    if (rows == 0 || T == 0) return SCANSCAM_OK;
+    if (n0 < 0 || n1 < 0 || T < 0 || T >= kMaxT) return SCANSCAM_EINVAL;
+    if (n0 == 0 || n1 == 0 || T == 0) return SCANSCAM_OK;
+    if (n1 > INT64_MAX / n0) return SCANSCAM_EINVAL;
+    const int64_t rows = n0 * n1;
     if (!a || !x || !y0 || (rev && (!h || !y1))) return SCANSCAM_EINVAL;
 
-    const void *ptrs[5] = {a, x, y0, rev ? h : a, rev ? y1 : y0};
+    const void *ptrs[5] = {a, x, rev ? h : a, y0, rev ? y1 : y0};
+    const bool used[5] = {true, true, rev, true, rev};
+    int64_t s0[5], s1[5];
+    for (int k = 0; k < 5; k++) {
+        const scanscam_strides *t = used[k] ? st[k] : nullptr;
+        s0[k] = t ? t->outer : n1 * T;
+        s1[k] = t ? t->row : T;
+        if (s0[k] < 0 || s1[k] < 0) return SCANSCAM_EINVAL;
+    }
+    // Rows are independent, so the two levels may be merged or exchanged freely as long as every
+    // tensor is walked the same way: one level when the groups follow each other at the row stride,
+    // otherwise the longer level inside (the kernels spread the inner level over blockIdx.x).
+    if (n1 == 1) {
+        n1 = n0;
+        n0 = 1;
+        for (int k = 0; k < 5; k++) s1[k] = s0[k];
+    }
+    bool one_level = true;
+    for (int k = 0; k < 5; k++) one_level = one_level && (!used[k] || s0[k] == n1 * s1[k]);
+    if (n0 > 1 && one_level) {
+        n1 = rows;
+        n0 = 1;
+    }
+    if (n0 > n1) {
+        for (int k = 0; k < 5; k++) {
+            const int64_t t = s0[k];
+            s0[k] = s1[k];
+            s1[k] = t;
+        }
+        const int64_t t = n0;
+        n0 = n1;
+        n1 = t;
+    }
+    for (int k = 0; k < 5; k++) {
+        if (n0 == 1) s0[k] = 0;
+        if (n1 == 1) s1[k] = 0;
+    }
+
+    // 16-byte vectors need every row of every tensor to start on a 16-byte border.
+    const int full = 16 / esize;
     bool aligned16 = true;
-    for (const void *p : ptrs) {
-        if (!aligned_to(p, (size_t)esize)) return SCANSCAM_EALIGN;
-        aligned16 = aligned16 && aligned_to(p, 16);
+    for (int k = 0; k < 5; k++) {
+        if (!used[k]) continue;
+        if (!aligned_to(ptrs[k], (size_t)esize)) return SCANSCAM_EALIGN;
+        aligned16 = aligned16 && aligned_to(ptrs[k], 16) && s0[k] % full == 0 && s1[k] % full == 0;
     }
 
     Resolved r;
@@ -211,7 +258,12 @@ int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y
     args.h = h;
     args.y0 = y0;
     args.y1 = y1;
+    for (int k = 0; k < 5; k++) {
+        args.s0[k] = s0[k];
+        args.s1[k] = s1[k];
+    }
     args.rows = rows;
+    args.n1 = n1;
     args.T = (int32_t)T;
     args.nch = r.nch;
     args.wpr = r.l.wpr;
@@ -224,6 +276,16 @@ int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y
     args.ws = nullptr;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
+    auto launch = [&](const ScanArgs &la, const Launch &l) {
+        switch (dtype) {
+        case SCANSCAM_F32: return scanscam::launch_scan<float>(la, l, rev, s);
+        case SCANSCAM_BF16: return scanscam::launch_scan<__bf16>(la, l, rev, s);
+        case SCANSCAM_F16: return scanscam::launch_scan<_Float16>(la, l, rev, s);
+        case SCANSCAM_F64: return scanscam::launch_scan<double>(la, l, rev, s);
+        default: return hipErrorInvalidValue;
+        }
+    };
+
     if (r.l.mode == kModeLookback) {
         if (!workspace || workspace_bytes < r.ws_bytes) return SCANSCAM_EWORKSPACE;
         if (!aligned_to(workspace, 8)) return SCANSCAM_EALIGN;
@@ -232,40 +294,43 @@ int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y
         hipLaunchKernelGGL(scan_ws_clear_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0,
                            s, args.ws, words);
         if (hipGetLastError() != hipSuccess) return SCANSCAM_ELAUNCH;
+        // One launch over all rows; the kernel splits a row index into (group, row). Its grid is far
+        // below every launch limit by construction.
+        return launch(args, r.l) == hipSuccess ? SCANSCAM_OK : SCANSCAM_ELAUNCH;
     }
 
-    // One launch may hold at most 2^32 - 1 threads. Rows are independent, so a ROW or SMALL launch
-    // that would exceed it is issued as several launches over consecutive slabs of rows (only
-    // tensors of tens of GB get there). LOOKBACK grids are far below the limit by construction.
+    // ROW and SMALL: blockIdx.x walks the n1 rows of a group, blockIdx.y the n0 groups. One launch
+    // may hold at most 2^32 - 1 threads and 65535 groups; rows are independent, so a larger problem
+    // is issued as several launches over consecutive slabs (only tensors of tens of GB get there).
     const int64_t threads = (int64_t)r.l.waves * kWave;
     const int64_t max_grid = ((int64_t(1) << 32) - 1) / threads;
     int64_t rows_per_wg = 1;
     if (r.l.mode == kModeRow) rows_per_wg = r.l.waves / r.l.wpr;
     if (r.l.mode == kModeSmall) rows_per_wg = (int64_t)r.l.waves * r.l.unroll * (kWave / r.l.group);
-    const int64_t slab_rows = (r.l.mode == kModeLookback || r.l.grid <= max_grid) ? rows : max_grid * rows_per_wg;
+    const int64_t grid_x_all = (n1 + rows_per_wg - 1) / rows_per_wg;
+    const int64_t slab_rows = grid_x_all <= max_grid ? n1 : max_grid * rows_per_wg;
 
-    for (int64_t row0 = 0; row0 < rows; row0 += slab_rows) {
-        const int64_t n = rows - row0 < slab_rows ? rows - row0 : slab_rows;
-        const int64_t byte_off = row0 * T * esize;
-        ScanArgs slab = args;
-        Launch l = r.l;
-        if (slab_rows != rows) {
-            slab.a = static_cast<const char *>(a) + byte_off;
-            slab.x = static_cast<const char *>(x) + byte_off;
-            slab.h = h ? static_cast<const char *>(h) + byte_off : nullptr;
-            slab.y0 = static_cast<char *>(y0) + byte_off;
-            slab.y1 = y1 ? static_cast<char *>(y1) + byte_off : nullptr;
+    for (int64_t row0 = 0; row0 < n1; row0 += slab_rows) {
+        const int64_t n = n1 - row0 < slab_rows ? n1 - row0 : slab_rows;
+        const int64_t grid_x = (n + rows_per_wg - 1) / rows_per_wg;
+        int64_t slab_groups = max_grid / grid_x;
+        if (slab_groups > 65535) slab_groups = 65535;
+        if (slab_groups < 1) slab_groups = 1;
+        for (int64_t g0 = 0; g0 < n0; g0 += slab_groups) {
+            ScanArgs slab = args;
+            Launch l = r.l;
+            const void **in[3] = {&slab.a, &slab.x, &slab.h};
+            void **out[2] = {&slab.y0, &slab.y1};
+            for (int k = 0; k < 5; k++) {
+                const int64_t byte_off = (g0 * s0[k] + row0 * s1[k]) * esize;
+                if (k < 3 && *in[k]) *in[k] = static_cast<const char *>(*in[k]) + byte_off;
+                if (k >= 3 && *out[k - 3]) *out[k - 3] = static_cast<char *>(*out[k - 3]) + byte_off;
+            }
             slab.rows = n;
-            l.grid = (n + rows_per_wg - 1) / rows_per_wg;
+            l.grid = grid_x;
+            l.grid_y = (int)(n0 - g0 < slab_groups ? n0 - g0 : slab_groups);
+            if (launch(slab, l) != hipSuccess) return SCANSCAM_ELAUNCH;
         }
-        hipError_t e = hipErrorInvalidValue;
-        switch (dtype) {
-        case SCANSCAM_F32: e = scanscam::launch_scan<float>(slab, l, rev, s); break;
-        case SCANSCAM_BF16: e = scanscam::launch_scan<__bf16>(slab, l, rev, s); break;
-        case SCANSCAM_F16: e = scanscam::launch_scan<_Float16>(slab, l, rev, s); break;
-        case SCANSCAM_F64: e = scanscam::launch_scan<double>(slab, l, rev, s); break;
-        }
-        if (e != hipSuccess) return SCANSCAM_ELAUNCH;
     }
     return SCANSCAM_OK;
 }
@@ -346,8 +411,9 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     return SCANSCAM_OK;
 }
 
-int run_cl(bool rev, const void *a, const void *x, const void *h, void *y0, void *y1, int64_t batch, int64_t T,
-           int64_t C, int dtype, void *workspace, size_t workspace_bytes, void *stream, const scanscam_plan *plan)
+int run_cl(bool rev, const void *a, const void *x, const void *h, void *y0, void *y1,
+           const scanscam_strides *const st[5], int64_t batch, int64_t T, int64_t C, int dtype, void *workspace,
+           size_t workspace_bytes, void *stream, const scanscam_plan *plan)
 {
     const int esize = elem_size(dtype);
     if (esize == 0) return SCANSCAM_EDTYPE;
@@ -355,11 +421,19 @@ int run_cl(bool rev, const void *a, const void *x, const void *h, void *y0, void
     if (batch == 0 || T == 0 || C == 0) return SCANSCAM_OK;
     if (!a || !x || !y0 || (rev && (!h || !y1))) return SCANSCAM_EINVAL;
 
-    const void *ptrs[5] = {a, x, y0, rev ? h : a, rev ? y1 : y0};
+    // Tensor order a, x, h, y0, y1; the forward pass has no h and no y1 (they alias a and y0).
+    const void *ptrs[5] = {a, x, rev ? h : a, y0, rev ? y1 : y0};
+    const int src[5] = {0, 1, rev ? 2 : 0, 3, rev ? 4 : 3};
+    const int full = 16 / esize;
+    int64_t sB[5], sT[5];
     bool aligned16 = true;
-    for (const void *p : ptrs) {
-        if (!aligned_to(p, (size_t)esize)) return SCANSCAM_EALIGN;
-        aligned16 = aligned16 && aligned_to(p, 16);
+    for (int k = 0; k < 5; k++) {
+        const scanscam_strides *t = st[src[k]];
+        sB[k] = batch == 1 ? 0 : (t ? t->outer : T * C);
+        sT[k] = T == 1 ? 0 : (t ? t->row : C);
+        if (sB[k] < 0 || sT[k] < 0 || sT[k] >= kMaxT) return SCANSCAM_EINVAL;
+        if (!aligned_to(ptrs[k], (size_t)esize)) return SCANSCAM_EALIGN;
+        aligned16 = aligned16 && aligned_to(ptrs[k], 16) && sB[k] % full == 0 && sT[k] % full == 0;
     }
     scanscam::ClLaunch l;
     const int rc = resolve_cl(plan, batch, T, C, dtype, aligned16, &l);
@@ -371,6 +445,10 @@ int run_cl(bool rev, const void *a, const void *x, const void *h, void *y0, void
     args.h = rev ? h : a;  // never read in the forward pass
     args.y0 = y0;
     args.y1 = rev ? y1 : y0;
+    for (int k = 0; k < 5; k++) {
+        args.sB[k] = sB[k];
+        args.sT[k] = (int32_t)sT[k];
+    }
     args.batch = batch;
     args.T = (int32_t)T;
     args.C = (int32_t)C;
@@ -417,13 +495,13 @@ extern "C" {
 int scanscam_scan_fwd(const void *a, const void *b, void *h, int64_t rows, int64_t T, int dtype,
                       void *workspace, size_t workspace_bytes, void *stream)
 {
-    return run(false, a, b, nullptr, h, nullptr, rows, T, dtype, workspace, workspace_bytes, stream, nullptr);
+    return run(false, a, b, nullptr, h, nullptr, kDense, 1, rows, T, dtype, workspace, workspace_bytes, stream, nullptr);
 }
 
 int scanscam_scan_bwd(const void *a, const void *h, const void *gh, void *ga, void *gb, int64_t rows,
                       int64_t T, int dtype, void *workspace, size_t workspace_bytes, void *stream)
 {
-    return run(true, a, gh, h, gb, ga, rows, T, dtype, workspace, workspace_bytes, stream, nullptr);
+    return run(true, a, gh, h, gb, ga, kDense, 1, rows, T, dtype, workspace, workspace_bytes, stream, nullptr);
 }
 
 size_t scanscam_workspace_bytes(int64_t rows, int64_t T, int dtype, int direction)
@@ -435,14 +513,14 @@ size_t scanscam_workspace_bytes(int64_t rows, int64_t T, int dtype, int directio
 int scanscam_scan_fwd_plan(const void *a, const void *b, void *h, int64_t rows, int64_t T, int dtype,
                            void *workspace, size_t workspace_bytes, void *stream, const scanscam_plan *plan)
 {
-    return run(false, a, b, nullptr, h, nullptr, rows, T, dtype, workspace, workspace_bytes, stream, plan);
+    return run(false, a, b, nullptr, h, nullptr, kDense, 1, rows, T, dtype, workspace, workspace_bytes, stream, plan);
 }
 
 int scanscam_scan_bwd_plan(const void *a, const void *h, const void *gh, void *ga, void *gb, int64_t rows,
                            int64_t T, int dtype, void *workspace, size_t workspace_bytes, void *stream,
                            const scanscam_plan *plan)
 {
-    return run(true, a, gh, h, gb, ga, rows, T, dtype, workspace, workspace_bytes, stream, plan);
+    return run(true, a, gh, h, gb, ga, kDense, 1, rows, T, dtype, workspace, workspace_bytes, stream, plan);
 }
 
 size_t scanscam_workspace_bytes_plan(int64_t rows, int64_t T, int dtype, int direction,
@@ -455,14 +533,14 @@ size_t scanscam_workspace_bytes_plan(int64_t rows, int64_t T, int dtype, int dir
 int scanscam_scan_fwd_cl(const void *a, const void *b, void *h, int64_t batch, int64_t T, int64_t C, int dtype,
                          void *workspace, size_t workspace_bytes, void *stream, const scanscam_plan *plan)
 {
-    return run_cl(false, a, b, nullptr, h, nullptr, batch, T, C, dtype, workspace, workspace_bytes, stream, plan);
+    return run_cl(false, a, b, nullptr, h, nullptr, kDense, batch, T, C, dtype, workspace, workspace_bytes, stream, plan);
 }
 
 int scanscam_scan_bwd_cl(const void *a, const void *h, const void *gh, void *ga, void *gb, int64_t batch,
                          int64_t T, int64_t C, int dtype, void *workspace, size_t workspace_bytes, void *stream,
                          const scanscam_plan *plan)
 {
-    return run_cl(true, a, gh, h, gb, ga, batch, T, C, dtype, workspace, workspace_bytes, stream, plan);
+    return run_cl(true, a, gh, h, gb, ga, kDense, batch, T, C, dtype, workspace, workspace_bytes, stream, plan);
 }
 
 size_t scanscam_workspace_bytes_cl(int64_t batch, int64_t T, int64_t C, int dtype, int direction,
@@ -476,6 +554,44 @@ size_t scanscam_workspace_bytes_cl(int64_t batch, int64_t T, int64_t C, int dtyp
         if (resolve_cl(plan, batch, T, C, dtype, al != 0, &l) == SCANSCAM_OK && l.ws_bytes > need) need = l.ws_bytes;
     }
     return need;
+}
+
+int scanscam_scan_fwd_strided(const void *a, const void *b, void *h, const scanscam_strides *sa,
+                              const scanscam_strides *sb, const scanscam_strides *sh, int64_t n0, int64_t n1,
+                              int64_t T, int dtype, void *workspace, size_t workspace_bytes, void *stream,
+                              const scanscam_plan *plan)
+{
+    const scanscam_strides *const st[5] = {sa, sb, nullptr, sh, nullptr};
+    return run(false, a, b, nullptr, h, nullptr, st, n0, n1, T, dtype, workspace, workspace_bytes, stream, plan);
+}
+
+int scanscam_scan_bwd_strided(const void *a, const void *h, const void *gh, void *ga, void *gb,
+                              const scanscam_strides *sa, const scanscam_strides *sh, const scanscam_strides *sgh,
+                              const scanscam_strides *sga, const scanscam_strides *sgb, int64_t n0, int64_t n1,
+                              int64_t T, int dtype, void *workspace, size_t workspace_bytes, void *stream,
+                              const scanscam_plan *plan)
+{
+    const scanscam_strides *const st[5] = {sa, sgh, sh, sgb, sga};
+    return run(true, a, gh, h, gb, ga, st, n0, n1, T, dtype, workspace, workspace_bytes, stream, plan);
+}
+
+int scanscam_scan_fwd_cl_strided(const void *a, const void *b, void *h, const scanscam_strides *sa,
+                                 const scanscam_strides *sb, const scanscam_strides *sh, int64_t batch, int64_t T,
+                                 int64_t C, int dtype, void *workspace, size_t workspace_bytes, void *stream,
+                                 const scanscam_plan *plan)
+{
+    const scanscam_strides *const st[5] = {sa, sb, nullptr, sh, nullptr};
+    return run_cl(false, a, b, nullptr, h, nullptr, st, batch, T, C, dtype, workspace, workspace_bytes, stream, plan);
+}
+
+int scanscam_scan_bwd_cl_strided(const void *a, const void *h, const void *gh, void *ga, void *gb,
+                                 const scanscam_strides *sa, const scanscam_strides *sh,
+                                 const scanscam_strides *sgh, const scanscam_strides *sga,
+                                 const scanscam_strides *sgb, int64_t batch, int64_t T, int64_t C, int dtype,
+                                 void *workspace, size_t workspace_bytes, void *stream, const scanscam_plan *plan)
+{
+    const scanscam_strides *const st[5] = {sa, sgh, sh, sgb, sga};
+    return run_cl(true, a, gh, h, gb, ga, st, batch, T, C, dtype, workspace, workspace_bytes, stream, plan);
 }
 
 int scanscam_resolve_plan(int64_t rows, int64_t T, int dtype, int direction, const scanscam_plan *plan,

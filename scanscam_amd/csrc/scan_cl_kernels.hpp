@@ -34,6 +34,8 @@ struct ClArgs {
     const void *h;  // forward: unused backward: saved forward output
     void *y0;       // forward: h      backward: gb
     void *y1;       // forward: unused backward: ga
+    int64_t sB[5];  // element stride from batch element to batch element, per tensor in the order above
+    int32_t sT[5];  // element stride from time step to time step (C when dense)
     int64_t batch;
     int32_t T;
     int32_t C;
@@ -47,6 +49,7 @@ struct ClArgs {
 template <typename ST> struct ClLane {
     const ST *a, *x, *h;
     ST *y0, *y1;
+    int pa, px, ph, py0, py1;  // elements from one time step to the next, per tensor
     bool c_ok;
 };
 
@@ -65,7 +68,7 @@ struct ClSteps {
     bool ok[S], h_ok[S];
     int tau0;  // scan position of the first step
 
-    __device__ __forceinline__ void load_fold(const ClLane<ST> &ln, int T, int C, int first_step, int limit,
+    __device__ __forceinline__ void load_fold(const ClLane<ST> &ln, int T, int first_step, int limit,
                                               CT (&A)[VEC], CT (&B)[VEC])
     {
         tau0 = first_step;
@@ -82,12 +85,12 @@ struct ClSteps {
             // The gate of step t is a[t] forwards and a[t+1] backwards (0 past the end); h[-1] = 0.
             a_ok[s] = ok[s] && (!REV || t + 1 < T);
             h_ok[s] = ok[s] && t > 0;
-            const int64_t off_x = ok[s] ? (int64_t)t * C : 0;
-            const int64_t off_a = a_ok[s] ? (int64_t)(REV ? t + 1 : t) * C : 0;
+            const int64_t off_x = ok[s] ? (int64_t)t * ln.px : 0;
+            const int64_t off_a = a_ok[s] ? (int64_t)(REV ? t + 1 : t) * ln.pa : 0;
             if (APPLY) {
                 ra[s] = V::load(ln.a + off_a);
                 rx[s] = V::load(ln.x + off_x);
-                if (REV) rh[s] = V::load(ln.h + (h_ok[s] ? (int64_t)(t - 1) * C : 0));
+                if (REV) rh[s] = V::load(ln.h + (h_ok[s] ? (int64_t)(t - 1) * ln.ph : 0));
             } else {
                 ra[s] = V::load_cached(ln.a + off_a);
                 rx[s] = V::load_cached(ln.x + off_x);
@@ -113,7 +116,7 @@ struct ClSteps {
         }
     }
 
-    __device__ __forceinline__ void apply(const ClLane<ST> &ln, int T, int C, CT (&mine)[VEC])
+    __device__ __forceinline__ void apply(const ClLane<ST> &ln, int T, CT (&mine)[VEC])
     {
 #pragma unroll
         for (int s = 0; s < S; s++) {
@@ -126,15 +129,15 @@ struct ClSteps {
                 out[k] = mine[k];
             }
             if (!REV) {
-                if (ok[s]) V::store(ln.y0 + (int64_t)t * C, V::pack(out));
+                if (ok[s]) V::store(ln.y0 + (int64_t)t * ln.py0, V::pack(out));
             } else {
                 CT fh[VEC], ga[VEC];
                 V::unpack(rh[s], fh);
 #pragma unroll
                 for (int k = 0; k < VEC; k++) ga[k] = out[k] * (h_ok[s] ? fh[k] : CT(0));
                 if (ok[s]) {
-                    V::store(ln.y0 + (int64_t)t * C, V::pack(out));
-                    V::store(ln.y1 + (int64_t)t * C, V::pack(ga));
+                    V::store(ln.y0 + (int64_t)t * ln.py0, V::pack(out));
+                    V::store(ln.y1 + (int64_t)t * ln.py1, V::pack(ga));
                 }
             }
         }
@@ -149,12 +152,12 @@ struct ClSteps {
 //                  (kept for callers that only need a pair; unused by the kernels here).
 // lds_A / lds_B: [W][VEC][64] values each; the caller alternates two buffers.
 template <typename ST, int VEC, int S, bool REV, bool APPLY, typename CT>
-__device__ __forceinline__ void cl_tile(const ClLane<ST> &ln, int T, int C, int tile0, int limit, int wave, int W,
+__device__ __forceinline__ void cl_tile(const ClLane<ST> &ln, int T, int tile0, int limit, int wave, int W,
                                         int lane, CT *lds_A, CT *lds_B, CT (&runA)[VEC], CT (&run)[VEC])
 {
     ClSteps<ST, VEC, S, REV, APPLY, CT> steps;
     CT A[VEC], B[VEC];
-    steps.load_fold(ln, T, C, tile0 + wave * S, limit, A, B);
+    steps.load_fold(ln, T, tile0 + wave * S, limit, A, B);
 
     CT mine[VEC];
 #pragma unroll
@@ -182,7 +185,7 @@ __device__ __forceinline__ void cl_tile(const ClLane<ST> &ln, int T, int C, int 
             if (!APPLY) runA[k] = A[k] * runA[k];
         }
     }
-    if (APPLY) steps.apply(ln, T, C, mine);
+    if (APPLY) steps.apply(ln, T, mine);
 }
 
 template <typename ST, int VEC>
@@ -191,12 +194,17 @@ __device__ __forceinline__ ClLane<ST> cl_lane(const ClArgs &p, int64_t batch_ind
     const int64_t c0 = ((int64_t)group * kWave + lane) * VEC;  // first channel of this lane
     ClLane<ST> ln;
     ln.c_ok = c0 < p.C;
-    const int64_t base = batch_index * p.T * p.C + (ln.c_ok ? c0 : 0);
-    ln.a = static_cast<const ST *>(p.a) + base;
-    ln.x = static_cast<const ST *>(p.x) + base;
-    ln.h = static_cast<const ST *>(p.h) + base;
-    ln.y0 = static_cast<ST *>(p.y0) + base;
-    ln.y1 = static_cast<ST *>(p.y1) + base;
+    const int64_t c = ln.c_ok ? c0 : 0;
+    ln.a = static_cast<const ST *>(p.a) + batch_index * p.sB[0] + c;
+    ln.x = static_cast<const ST *>(p.x) + batch_index * p.sB[1] + c;
+    ln.h = static_cast<const ST *>(p.h) + batch_index * p.sB[2] + c;
+    ln.y0 = static_cast<ST *>(p.y0) + batch_index * p.sB[3] + c;
+    ln.y1 = static_cast<ST *>(p.y1) + batch_index * p.sB[4] + c;
+    ln.pa = p.sT[0];
+    ln.px = p.sT[1];
+    ln.ph = p.sT[2];
+    ln.py0 = p.sT[3];
+    ln.py1 = p.sT[4];
     return ln;
 }
 
@@ -223,7 +231,7 @@ __global__ __launch_bounds__(MAXT) void scan_cl_kernel(const ClArgs p)
 
     for (int it = 0; it < ntiles; it++) {
         CT *lds_A = lds + (it & 1) * 2 * plane;
-        cl_tile<ST, VEC, S, REV, true, CT>(ln, p.T, p.C, it * tile_steps, p.T, wave, W, lane, lds_A, lds_A + plane,
+        cl_tile<ST, VEC, S, REV, true, CT>(ln, p.T, it * tile_steps, p.T, wave, W, lane, lds_A, lds_A + plane,
                                            unused, carry);
     }
 }
@@ -307,7 +315,7 @@ __global__ __launch_bounds__(MAXT) void scan_cl_lookback_kernel(const ClArgs p)
 
     ClSteps<ST, VEC, S, REV, true, CT> steps;
     CT A[VEC], B[VEC];
-    steps.load_fold(ln, p.T, p.C, tile * W * S + wave * S, p.T, A, B);
+    steps.load_fold(ln, p.T, tile * W * S + wave * S, p.T, A, B);
 #pragma unroll
     for (int k = 0; k < VEC; k++) {
         AT(exA, wave, k) = A[k];
@@ -483,7 +491,7 @@ __global__ __launch_bounds__(MAXT) void scan_cl_lookback_kernel(const ClArgs p)
 #pragma unroll
         for (int k = 0; k < VEC; k++) carry[k] = fma_(AT(exA, q, k), carry[k], AT(exB, q, k));
     }
-    steps.apply(ln, p.T, p.C, carry);
+    steps.apply(ln, p.T, carry);
 #undef AT
 }
 

@@ -50,13 +50,21 @@ constexpr int kMaxWaves = 16;
 // ---------------------------------------------------------------------------
 // Kernel arguments (plain pointers; the host fills them per launch).
 // ---------------------------------------------------------------------------
+//
+// Rows form a two-level grid of n0 groups of n1 rows. Row r1 of group r0 of tensor k starts at
+// element r0 * s0[k] + r1 * s1[k]; time is unit-stride. A contiguous [rows, T] tensor is one group
+// with s1 = T. The ROW and SMALL kernels take the group from blockIdx.y and `rows` = n1; the
+// LOOKBACK kernel takes `rows` = n0 * n1 and divides.
 struct ScanArgs {
     const void *a;   // gates                       [rows, T]
     const void *x;   // forward: b      backward: gh
     const void *h;   // forward: unused backward: saved forward output
     void *y0;        // forward: h      backward: gb (value grad)
     void *y1;        // forward: unused backward: ga (gate grad)
+    int64_t s0[5];   // element stride from group to group, per tensor in the order above
+    int64_t s1[5];   // element stride from row to row
     int64_t rows;
+    int64_t n1;      // LOOKBACK: rows per group
     int32_t T;
     int32_t nch;            // chunks per row = ceil(T / (64*VEC))
     int32_t wpr;            // ROW: waves cooperating on one row
@@ -257,11 +265,29 @@ struct WaveTile {
     using raw_t = typename V::raw_t;
     using CT = typename ComputeOf<ST>::type;
 
-    // Where this lane's vector of chunk u lives.
-    int64_t off[U];  // element offset of the vector from the tensor base
-    int32_t m[U];    // vector index inside the row (element m*VEC)
+    // Where this lane's vector of chunk u lives. Lanes without a vector point at element 0 of an
+    // existing row (col = 0), which is always readable.
+    int32_t col[U];  // first element of the vector inside its row (m*VEC)
+    int32_t m[U];    // vector index inside the row
     bool valid[U];   // inside the row (and the row exists)
     int32_t count[RAGGED ? U : 1];  // RAGGED: elements of the vector inside the row (1..VEC)
+    // Start of the row in tensor k = 0..4 (a, x, h, y0, y1), in elements. The ROW and LOOKBACK kernels
+    // have one row per wave (wave-uniform); in the SMALL kernel `base` is the start of the group and
+    // the row of chunk u, which differs from lane to lane, is added per access.
+    int64_t base[5];
+    int64_t rowi[GROUPED ? U : 1];
+
+    __device__ __forceinline__ void set_row(const ScanArgs &p, int64_t group, int64_t row)
+    {
+#pragma unroll
+        for (int k = 0; k < 5; k++) base[k] = group * p.s0[k] + row * p.s1[k];
+    }
+    template <int K> __device__ __forceinline__ int64_t at(const ScanArgs &p, int u) const
+    {
+        int64_t o = base[K] + col[u];
+        if (GROUPED) o += rowi[u] * p.s1[K];
+        return o;
+    }
 
     __device__ __forceinline__ raw_t fetch(const ST *p, int u) const
     {
@@ -294,21 +320,20 @@ struct WaveTile {
 #pragma unroll
         for (int u = 0; u < U; u++) {
             if (!RAGGED) {
-                // Unconditional: lanes outside the row read element 0 of the tensor instead and are
+                // Unconditional: lanes outside the row read element 0 of a row instead and are
                 // masked in reduce(). No branch separates the loads, so all of the wave's U x streams
                 // loads are in flight before the first one is waited for.
-                const int64_t o = valid[u] ? off[u] : 0;
-                ra[u] = V::load(a + o);
-                rx[u] = V::load(x + o);
-                if (REV) rh[u] = V::load(h + o);
+                ra[u] = V::load(a + at<0>(p, u));
+                rx[u] = V::load(x + at<1>(p, u));
+                if (REV) rh[u] = V::load(h + at<2>(p, u));
             } else {
                 ra[u] = V::zero_raw();
                 rx[u] = V::zero_raw();
                 if (REV) rh[u] = V::zero_raw();
                 if (valid[u]) {
-                    ra[u] = fetch(a + off[u], u);
-                    rx[u] = fetch(x + off[u], u);
-                    if (REV) rh[u] = fetch(h + off[u], u);
+                    ra[u] = fetch(a + at<0>(p, u), u);
+                    rx[u] = fetch(x + at<1>(p, u), u);
+                    if (REV) rh[u] = fetch(h + at<2>(p, u), u);
                 }
             }
             if (REV) {
@@ -319,8 +344,8 @@ struct WaveTile {
                 // inner ones are taken from the neighbouring chunk's registers in reduce().
                 const bool need_a = !CHAIN || u == 0;
                 const bool need_h = !CHAIN || u == U - 1;
-                if (need_a && valid[u] && j == 0 && (m[u] + 1) * VEC < p.T) edge_a[u] = (CT)a[off[u] + VEC];
-                if (need_h && valid[u] && j == jlast && m[u] > 0) edge_h[u] = (CT)h[off[u] - 1];
+                if (need_a && valid[u] && j == 0 && (m[u] + 1) * VEC < p.T) edge_a[u] = (CT)a[at<0>(p, u) + VEC];
+                if (need_h && valid[u] && j == jlast && m[u] > 0) edge_h[u] = (CT)h[at<2>(p, u) - 1];
             }
         }
     }
@@ -434,7 +459,7 @@ struct WaveTile {
             if (CHAIN && u + 1 < U)
                 carry = fma_(read_lane(PA[u], 63), carry, read_lane(PB[u], 63));
             if (!REV) {
-                if (valid[u]) put(y0 + off[u], V::pack(out), u);
+                if (valid[u]) put(y0 + at<3>(p, u), V::pack(out), u);
             } else {
                 CT gb[VEC], ga[VEC];
 #pragma unroll
@@ -443,8 +468,8 @@ struct WaveTile {
                     ga[VEC - 1 - k] = out[k] * hp[u][k];
                 }
                 if (valid[u]) {
-                    put(y0 + off[u], V::pack(gb), u);
-                    put(y1 + off[u], V::pack(ga), u);
+                    put(y0 + at<3>(p, u), V::pack(gb), u);
+                    put(y1 + at<4>(p, u), V::pack(ga), u);
                 }
             }
         }
@@ -464,7 +489,7 @@ __global__ __launch_bounds__(MAXT) void scan_row_kernel(const ScanArgs p)
     __shared__ CT lds_B[2][kMaxWaves];
 
     const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x / kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // wave-uniform, kept in a scalar register
     const int nwaves = blockDim.x / kWave;
     const int wpr = p.wpr;
     const int rows_per_wg = nwaves / wpr;
@@ -474,12 +499,12 @@ __global__ __launch_bounds__(MAXT) void scan_row_kernel(const ScanArgs p)
     // rows; giving each XCD one contiguous eighth of the rows instead measured 5 % slower.
     const int64_t row = (int64_t)blockIdx.x * rows_per_wg + wave / wpr;
     const bool row_ok = row < p.rows;
-    const int64_t row_off = row_ok ? row * (int64_t)p.T : 0;
     const int nvp = p.nch * kWave;      // vectors per row, padded to whole chunks
     const int tile_chunks = wpr * U;
     const int ntiles = (p.nch + tile_chunks - 1) / tile_chunks;
 
     WaveTile<ST, VEC, U, REV, false, true, RAGGED> w;
+    w.set_row(p, blockIdx.y, row_ok ? row : 0);
     CT hp[REV ? U : 1][VEC];
     CT row_carry = CT(0);
 
@@ -491,7 +516,7 @@ __global__ __launch_bounds__(MAXT) void scan_row_kernel(const ScanArgs p)
             const int m = REV ? nvp - 1 - s : s;
             w.m[u] = m;
             w.valid[u] = row_ok && m >= 0 && (int64_t)m * VEC < p.T;
-            w.off[u] = row_off + (int64_t)m * VEC;
+            w.col[u] = w.valid[u] ? m * VEC : 0;
             if (RAGGED) w.count[u] = p.T - m * VEC;
         }
         w.load(p, lane, kWave - 1);
@@ -537,6 +562,7 @@ __global__ __launch_bounds__(MAXT) void scan_small_kernel(const ScanArgs p)
     const int64_t row0 = wave_id * (U * rows_per_chunk) + lane / G;
 
     WaveTile<ST, VEC, U, REV, true, false> w;
+    w.set_row(p, blockIdx.y, 0);
     CT hp[REV ? U : 1][VEC];
 #pragma unroll
     for (int u = 0; u < U; u++) {
@@ -544,7 +570,8 @@ __global__ __launch_bounds__(MAXT) void scan_small_kernel(const ScanArgs p)
         const int m = REV ? G - 1 - j : j;
         w.m[u] = m;
         w.valid[u] = row < p.rows && m * VEC < p.T;
-        w.off[u] = (w.valid[u] ? row * (int64_t)p.T : 0) + (int64_t)m * VEC;
+        w.rowi[u] = w.valid[u] ? row : 0;
+        w.col[u] = w.valid[u] ? m * VEC : 0;
     }
     w.load(p, j, G - 1);
     w.reduce(j, G - 1, hp);
@@ -748,11 +775,12 @@ __global__ __launch_bounds__(MAXT) void scan_lookback_kernel(const ScanArgs p)
     if ((int64_t)ticket >= rows_here * p.tiles_per_row) return;  // surplus workgroup of an uneven split
     const int64_t row = ctr + (int64_t)nctr * (ticket % (uint64_t)rows_here);
     const int tile = (int)(ticket / (uint64_t)rows_here);
-    const int64_t row_off = row * (int64_t)p.T;
     const int nvp = p.nch * kWave;
     const int chunk0 = (tile * nwaves + wave) * U;
 
     WaveTile<ST, VEC, U, REV, false, true, RAGGED> w;
+    const int64_t group = row / p.n1;
+    w.set_row(p, group, row - group * p.n1);
     CT hp[REV ? U : 1][VEC];
 #pragma unroll
     for (int u = 0; u < U; u++) {
@@ -760,7 +788,7 @@ __global__ __launch_bounds__(MAXT) void scan_lookback_kernel(const ScanArgs p)
         const int m = REV ? nvp - 1 - s : s;
         w.m[u] = m;
         w.valid[u] = m >= 0 && (int64_t)m * VEC < p.T;
-        w.off[u] = row_off + (int64_t)m * VEC;
+        w.col[u] = w.valid[u] ? m * VEC : 0;
         if (RAGGED) w.count[u] = p.T - m * VEC;
     }
     w.load(p, lane, kWave - 1);

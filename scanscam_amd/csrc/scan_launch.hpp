@@ -18,6 +18,7 @@ struct Launch {
     int group;   // SMALL: lanes per row
     int64_t grid;
     bool ragged; // ROW / LOOKBACK with the full vector on rows that start at any element
+    int grid_y;  // ROW / SMALL: groups of rows (blockIdx.y); 1 for LOOKBACK
 };
 
 // Largest workgroup (threads) a kernel with U chunks per wave is compiled for.
@@ -65,7 +66,7 @@ hipError_t launch_scan(const ScanArgs &args, const Launch &l, bool rev, hipStrea
     hipError_t launch_scan<ST>(const ScanArgs &args, const Launch &l, bool rev, hipStream_t stream)  \
     {                                                                                                \
         constexpr int FULL = 16 / (int)sizeof(ST);                                                   \
-        const dim3 grid((unsigned)l.grid), block((unsigned)(l.waves * kWave));                       \
+        const dim3 grid((unsigned)l.grid, (unsigned)l.grid_y), block((unsigned)(l.waves * kWave));   \
         SCANSCAM_RAGGED_CASE(ST, FULL, 2)                                                            \
         SCANSCAM_RAGGED_CASE(ST, FULL, 4)                                                            \
         if (l.ragged) return hipErrorInvalidValue;                                                   \

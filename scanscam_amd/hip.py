@@ -53,10 +53,30 @@ class Plan(ctypes.Structure):
         )
 
 
+class Strides(ctypes.Structure):
+    """``scanscam_strides``: element strides of the two levels above the unit-stride dimension."""
+
+    _fields_ = [("outer", ctypes.c_int64), ("row", ctypes.c_int64)]
+
+    def __repr__(self) -> str:
+        return f"Strides(outer={self.outer}, row={self.row})"
+
+
 def _bind(path: str) -> ctypes.CDLL:
     lib = ctypes.CDLL(path)
     p, i64, i32, sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t
     plan_p = ctypes.POINTER(Plan)
+    st_p = ctypes.POINTER(Strides)
+    lib.scanscam_scan_fwd_strided.argtypes = [p, p, p, st_p, st_p, st_p, i64, i64, i64, i32, p, sz, p, plan_p]
+    lib.scanscam_scan_fwd_strided.restype = i32
+    lib.scanscam_scan_bwd_strided.argtypes = [p, p, p, p, p, st_p, st_p, st_p, st_p, st_p, i64, i64, i64, i32,
+                                              p, sz, p, plan_p]
+    lib.scanscam_scan_bwd_strided.restype = i32
+    lib.scanscam_scan_fwd_cl_strided.argtypes = [p, p, p, st_p, st_p, st_p, i64, i64, i64, i32, p, sz, p, plan_p]
+    lib.scanscam_scan_fwd_cl_strided.restype = i32
+    lib.scanscam_scan_bwd_cl_strided.argtypes = [p, p, p, p, p, st_p, st_p, st_p, st_p, st_p, i64, i64, i64, i32,
+                                                 p, sz, p, plan_p]
+    lib.scanscam_scan_bwd_cl_strided.restype = i32
     lib.scanscam_scan_fwd.argtypes = [p, p, p, i64, i64, i32, p, sz, p]
     lib.scanscam_scan_fwd.restype = i32
     lib.scanscam_scan_bwd.argtypes = [p, p, p, p, p, i64, i64, i32, p, sz, p]
@@ -370,3 +390,155 @@ def transposed_linear_scan_backward(x: torch.Tensor, y: torch.Tensor, z: torch.T
     if rc != 0:
         raise RuntimeError(f"scanscam_scan_bwd_cl: {strerror(rc)}")
     return out_a, out_b
+
+
+# ---------------------------------------------------------------------------
+# Views without a copy. The reference's wrappers make every argument contiguous
+# first (``cuda.py:36-37, 60-62``); here a view whose scan dimension (or, for
+# channels-last storage, channel dimension) is unit-stride is handed to the
+# kernels as it is: a half of a fused projection, a slice of a longer buffer, a
+# gate broadcast over the batch.
+# ---------------------------------------------------------------------------
+def _joint_levels(sizes, strides_list):
+    """Merge leading dimensions into as few levels as all tensors allow.
+
+    ``sizes``: the shared sizes of the leading dimensions; ``strides_list``: their
+    strides, one sequence per tensor. Two neighbouring dimensions merge when, in
+    every tensor, the outer stride equals inner stride x inner size. Returns a
+    list of ``(size, [stride per tensor])``, outermost first.
+    """
+    levels = []
+    for i, n in enumerate(sizes):
+        if n == 1:
+            continue
+        st = [s[i] for s in strides_list]
+        if levels and all(p == q * n for p, q in zip(levels[-1][1], st)):
+            levels[-1] = (levels[-1][0] * n, st)
+        else:
+            levels.append((n, st))
+    return levels
+
+
+def _two_levels(sizes, strides_list):
+    """``(n0, n1, [Strides per tensor])`` if the leading dimensions fit two levels, else ``None``."""
+    levels = _joint_levels(sizes, strides_list)
+    if len(levels) > 2:
+        return None
+    zero = [0] * len(strides_list)
+    while len(levels) < 2:
+        levels.insert(0, (1, zero))
+    (n0, s0), (n1, s1) = levels
+    return n0, n1, [Strides(int(a), int(b)) for a, b in zip(s0, s1)]
+
+
+def _is_row_view(t: torch.Tensor) -> bool:
+    return t.shape[-1] == 1 or t.stride(-1) == 1
+
+
+def _is_cl_view(t: torch.Tensor) -> bool:
+    """``[..., C, T]`` with unit stride along C (and not along T): stored channels-last, possibly strided."""
+    return t.dim() >= 2 and t.shape[-2] > 1 and t.stride(-2) == 1 and not _is_row_view(t)
+
+
+def _check_same(*tensors: torch.Tensor) -> None:
+    first = tensors[0]
+    for t in tensors:
+        if t.device.type != "cuda" or t.device != first.device:
+            raise RuntimeError(f"scanscam_amd.hip: expected GPU tensors on one device, got {t.device}")
+        if t.dtype != first.dtype:
+            raise TypeError(f"scanscam_amd.hip: tensors differ in dtype ({first.dtype} and {t.dtype})")
+        if t.shape != first.shape or t.dim() < 1:
+            raise AssertionError("scanscam_amd.hip: expected tensors of one shape with at least 1 dimension")
+
+
+def _plan_ref(plan: Optional[Plan]):
+    return ctypes.byref(plan) if plan is not None else None
+
+
+def _to_cl(t: torch.Tensor) -> torch.Tensor:
+    """``t`` itself if it is stored channels-last, else a channels-last copy."""
+    return t if _is_cl_view(t) else t.mT.contiguous().mT
+
+
+def _run_rows(inputs, n_out: int, direction: int, plan: Optional[Plan]):
+    """Row layout: ``inputs`` are views with unit stride along T; outputs are new contiguous tensors."""
+    L = lib()
+    first = inputs[0]
+    shape = first.shape
+    T = shape[-1]
+    outs = [torch.empty(shape, dtype=first.dtype, device=first.device) for _ in range(n_out)]
+    if first.numel() == 0:
+        return outs
+    tensors = list(inputs) + outs
+    lv = _two_levels(shape[:-1], [t.stride()[:-1] for t in tensors])
+    if lv is None:  # more than two levels of strides: copy what is not dense
+        tensors = [t.contiguous() for t in inputs] + outs
+        lv = _two_levels(shape[:-1], [t.stride()[:-1] for t in tensors])
+    n0, n1, st = lv
+    code = _dtype_code(first.dtype)
+    with torch.cuda.device(first.device):
+        ws, ws_ptr, ws_n = _workspace(n0 * n1, T, first.dtype, direction, plan, first.device)
+        stream = torch.cuda.current_stream().cuda_stream
+        ptrs = [t.data_ptr() for t in tensors]
+        refs = [ctypes.byref(x) for x in st]
+        fn = L.scanscam_scan_fwd_strided if direction == FORWARD else L.scanscam_scan_bwd_strided
+        rc = fn(*ptrs, *refs, n0, n1, T, code, ws_ptr, ws_n, stream, _plan_ref(plan))
+    if rc != 0:
+        raise RuntimeError(f"scanscam_scan_{'fwd' if direction == FORWARD else 'bwd'}_strided: {strerror(rc)}")
+    return outs
+
+
+def _run_cl(inputs, n_out: int, direction: int, plan: Optional[Plan]):
+    """Channels-last: ``inputs`` are ``[..., C, T]`` views with unit stride along C; so are the outputs."""
+    L = lib()
+    first = inputs[0]
+    shape = first.shape
+    C, T = shape[-2], shape[-1]
+    outs = [torch.empty(shape[:-2] + (T, C), dtype=first.dtype, device=first.device).mT for _ in range(n_out)]
+    if first.numel() == 0:
+        return outs
+    tensors = list(inputs) + outs
+    levels = _joint_levels(shape[:-2], [t.stride()[:-2] for t in tensors])
+    if len(levels) > 1 or any(t.stride(-1) >= 2 ** 31 for t in tensors):
+        tensors = [t.mT.contiguous().mT for t in inputs] + outs
+        levels = _joint_levels(shape[:-2], [t.stride()[:-2] for t in tensors])
+    batch, sb = levels[0] if levels else (1, [0] * len(tensors))
+    st = [Strides(int(b), int(t.stride(-1))) for b, t in zip(sb, tensors)]
+    plan_ref = _plan_ref(plan)
+    with torch.cuda.device(first.device):
+        ws, ws_ptr, ws_n = _workspace_cl(L, batch, T, C, first.dtype, direction, plan_ref, first.device)
+        stream = torch.cuda.current_stream().cuda_stream
+        ptrs = [t.data_ptr() for t in tensors]
+        refs = [ctypes.byref(x) for x in st]
+        fn = L.scanscam_scan_fwd_cl_strided if direction == FORWARD else L.scanscam_scan_bwd_cl_strided
+        rc = fn(*ptrs, *refs, batch, T, C, _dtype_code(first.dtype), ws_ptr, ws_n, stream, plan_ref)
+    if rc != 0:
+        raise RuntimeError(f"scanscam_scan_{'fwd' if direction == FORWARD else 'bwd'}_cl_strided: {strerror(rc)}")
+    return outs
+
+
+def scan_forward(gate: torch.Tensor, value: torch.Tensor, plan: Optional[Plan] = None) -> torch.Tensor:
+    """Forward scan along the last dimension of GPU tensors of any strides; no copy where a view will do.
+
+    Both stored channels-last (unit stride along ``dim=-2``): the channels-last
+    kernels, and the result is stored channels-last too (the rule of the
+    reference's ``op.py:28-29``). Otherwise the row kernels on every tensor whose
+    last dimension is unit-stride as it is (others are copied), result contiguous.
+    """
+    _check_same(gate, value)
+    if _is_cl_view(gate) and _is_cl_view(value):
+        return _run_cl([gate, value], 1, FORWARD, plan)[0]
+    inputs = [t if _is_row_view(t) else t.contiguous() for t in (gate, value)]
+    return _run_rows(inputs, 1, FORWARD, plan)[0]
+
+
+def scan_backward(gate: torch.Tensor, output: torch.Tensor, out_grad: torch.Tensor,
+                  plan: Optional[Plan] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``(gate_grad, value_grad)`` for tensors of any strides; the counterpart of ``scan_forward``."""
+    _check_same(gate, output, out_grad)
+    if _is_cl_view(gate) and _is_cl_view(output):
+        ga, gb = _run_cl([gate, output, _to_cl(out_grad)], 2, BACKWARD, plan)
+        return ga, gb
+    inputs = [t if _is_row_view(t) else t.contiguous() for t in (gate, output, out_grad)]
+    ga, gb = _run_rows(inputs, 2, BACKWARD, plan)
+    return ga, gb

@@ -130,6 +130,87 @@ static int check_case(const char *name, long rows, long T, long C, int channels_
     return failures;
 }
 
+/*
+ * Strided entry points on the two halves of one buffer x: row layout x[B][2C][T] with a = x[:, :C],
+ * b = x[:, C:]; channels-last x[B][T][2C] with a = x[..., :C], b = x[..., C:]. Outputs are dense.
+ */
+static int check_strided(const char *name, long B, long C, long T, int channels_last, hipStream_t stream)
+{
+    const size_t n = (size_t)B * C * T;
+    float *x = malloc(2 * n * 4), *gh = malloc(n * 4), *h = malloc(n * 4), *ga = malloc(n * 4), *gb = malloc(n * 4),
+          *got = malloc(n * 4);
+    /* element (batch i, channel c, time t): in a half of x, and in a dense tensor of the same layout */
+#define XIDX(i, c, t) (channels_last ? ((size_t)(i) * T + (t)) * 2 * C + (c) : ((size_t)(i) * 2 * C + (c)) * T + (t))
+#define DIDX(i, c, t) (channels_last ? ((size_t)(i) * T + (t)) * C + (c) : ((size_t)(i) * C + (c)) * T + (t))
+    const size_t b_off = channels_last ? (size_t)C : (size_t)C * T; /* where the second half starts */
+    for (size_t i = 0; i < 2 * n; i++) x[i] = uniform01();
+    for (size_t i = 0; i < n; i++) gh[i] = 2.0f * uniform01() - 1.0f;
+    for (long i = 0; i < B; i++)
+        for (long c = 0; c < C; c++) {
+            float acc = 0.0f;
+            for (long t = 0; t < T; t++) {
+                acc = acc * x[XIDX(i, c, t)] + x[XIDX(i, c, t) + b_off];
+                h[DIDX(i, c, t)] = acc;
+            }
+            float d = 0.0f;
+            for (long t = T - 1; t >= 0; t--) {
+                d += gh[DIDX(i, c, t)];
+                gb[DIDX(i, c, t)] = d;
+                ga[DIDX(i, c, t)] = d * (t > 0 ? h[DIDX(i, c, t - 1)] : 0.0f);
+                d *= x[XIDX(i, c, t)];
+            }
+        }
+#undef XIDX
+#undef DIDX
+    float *dx = device_copy(x, 2 * n), *dgh = device_copy(gh, n), *dh = device_copy(h, n);
+    float *o0, *o1;
+    HIP_OK(hipMalloc((void **)&o0, n * 4));
+    HIP_OK(hipMalloc((void **)&o1, n * 4));
+    size_t ws_bytes = 0;
+    for (int dir = 0; dir < 2; dir++) {
+        size_t need = channels_last ? scanscam_workspace_bytes_cl(B, T, C, SCANSCAM_F32, dir, NULL)
+                                    : scanscam_workspace_bytes(B * C, T, SCANSCAM_F32, dir);
+        if (need > ws_bytes) ws_bytes = need;
+    }
+    void *ws = NULL;
+    if (ws_bytes) HIP_OK(hipMalloc(&ws, ws_bytes));
+
+    /* both halves have the strides of x; NULL = dense */
+    const scanscam_strides sx = {2 * C * T, channels_last ? 2 * C : T};
+    int failures = 0;
+    int rc = channels_last ? scanscam_scan_fwd_cl_strided(dx, dx + b_off, o0, &sx, &sx, NULL, B, T, C, SCANSCAM_F32, ws,
+                                                          ws_bytes, stream, NULL)
+                           : scanscam_scan_fwd_strided(dx, dx + b_off, o0, &sx, &sx, NULL, B, C, T, SCANSCAM_F32, ws,
+                                                       ws_bytes, stream, NULL);
+    if (rc != SCANSCAM_OK) {
+        fprintf(stderr, "abi_check: %s forward: %s\n", name, scanscam_strerror(rc));
+        failures++;
+    }
+    HIP_OK(hipStreamSynchronize(stream));
+    HIP_OK(hipMemcpy(got, o0, n * 4, hipMemcpyDeviceToHost));
+    const double eh = worst(got, h, n);
+    rc = channels_last ? scanscam_scan_bwd_cl_strided(dx, dh, dgh, o1, o0, &sx, NULL, NULL, NULL, NULL, B, T, C,
+                                                      SCANSCAM_F32, ws, ws_bytes, stream, NULL)
+                       : scanscam_scan_bwd_strided(dx, dh, dgh, o1, o0, &sx, NULL, NULL, NULL, NULL, B, C, T,
+                                                   SCANSCAM_F32, ws, ws_bytes, stream, NULL);
+    if (rc != SCANSCAM_OK) {
+        fprintf(stderr, "abi_check: %s backward: %s\n", name, scanscam_strerror(rc));
+        failures++;
+    }
+    HIP_OK(hipStreamSynchronize(stream));
+    HIP_OK(hipMemcpy(got, o0, n * 4, hipMemcpyDeviceToHost));
+    const double egb = worst(got, gb, n);
+    HIP_OK(hipMemcpy(got, o1, n * 4, hipMemcpyDeviceToHost));
+    const double ega = worst(got, ga, n);
+    printf("abi_check: %-28s workspace %8zu B  worst relative error h %.2e  grad_b %.2e  grad_a %.2e\n", name,
+           ws_bytes, eh, egb, ega);
+    if (!(eh <= 1e-5) || !(egb <= 1e-5) || !(ega <= 2e-5)) failures++;
+    hipFree(dx); hipFree(dgh); hipFree(dh); hipFree(o0); hipFree(o1);
+    if (ws) hipFree(ws);
+    free(x); free(gh); free(h); free(ga); free(gb); free(got);
+    return failures;
+}
+
 int main(void)
 {
     if (scanscam_abi_version() != 1) {
@@ -145,6 +226,9 @@ int main(void)
     failures += check_case("long rows [3, 300000]", 3, 300000, 0, 0, stream);
     failures += check_case("channels-last [4, 999, 320]", 4 * 320, 999, 320, 1, stream);
     failures += check_case("channels-last [1, 2048, 64]", 64, 2048, 64, 1, stream);
+    failures += check_strided("halves of x[6][2*40][1000]", 6, 40, 1000, 0, stream);
+    failures += check_strided("halves of x[2][2*3][200000]", 2, 3, 200000, 0, stream);
+    failures += check_strided("halves of x[5][777][2*192]", 5, 192, 777, 1, stream);
     /* Argument errors come back as codes, with nothing launched. */
     if (scanscam_scan_fwd(NULL, NULL, NULL, 4, 8, SCANSCAM_F32, NULL, 0, stream) != SCANSCAM_EINVAL) failures++;
     if (scanscam_scan_fwd(NULL, NULL, NULL, 0, 8, SCANSCAM_F32, NULL, 0, stream) != SCANSCAM_OK) failures++;

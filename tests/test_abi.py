@@ -32,7 +32,7 @@ def test_library_is_built_and_loads():
 
 def test_every_declared_symbol_is_exported():
     names = declared_functions()
-    assert "scanscam_scan_fwd" in names and "scanscam_scan_bwd" in names and len(names) == 12
+    assert "scanscam_scan_fwd" in names and "scanscam_scan_bwd" in names and len(names) == 16
     raw = ctypes.CDLL(hip.LIB_PATH)
     for name in names:
         assert hasattr(raw, name), f"{name} declared in scanscam_hip.h but not exported"
@@ -90,6 +90,35 @@ def test_argument_errors_are_reported_before_any_launch():
     # ... and element-aligned long rows only with 2 or 4 chunks per wave.
     v4u8 = hip.Plan(vec=4, unroll=8)
     assert L.scanscam_scan_fwd_plan(fake, fake, fake, 4, 1025, 0, None, 0, None, ctypes.byref(v4u8)) == E_PLAN
+
+
+def test_strided_calls_check_their_arguments():
+    L = hip.lib()
+    fake = ctypes.c_void_p(0x1000)
+    S = hip.Strides
+    assert ctypes.sizeof(S) == 16
+    dense = ctypes.byref(S(4096, 64))
+    neg = ctypes.byref(S(-1, 64))
+    # negative strides, negative sizes and a row count that overflows are rejected before any launch
+    assert L.scanscam_scan_fwd_strided(fake, fake, fake, neg, dense, dense, 4, 64, 64, 0, None, 0, None, None) == E_INVAL
+    assert L.scanscam_scan_fwd_strided(fake, fake, fake, dense, dense, dense, -1, 64, 64, 0, None, 0, None, None) == E_INVAL
+    assert L.scanscam_scan_fwd_strided(fake, fake, fake, None, None, None, 1 << 40, 1 << 40, 64, 0, None, 0, None,
+                                       None) == E_INVAL
+    assert L.scanscam_scan_bwd_strided(fake, fake, fake, fake, None, None, None, None, None, None, 4, 64, 64, 0, None,
+                                       0, None, None) == E_INVAL
+    # rows whose starts are not all 16-byte aligned cannot take a forced 16-byte vector when short
+    v4 = hip.Plan(vec=4)
+    odd = ctypes.byref(S(4096, 65))
+    assert L.scanscam_scan_fwd_strided(fake, fake, fake, odd, dense, dense, 4, 64, 64, 0, None, 0, None,
+                                       ctypes.byref(v4)) == E_PLAN
+    # channels-last: the time stride is a 32-bit quantity
+    big = ctypes.byref(S(0, 1 << 31))
+    assert L.scanscam_scan_fwd_cl_strided(fake, fake, fake, big, None, None, 2, 8, 64, 0, None, 0, None, None) == E_INVAL
+    assert L.scanscam_scan_bwd_cl_strided(fake, fake, fake, fake, fake, neg, None, None, None, None, 2, 8, 64, 0, None,
+                                          0, None, None) == E_INVAL
+    # empty problems succeed without touching anything
+    assert L.scanscam_scan_fwd_strided(None, None, None, None, None, None, 0, 5, 64, 0, None, 0, None, None) == E_OK
+    assert L.scanscam_scan_fwd_cl_strided(None, None, None, None, None, None, 3, 0, 64, 0, None, 0, None, None) == E_OK
 
 
 def test_empty_inputs_are_a_successful_noop():
