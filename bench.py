@@ -215,6 +215,54 @@ def reference_grid(dev, args, hip, torch):
     return out
 
 
+def strided_views(dev, args, hip, torch):
+    """Views scanned in place against copy-then-scan (what the reference's wrappers do, cuda.py:36-37).
+
+    Row layout: the halves of one fused projection x[8, 2*2048, 4096] (a, b = x.chunk(2, dim=1)), i.e.
+    config 2's shape with two levels of row strides. Channels-last: the halves of x[64, 2048, 2*1024].
+    Mean microseconds per call, output allocation included on both sides.
+    """
+    def mean_us(fn):
+        for _ in range(max(3, args.warmup // 2)):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(args.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.steps * 1e3
+
+    out = {}
+    torch.manual_seed(0)
+    for name, shape, dim, to_logical in (
+            ("rows_halves_of_8x4096x4096", (8, 4096, 4096), 1, lambda t: t),
+            ("channels_last_halves_of_64x2048x2048", (64, 2048, 2048), 2, lambda t: t.mT)):
+        x = torch.randn(shape, device=dev)
+        g = torch.randn(shape, device=dev)
+        half = shape[dim] // 2
+        x.narrow(dim, 0, half).sigmoid_()
+        a, b = (to_logical(t) for t in x.chunk(2, dim=dim))
+        gh = to_logical(g.narrow(dim, half, half))
+        h = hip.scan_forward(a, b)
+        n = a.numel()
+        dense = (lambda t: t.contiguous()) if dim == 1 else (lambda t: t.mT.contiguous().mT)
+        f_us = mean_us(lambda: hip.scan_forward(a, b))
+        b_us = mean_us(lambda: hip.scan_backward(a, h, gh))
+        fc_us = mean_us(lambda: hip.scan_forward(dense(a), dense(b)))
+        bc_us = mean_us(lambda: hip.scan_backward(dense(a), h, dense(gh)))
+        out[name] = {
+            "fwd_us": round(f_us, 1), "bwd_us": round(b_us, 1),
+            "fwd_frac": round(12 * n / (f_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+            "bwd_frac": round(20 * n / (b_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+            "copy_first_fwd_us": round(fc_us, 1), "copy_first_bwd_us": round(bc_us, 1),
+        }
+        del x, g, a, b, gh, h
+        torch.cuda.empty_cache()
+    return out
+
+
 def cpu_baseline(a, b, gh, reps):
     """The reference's CPU loop on the same tensors, one thread."""
     import numpy as np
@@ -402,6 +450,7 @@ def main():
 
     if not args.no_configs:
         out["reference_grid"] = reference_grid(dev, args, hip, torch)
+        out["strided_views"] = strided_views(dev, args, hip, torch)
 
     if not args.no_cpu:
         # 16-bit workloads: the reference has no 16-bit path, so its loop runs on the exact fp32 upcast.

@@ -91,6 +91,50 @@ def test_gpu_entry_points_reject_cpu_tensors_and_unknown_dtypes():
         hip.resolve_plan(4, 8, torch.int32)
 
 
+def _levels(*tensors):
+    return hip._two_levels(tensors[0].shape[:-1], [t.stride()[:-1] for t in tensors])
+
+
+def test_views_are_described_by_at_most_two_stride_levels():
+    """The host logic that lets the strided entry points take views as they are (no GPU involved)."""
+    T = 12
+    dense = torch.zeros(4, 6, T)
+    n0, n1, st = _levels(dense)
+    assert (n0, n1) == (1, 24) and (st[0].outer, st[0].row) == (0, T)       # one level: rows follow each other
+    x = torch.zeros(4, 12, T)
+    a, b = x.chunk(2, dim=1)                                                # halves of a fused projection
+    n0, n1, st = _levels(a, b, dense)
+    assert (n0, n1) == (4, 6)
+    assert [(s.outer, s.row) for s in st] == [(12 * T, T), (12 * T, T), (6 * T, T)]
+    sl = torch.zeros(4, 6, 20)[..., 3:3 + T]                                # a slice along time: one level, pitch 20
+    n0, n1, st = _levels(sl)
+    assert (n0, n1) == (1, 24) and st[0].row == 20
+    bc = torch.zeros(1, 6, T).expand(4, 6, T)                               # broadcast over the batch: stride 0
+    n0, n1, st = _levels(bc, dense)
+    assert (n0, n1) == (4, 6) and (st[0].outer, st[0].row) == (0, T) and (st[1].outer, st[1].row) == (6 * T, T)
+    assert _levels(torch.zeros(2, 6, 8, T)[:, :3, :4]) is None               # three levels: needs a copy
+    assert _levels(torch.zeros(2, 1, 8, T)[:, :, :4])[:2] == (2, 4)          # size-1 dimensions do not count
+    assert _levels(torch.zeros(T))[:2] == (1, 1)                            # a single row
+    # size-1 dimensions merge with anything
+    assert hip._joint_levels((3, 1, 5), [(40, 7, 8)]) == [(15, [8])]
+
+
+def test_layout_classification_of_views():
+    x = torch.zeros(2, 5, 3)
+    assert hip._is_row_view(x) and not hip._is_cl_view(x)
+    assert hip._is_cl_view(x.mT) and not hip._is_row_view(x.mT)
+    half = torch.zeros(2, 5, 6).chunk(2, dim=-1)[0].mT                       # [2, 3, 5] stored [2, 5, 2*3]
+    assert hip._is_cl_view(half) and half.stride(-1) == 6
+    assert hip._is_row_view(torch.zeros(4, 9)[:, 2:7])
+    assert not hip._is_row_view(torch.zeros(4, 9)[:, ::2]) and not hip._is_cl_view(torch.zeros(4, 9)[:, ::2])
+    assert hip._is_row_view(torch.zeros(4, 1).expand(4, 1))                  # T == 1: any stride will do
+    for bad in (torch.zeros(2, 8), ):
+        with pytest.raises(RuntimeError, match="GPU tensors"):
+            hip.scan_forward(bad, bad)
+        with pytest.raises(RuntimeError, match="GPU tensors"):
+            hip.scan_backward(bad, bad, bad)
+
+
 def test_package_never_imports_the_oracle():
     import os
     import re
