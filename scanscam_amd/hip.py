@@ -199,7 +199,7 @@ def scan_forward_out(gate: torch.Tensor, value: torch.Tensor, out: torch.Tensor,
     code = _dtype_code(gate.dtype)
     if rows == 0 or T == 0:
         return
-    with torch.cuda.device(gate.device):
+    with _on(gate.device):
         ws, ws_ptr, ws_n = _workspace(rows, T, gate.dtype, FORWARD, plan, gate.device)
         stream = torch.cuda.current_stream().cuda_stream
         rc = L.scanscam_scan_fwd_plan(gate.data_ptr(), value.data_ptr(), out.data_ptr(), rows, T, code,
@@ -218,7 +218,7 @@ def scan_backward_out(gate: torch.Tensor, output: torch.Tensor, out_grad: torch.
     code = _dtype_code(gate.dtype)
     if rows == 0 or T == 0:
         return
-    with torch.cuda.device(gate.device):
+    with _on(gate.device):
         ws, ws_ptr, ws_n = _workspace(rows, T, gate.dtype, BACKWARD, plan, gate.device)
         stream = torch.cuda.current_stream().cuda_stream
         rc = L.scanscam_scan_bwd_plan(gate.data_ptr(), output.data_ptr(), out_grad.data_ptr(),
@@ -360,7 +360,7 @@ def transposed_linear_scan_forward(x: torch.Tensor, y: torch.Tensor, channels_pe
     if x.numel() == 0:
         return out
     plan_ref = ctypes.byref(plan) if plan is not None else None
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         ws, ws_ptr, ws_n = _workspace_cl(L, batch, T, C, x.dtype, FORWARD, plan_ref, x.device)
         rc = L.scanscam_scan_fwd_cl(x.data_ptr(), y.data_ptr(), out.data_ptr(), batch, T, C, _dtype_code(x.dtype),
                                     ws_ptr, ws_n, torch.cuda.current_stream().cuda_stream, plan_ref)
@@ -382,7 +382,7 @@ def transposed_linear_scan_backward(x: torch.Tensor, y: torch.Tensor, z: torch.T
     if x.numel() == 0:
         return out_a, out_b
     plan_ref = ctypes.byref(plan) if plan is not None else None
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         ws, ws_ptr, ws_n = _workspace_cl(L, batch, T, C, x.dtype, BACKWARD, plan_ref, x.device)
         rc = L.scanscam_scan_bwd_cl(x.data_ptr(), y.data_ptr(), z.data_ptr(), out_a.data_ptr(), out_b.data_ptr(),
                                     batch, T, C, _dtype_code(x.dtype), ws_ptr, ws_n,
@@ -460,6 +460,26 @@ def _to_cl(t: torch.Tensor) -> torch.Tensor:
     return t if _is_cl_view(t) else t.mT.contiguous().mT
 
 
+class _NoSwitch:
+    """Stands in for ``torch.cuda.device(...)`` when that device is already current."""
+
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _on(device: torch.device):
+    """Context that makes ``device`` current; free when it already is (the usual case)."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NO_SWITCH
+    return torch.cuda.device(device)
+
+
 def _run_rows(inputs, n_out: int, direction: int, plan: Optional[Plan]):
     """Row layout: ``inputs`` are views with unit stride along T; outputs are new contiguous tensors."""
     L = lib()
@@ -470,17 +490,20 @@ def _run_rows(inputs, n_out: int, direction: int, plan: Optional[Plan]):
     if first.numel() == 0:
         return outs
     tensors = list(inputs) + outs
-    lv = _two_levels(shape[:-1], [t.stride()[:-1] for t in tensors])
-    if lv is None:  # more than two levels of strides: copy what is not dense
-        tensors = [t.contiguous() for t in inputs] + outs
+    if all(t.is_contiguous() for t in inputs):  # the common case, kept short: one level, dense
+        n0, n1, refs = 1, first.numel() // T, (None,) * len(tensors)
+    else:
         lv = _two_levels(shape[:-1], [t.stride()[:-1] for t in tensors])
-    n0, n1, st = lv
+        if lv is None:  # more than two levels of strides: copy what is not dense
+            tensors = [t.contiguous() for t in inputs] + outs
+            lv = _two_levels(shape[:-1], [t.stride()[:-1] for t in tensors])
+        n0, n1, st = lv
+        refs = [ctypes.byref(x) for x in st]
     code = _dtype_code(first.dtype)
-    with torch.cuda.device(first.device):
+    with _on(first.device):
         ws, ws_ptr, ws_n = _workspace(n0 * n1, T, first.dtype, direction, plan, first.device)
         stream = torch.cuda.current_stream().cuda_stream
         ptrs = [t.data_ptr() for t in tensors]
-        refs = [ctypes.byref(x) for x in st]
         fn = L.scanscam_scan_fwd_strided if direction == FORWARD else L.scanscam_scan_bwd_strided
         rc = fn(*ptrs, *refs, n0, n1, T, code, ws_ptr, ws_n, stream, _plan_ref(plan))
     if rc != 0:
@@ -505,7 +528,7 @@ def _run_cl(inputs, n_out: int, direction: int, plan: Optional[Plan]):
     batch, sb = levels[0] if levels else (1, [0] * len(tensors))
     st = [Strides(int(b), int(t.stride(-1))) for b, t in zip(sb, tensors)]
     plan_ref = _plan_ref(plan)
-    with torch.cuda.device(first.device):
+    with _on(first.device):
         ws, ws_ptr, ws_n = _workspace_cl(L, batch, T, C, first.dtype, direction, plan_ref, first.device)
         stream = torch.cuda.current_stream().cuda_stream
         ptrs = [t.data_ptr() for t in tensors]
