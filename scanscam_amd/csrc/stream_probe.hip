@@ -10,6 +10,10 @@
 //   stream_probe policy [rows]   the same two shapes with every combination of the sc0 / sc1 / nt cache-policy bits on
 //                             the loads or on the stores, over 8 rotated buffer sets so that no cache level can
 //                             hold an output between launches. Shows which policy the kernels should use.
+//   stream_probe mix             what the memory system gives each mix of read and write streams (1R0W ... 3R2W,
+//                             268 MB per stream, 4 rotated buffer sets) and each workgroup shape (W waves x U
+//                             16-byte accesses per lane per stream): the ceilings the scan kernels are measured
+//                             against.
 //
 //   hipcc -O3 --offload-arch=gfx950 stream_probe.hip -o stream_probe
 #include <hip/hip_runtime.h>
@@ -55,6 +59,44 @@ __global__ __launch_bounds__(256) void stream_shape_kernel(const f4 *__restrict_
 #pragma unroll
     for (int u = 0; u < 4; u++) {
         f4 r = va[u];
+        if (READS > 1) r += vb[u];
+        if (READS > 2) r *= vc[u];
+        __builtin_nontemporal_store(r, o0 + base + u * 64);
+        if (WRITES > 1) __builtin_nontemporal_store(r + 1.0f, o1 + base + u * 64);
+    }
+}
+
+// The same for any mix of streams and any workgroup shape: W waves, U consecutive 1 KiB spans per wave and
+// stream, all loads issued before the first store. With no output stream the sum of what was read is
+// compared with a value it never takes, so the loads stay.
+template <int READS, int WRITES, int U, int W>
+__global__ __launch_bounds__(W * 64) void stream_mix_kernel(const f4 *__restrict__ a, const f4 *__restrict__ b,
+                                                            const f4 *__restrict__ c, f4 *__restrict__ o0,
+                                                            f4 *__restrict__ o1, float never)
+{
+    const size_t base = (size_t)blockIdx.x * (W * U * 64) + (threadIdx.x / 64) * (U * 64) + (threadIdx.x % 64);
+    f4 va[U], vb[U], vc[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        if (READS > 0) va[u] = __builtin_nontemporal_load(a + base + u * 64);
+        if (READS > 1) vb[u] = __builtin_nontemporal_load(b + base + u * 64);
+        if (READS > 2) vc[u] = __builtin_nontemporal_load(c + base + u * 64);
+    }
+    if (WRITES == 0) {
+        f4 s = 0;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            s += va[u];
+            if (READS > 1) s += vb[u];
+            if (READS > 2) s += vc[u];
+        }
+        if (s.x + s.y + s.z + s.w == never) o0[base] = s;
+        return;
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        f4 r = never;
+        if (READS > 0) r = va[u];
         if (READS > 1) r += vb[u];
         if (READS > 2) r *= vc[u];
         __builtin_nontemporal_store(r, o0 + base + u * 64);
@@ -207,11 +249,66 @@ static int run_policy(size_t rows)
     return hipDeviceSynchronize() == hipSuccess ? 0 : 1;
 }
 
+static f4 *g_mix[4][5];
+
+template <int READS, int WRITES, int U, int W> static void mix_case()
+{
+    const size_t n = (size_t)16384 * 4096;  // elements per stream
+    int i = 0;
+    const float ms = mean_ms(
+        [&] {
+            f4 **s = g_mix[i++ % 4];
+            hipLaunchKernelGGL((stream_mix_kernel<READS, WRITES, U, W>), dim3((unsigned)(n / 4 / (W * U * 64))),
+                               dim3(W * 64), 0, 0, s[0], s[1], s[2], s[3], s[4], 12345.678f);
+        },
+        40);
+    const double bytes = (double)(READS + WRITES) * n * 4;
+    printf("  %dR%dW  %2d waves x %d accesses  %7.1f us  %7.1f GB/s  %4.1f %% of 8 TB/s\n", READS, WRITES, W, U, ms * 1e3,
+           bytes / (ms * 1e-3) / 1e9, bytes / (ms * 1e-3) / 8e12 * 100);
+}
+
+static int run_mix()
+{
+    const size_t bytes = (size_t)16384 * 4096 * 4;
+    for (auto &set : g_mix)
+        for (auto &p : set) {
+            CHECK(hipMalloc(&p, bytes));
+            CHECK(hipMemset(p, 0, bytes));
+        }
+    printf("stream mixes, 67 108 864 fp32 per stream, non-temporal 16-byte accesses, 4 rotated buffer sets:\n");
+    mix_case<1, 0, 4, 4>();
+    mix_case<1, 0, 1, 16>();
+    mix_case<2, 0, 4, 4>();
+    mix_case<3, 0, 4, 4>();
+    mix_case<0, 1, 4, 4>();
+    mix_case<0, 2, 4, 4>();
+    mix_case<1, 1, 4, 4>();
+    printf("forward mix (2 reads + 1 write) by workgroup shape:\n");
+    mix_case<2, 1, 1, 4>();
+    mix_case<2, 1, 2, 4>();
+    mix_case<2, 1, 4, 4>();
+    mix_case<2, 1, 8, 4>();
+    mix_case<2, 1, 2, 8>();
+    mix_case<2, 1, 4, 8>();
+    mix_case<2, 1, 1, 16>();
+    mix_case<2, 1, 4, 16>();
+    printf("backward mix (3 reads + 2 writes) by workgroup shape:\n");
+    mix_case<3, 2, 1, 4>();
+    mix_case<3, 2, 2, 4>();
+    mix_case<3, 2, 4, 4>();
+    mix_case<3, 2, 2, 8>();
+    mix_case<3, 2, 4, 8>();
+    mix_case<3, 2, 1, 16>();
+    mix_case<3, 2, 4, 16>();
+    return hipDeviceSynchronize() == hipSuccess ? 0 : 1;
+}
+
 int main(int argc, char **argv)
 {
+    if (argc > 1 && strcmp(argv[1], "mix") == 0) return run_mix();
     if (argc > 1 && strcmp(argv[1], "ceiling") == 0) return run_ceiling(argc > 2 ? (size_t)atol(argv[2]) : 16384);
     if (argc > 1 && strcmp(argv[1], "copy") == 0) return run_copy(argc > 2 ? (size_t)atol(argv[2]) : 1024);
     if (argc > 1 && strcmp(argv[1], "policy") == 0) return run_policy(argc > 2 ? (size_t)atol(argv[2]) : 16384);
-    fprintf(stderr, "usage: %s copy [MiB] | ceiling [rows] | policy [rows]\n", argv[0]);
+    fprintf(stderr, "usage: %s copy [MiB] | ceiling [rows] | policy [rows] | mix\n", argv[0]);
     return 2;
 }
