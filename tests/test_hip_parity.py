@@ -486,3 +486,51 @@ def test_launch_is_split_when_a_grid_would_exceed_2_pow_32_threads(gpu):
     ga, gb = hip.linear_scan_backward(a, h, b, plan)
     wga, wgb = hip.linear_scan_backward(a, h, b)
     assert float((gb - wgb).abs().max()) <= 1e-5 and float((ga - wga).abs().max()) <= 1e-4
+
+
+def test_more_than_2_pow_32_elements(gpu):
+    # Offsets beyond 32 bits. Rows are independent and the result of a row does not depend on the
+    # launch it is part of, so a slab of rows scanned on its own must be bit-identical to the same
+    # rows of the full tensor; slabs are taken at the start, across element 2^31, across element 2^32
+    # and at the end, and one slab is also checked against the oracle.
+    free, _ = torch.cuda.mem_get_info(gpu)
+    rows, T = (1 << 20) + 3, 4104
+    if free < 6 * rows * T * 2 + (4 << 30):
+        pytest.skip("not enough free device memory for six 8.6 GB tensors")
+    assert rows * T > (1 << 32)
+    g = torch.Generator(device=gpu).manual_seed(11)
+    a = torch.rand((rows, T), generator=g, device=gpu, dtype=torch.bfloat16)
+    b = torch.randn((rows, T), generator=g, device=gpu, dtype=torch.bfloat16)
+    h = hip.linear_scan_forward(a, b)
+    ga, gb = hip.linear_scan_backward(a, h, b)
+    r31, r32 = (1 << 31) // T, (1 << 32) // T
+    for r0 in (0, r31 - 2, r32 - 2, rows - 5):
+        s = slice(r0, r0 + 5)
+        a_s, b_s, h_s = a[s].clone(), b[s].clone(), h[s].clone()
+        assert torch.equal(hip.linear_scan_forward(a_s, b_s), h[s]), f"forward rows {r0}.."
+        ga_s, gb_s = hip.linear_scan_backward(a_s, h_s, b_s)
+        assert torch.equal(ga_s, ga[s]) and torch.equal(gb_s, gb[s]), f"backward rows {r0}.."
+    s = slice(r32 - 2, r32 + 3)
+    assert rel_err(to_np(h[s]), oracle.fwd(upcast(a[s].cpu()), upcast(b[s].cpu()))) <= HALF_BAR
+    del a, b, h, ga, gb
+
+    # The look-back kernel: 5 rows of 2^30 float32 (5.4e9 elements). Gate 0 makes the scan the
+    # identity, so every element of the output names the input element it was read from; then a
+    # slab against the same row scanned alone.
+    rows, T = 5, 1 << 30
+    if free < 3 * rows * T * 4 + (8 << 30):
+        pytest.skip("not enough free device memory for three 21 GB tensors")
+    b = torch.randn((rows, T), generator=g, device=gpu)
+    a = torch.zeros_like(b)
+    h = hip.linear_scan_forward(a, b)
+    assert torch.equal(h, b)
+    a.uniform_(0.9, 1.0, generator=g)
+    h = hip.linear_scan_forward(a, b)
+    for r in (0, 2, 4):
+        assert torch.equal(hip.linear_scan_forward(a[r:r + 1].clone(), b[r:r + 1].clone()), h[r:r + 1]), f"row {r}"
+    # restart property across element 2^32 of the tensor (row 4 starts at 2^32)
+    k = 1 << 29
+    b_tail = b[4:5, k:].clone()
+    b_tail[:, 0] += a[4, k] * h[4, k - 1]
+    tail = hip.linear_scan_forward(a[4:5, k:].contiguous(), b_tail)
+    assert float((tail - h[4:5, k:]).abs().max()) <= 1e-4
