@@ -14,6 +14,11 @@
 //                             268 MB per stream, 4 rotated buffer sets) and each workgroup shape (W waves x U
 //                             16-byte accesses per lane per stream): the ceilings the scan kernels are measured
 //                             against.
+//   stream_probe order           the look-back kernel's tile shape (8 waves x 4 accesses) with its order of work:
+//                             the 67 108 864 elements of a stream are cut into R rows, and workgroup k takes tile
+//                             k / R of row k % R, so that tiles of all rows are in flight together. R = 1 is the
+//                             plain linear order. What the memory system gives that order with no scan, no tickets
+//                             and no carry chain.
 //
 //   hipcc -O3 --offload-arch=gfx950 stream_probe.hip -o stream_probe
 #include <hip/hip_runtime.h>
@@ -98,6 +103,30 @@ __global__ __launch_bounds__(W * 64) void stream_mix_kernel(const f4 *__restrict
         f4 r = never;
         if (READS > 0) r = va[u];
         if (READS > 1) r += vb[u];
+        if (READS > 2) r *= vc[u];
+        __builtin_nontemporal_store(r, o0 + base + u * 64);
+        if (WRITES > 1) __builtin_nontemporal_store(r + 1.0f, o1 + base + u * 64);
+    }
+}
+
+// stream_mix_kernel with the look-back kernel's order of work: workgroup k works on tile k / R of row k % R.
+template <int READS, int WRITES, int U, int W>
+__global__ __launch_bounds__(W * 64) void stream_order_kernel(const f4 *__restrict__ a, const f4 *__restrict__ b,
+                                                              const f4 *__restrict__ c, f4 *__restrict__ o0,
+                                                              f4 *__restrict__ o1, unsigned R, size_t row_vecs)
+{
+    const size_t base = (size_t)(blockIdx.x % R) * row_vecs + (size_t)(blockIdx.x / R) * (W * U * 64) +
+                        (threadIdx.x / 64) * (U * 64) + (threadIdx.x % 64);
+    f4 va[U], vb[U], vc[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        va[u] = __builtin_nontemporal_load(a + base + u * 64);
+        vb[u] = __builtin_nontemporal_load(b + base + u * 64);
+        if (READS > 2) vc[u] = __builtin_nontemporal_load(c + base + u * 64);
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        f4 r = va[u] + vb[u];
         if (READS > 2) r *= vc[u];
         __builtin_nontemporal_store(r, o0 + base + u * 64);
         if (WRITES > 1) __builtin_nontemporal_store(r + 1.0f, o1 + base + u * 64);
@@ -303,12 +332,44 @@ static int run_mix()
     return hipDeviceSynchronize() == hipSuccess ? 0 : 1;
 }
 
+template <int READS, int WRITES> static void order_case(unsigned R)
+{
+    constexpr int U = 4, W = 8;
+    const size_t n = (size_t)16384 * 4096, vecs = n / 4, tile_vecs = W * U * 64;  // R divides vecs / tile_vecs
+    int i = 0;
+    const float ms = mean_ms(
+        [&] {
+            f4 **s = g_mix[i++ % 4];
+            hipLaunchKernelGGL((stream_order_kernel<READS, WRITES, U, W>), dim3((unsigned)(vecs / tile_vecs)), dim3(W * 64),
+                               0, 0, s[0], s[1], s[2], s[3], s[4], R, vecs / R);
+        },
+        40);
+    const double bytes = (double)(READS + WRITES) * n * 4;
+    printf("  %dR%dW  %5u rows of %8zu  %7.1f us  %7.1f GB/s  %4.1f %% of 8 TB/s\n", READS, WRITES, R, n / R, ms * 1e3,
+           bytes / (ms * 1e-3) / 1e9, bytes / (ms * 1e-3) / 8e12 * 100);
+}
+
+static int run_order()
+{
+    const size_t bytes = (size_t)16384 * 4096 * 4;
+    for (auto &set : g_mix)
+        for (auto &p : set) {
+            CHECK(hipMalloc(&p, bytes));
+            CHECK(hipMemset(p, 0, bytes));
+        }
+    printf("order of work, 67 108 864 fp32 per stream, 8 waves x 4 accesses (8192-element tiles), workgroup k -> tile k / R of row k %% R:\n");
+    for (unsigned R : {1u, 8u, 64u, 256u, 1024u}) order_case<2, 1>(R);
+    for (unsigned R : {1u, 8u, 64u, 256u, 1024u}) order_case<3, 2>(R);
+    return hipDeviceSynchronize() == hipSuccess ? 0 : 1;
+}
+
 int main(int argc, char **argv)
 {
+    if (argc > 1 && strcmp(argv[1], "order") == 0) return run_order();
     if (argc > 1 && strcmp(argv[1], "mix") == 0) return run_mix();
     if (argc > 1 && strcmp(argv[1], "ceiling") == 0) return run_ceiling(argc > 2 ? (size_t)atol(argv[2]) : 16384);
     if (argc > 1 && strcmp(argv[1], "copy") == 0) return run_copy(argc > 2 ? (size_t)atol(argv[2]) : 1024);
     if (argc > 1 && strcmp(argv[1], "policy") == 0) return run_policy(argc > 2 ? (size_t)atol(argv[2]) : 16384);
-    fprintf(stderr, "usage: %s copy [MiB] | ceiling [rows] | policy [rows] | mix\n", argv[0]);
+    fprintf(stderr, "usage: %s copy [MiB] | ceiling [rows] | policy [rows] | mix | order\n", argv[0]);
     return 2;
 }
