@@ -16,7 +16,8 @@ region instead of configuration 2 (used for the rocprofv3 summaries under profil
 
 Prints ONE JSON line. Besides the contract fields it carries
   roofline      the dominant kernel (backward) against the 8 TB/s HBM peak, its
-                duration measured with HIP events on the launch stream;
+                duration measured with HIP events on the launch stream, bound to
+                the kernel itself (start and end of the kernel on the GPU);
   roofline_fwd  the same for the forward kernel;
   cpu_baseline  the reference's single-threaded CPU loop on the same tensors,
                 timed on this host (oracle/_ref if it was built, else the C
@@ -109,36 +110,35 @@ def time_kernels(sets, steps, warmup, hip, torch):
     """Runs (forward; backward) `steps` times, rotating over `sets`.
 
     Returns (wall seconds per step, mean fwd kernel ms, mean bwd kernel ms,
-    min fwd ms, min bwd ms); the kernel times come from HIP events recorded on
-    the launch stream around the launches of a sample of the steps.
+    min fwd ms, min bwd ms). The kernel times come from HIP events on the launch
+    stream that the library binds to the scan kernels themselves
+    (scanscam_scan_fwd_timed / _bwd_timed): each pair holds its kernel's start and
+    end on the GPU. Ten steps spread evenly over the region are sampled (a launch
+    that carries events costs a few microseconds more on the stream, which the
+    wall time of the region would otherwise show).
     """
     calls = [(hip.prepare_forward(s.a, s.b, s.h), hip.prepare_backward(s.a, s.h, s.gh, s.ga, s.gb)) for s in sets]
+    stride = max(1, steps // 10)
+    timed = {}
+    for i in range(0, steps, stride):
+        s = sets[i % len(sets)]
+        ef, eb = hip.KernelEvents(), hip.KernelEvents()
+        timed[i] = (hip.prepare_forward(s.a, s.b, s.h, events=ef),
+                    hip.prepare_backward(s.a, s.h, s.gh, s.ga, s.gb, events=eb), ef, eb)
     for i in range(warmup):
         f, b = calls[i % len(calls)]
         f()
         b()
-    # Events bracket the launches of every `stride`-th step only (at least 10 steps): an event pair
-    # around every launch would put ~3 us of event packets between all kernels of the timed region.
-    stride = max(1, steps // 10)
-    ev = {i: [torch.cuda.Event(enable_timing=True) for _ in range(3)] for i in range(0, steps, stride)}
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(steps):
-        f, b = calls[i % len(calls)]
-        e = ev.get(i)
-        if e is None:
-            f()
-            b()
-        else:
-            e[0].record()
-            f()
-            e[1].record()
-            b()
-            e[2].record()
+        f, b = timed[i][:2] if i in timed else calls[i % len(calls)]
+        f()
+        b()
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / steps
-    fwd = [e[0].elapsed_time(e[1]) for e in ev.values()]
-    bwd = [e[1].elapsed_time(e[2]) for e in ev.values()]
+    fwd = [t[2].elapsed_ms() for t in timed.values()]
+    bwd = [t[3].elapsed_ms() for t in timed.values()]
     return wall, statistics.fmean(fwd), statistics.fmean(bwd), min(fwd), min(bwd)
 
 

@@ -116,6 +116,21 @@ size_t scanscam_workspace_bytes_plan(int64_t rows, int64_t T, int dtype, int dir
                                      const scanscam_plan *plan);
 
 /*
+ * Measurement aid (no counterpart in the reference): the _plan calls with the scan kernel's own start
+ * and end on the GPU recorded into two HIP events the caller created (hipEventCreate), so that
+ * hipEventElapsedTime(start, stop) is the kernel's duration, free of launch gaps and of the event
+ * packets a hipEventRecord pair would put around it. Either event may be NULL. The kernel that
+ * clears the workspace of a long-row launch is not part of the interval. A problem so large that it
+ * needs several launches (more than 2^32 threads) returns SCANSCAM_EINVAL here.
+ */
+int scanscam_scan_fwd_timed(const void *a, const void *b, void *h, int64_t rows, int64_t T, int dtype,
+                            void *workspace, size_t workspace_bytes, void *stream, const scanscam_plan *plan,
+                            void *start_event, void *stop_event);
+int scanscam_scan_bwd_timed(const void *a, const void *h, const void *gh, void *ga, void *gb, int64_t rows,
+                            int64_t T, int dtype, void *workspace, size_t workspace_bytes, void *stream,
+                            const scanscam_plan *plan, void *start_event, void *stop_event);
+
+/*
  * Channels-last storage: every tensor is a dense [batch, T, C] array (C
  * fastest) scanned along T -- the layout of a [batch, C, T] tensor whose last
  * two dimensions were transposed. Same arithmetic as the calls above.

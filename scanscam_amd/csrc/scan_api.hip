@@ -191,7 +191,8 @@ const scanscam_strides *const kDense[5] = {nullptr, nullptr, nullptr, nullptr, n
 // gb backwards; h and y1 = ga exist only backwards). st[k] == nullptr means dense.
 int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y1,
         const scanscam_strides *const st[5], int64_t n0, int64_t n1, int64_t T, int dtype, void *workspace,
-        size_t workspace_bytes, void *stream, const scanscam_plan *plan)
+        size_t workspace_bytes, void *stream, const scanscam_plan *plan, void *start_event = nullptr,
+        void *stop_event = nullptr)
 {
     const int esize = elem_size(dtype);
     if (esize == 0) return SCANSCAM_EDTYPE;
@@ -276,12 +277,15 @@ int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y
     args.ws = nullptr;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
+    // The caller's events, if any, are bound to the scan kernel itself (its start and end on the GPU).
+    hipEvent_t ev0 = static_cast<hipEvent_t>(start_event), ev1 = static_cast<hipEvent_t>(stop_event);
+    const bool timed = ev0 || ev1;
     auto launch = [&](const ScanArgs &la, const Launch &l) {
         switch (dtype) {
-        case SCANSCAM_F32: return scanscam::launch_scan<float>(la, l, rev, s);
-        case SCANSCAM_BF16: return scanscam::launch_scan<__bf16>(la, l, rev, s);
-        case SCANSCAM_F16: return scanscam::launch_scan<_Float16>(la, l, rev, s);
-        case SCANSCAM_F64: return scanscam::launch_scan<double>(la, l, rev, s);
+        case SCANSCAM_F32: return scanscam::launch_scan<float>(la, l, rev, s, ev0, ev1);
+        case SCANSCAM_BF16: return scanscam::launch_scan<__bf16>(la, l, rev, s, ev0, ev1);
+        case SCANSCAM_F16: return scanscam::launch_scan<_Float16>(la, l, rev, s, ev0, ev1);
+        case SCANSCAM_F64: return scanscam::launch_scan<double>(la, l, rev, s, ev0, ev1);
         default: return hipErrorInvalidValue;
         }
     };
@@ -309,6 +313,8 @@ int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y
     if (r.l.mode == kModeSmall) rows_per_wg = (int64_t)r.l.waves * r.l.unroll * (kWave / r.l.group);
     const int64_t grid_x_all = (n1 + rows_per_wg - 1) / rows_per_wg;
     const int64_t slab_rows = grid_x_all <= max_grid ? n1 : max_grid * rows_per_wg;
+    if (timed && (grid_x_all > max_grid || n0 > 65535 || n0 * grid_x_all > max_grid))
+        return SCANSCAM_EINVAL;  // several launches: one pair of events cannot bracket them
 
     for (int64_t row0 = 0; row0 < n1; row0 += slab_rows) {
         const int64_t n = n1 - row0 < slab_rows ? n1 - row0 : slab_rows;
@@ -528,6 +534,22 @@ size_t scanscam_workspace_bytes_plan(int64_t rows, int64_t T, int dtype, int dir
 {
     (void)direction;
     return workspace_for(rows, T, dtype, plan);
+}
+
+int scanscam_scan_fwd_timed(const void *a, const void *b, void *h, int64_t rows, int64_t T, int dtype,
+                            void *workspace, size_t workspace_bytes, void *stream, const scanscam_plan *plan,
+                            void *start_event, void *stop_event)
+{
+    return run(false, a, b, nullptr, h, nullptr, kDense, 1, rows, T, dtype, workspace, workspace_bytes, stream, plan,
+               start_event, stop_event);
+}
+
+int scanscam_scan_bwd_timed(const void *a, const void *h, const void *gh, void *ga, void *gb, int64_t rows,
+                            int64_t T, int dtype, void *workspace, size_t workspace_bytes, void *stream,
+                            const scanscam_plan *plan, void *start_event, void *stop_event)
+{
+    return run(true, a, gh, h, gb, ga, kDense, 1, rows, T, dtype, workspace, workspace_bytes, stream, plan, start_event,
+               stop_event);
 }
 
 int scanscam_scan_fwd_cl(const void *a, const void *b, void *h, int64_t batch, int64_t T, int64_t C, int dtype,

@@ -1,6 +1,8 @@
 // Host-side launch plumbing shared by the per-dtype translation units.
 #pragma once
 
+#include <hip/hip_ext.h>
+
 #include "scan_cl_kernels.hpp"
 #include "scan_kernels.hpp"
 
@@ -25,22 +27,24 @@ struct Launch {
 constexpr int max_threads_for_unroll(int unroll) { return unroll <= 4 ? 1024 : 256; }
 
 // One per storage type, defined in scan_f32.hip / scan_bf16.hip / scan_f16.hip.
-// Returns hipErrorInvalidValue when (vec, unroll) is not an instantiated pair.
+// Returns hipErrorInvalidValue when (vec, unroll) is not an instantiated pair. `start` / `stop`
+// (may be null) receive the kernel's own start and end time stamps.
 template <typename ST>
-hipError_t launch_scan(const ScanArgs &args, const Launch &l, bool rev, hipStream_t stream);
+hipError_t launch_scan(const ScanArgs &args, const Launch &l, bool rev, hipStream_t stream, hipEvent_t start,
+                       hipEvent_t stop);
 
 #define SCANSCAM_LAUNCH_CASE(ST, VEC, U)                                                             \
     if (l.vec == (VEC) && l.unroll == (U)) {                                                         \
         constexpr int MAXT = max_threads_for_unroll(U);                                              \
         if (l.mode == kModeSmall) {                                                                  \
-            if (rev) hipLaunchKernelGGL((scan_small_kernel<ST, VEC, U, true, MAXT>), grid, block, 0, stream, args);    \
-            else     hipLaunchKernelGGL((scan_small_kernel<ST, VEC, U, false, MAXT>), grid, block, 0, stream, args);   \
+            if (rev) hipExtLaunchKernelGGL((scan_small_kernel<ST, VEC, U, true, MAXT>), grid, block, 0, stream, start, stop, 0, args);    \
+            else     hipExtLaunchKernelGGL((scan_small_kernel<ST, VEC, U, false, MAXT>), grid, block, 0, stream, start, stop, 0, args);   \
         } else if (l.mode == kModeRow) {                                                             \
-            if (rev) hipLaunchKernelGGL((scan_row_kernel<ST, VEC, U, true, MAXT>), grid, block, 0, stream, args);      \
-            else     hipLaunchKernelGGL((scan_row_kernel<ST, VEC, U, false, MAXT>), grid, block, 0, stream, args);     \
+            if (rev) hipExtLaunchKernelGGL((scan_row_kernel<ST, VEC, U, true, MAXT>), grid, block, 0, stream, start, stop, 0, args);      \
+            else     hipExtLaunchKernelGGL((scan_row_kernel<ST, VEC, U, false, MAXT>), grid, block, 0, stream, start, stop, 0, args);     \
         } else {                                                                                     \
-            if (rev) hipLaunchKernelGGL((scan_lookback_kernel<ST, VEC, U, true, MAXT>), grid, block, 0, stream, args); \
-            else     hipLaunchKernelGGL((scan_lookback_kernel<ST, VEC, U, false, MAXT>), grid, block, 0, stream, args);\
+            if (rev) hipExtLaunchKernelGGL((scan_lookback_kernel<ST, VEC, U, true, MAXT>), grid, block, 0, stream, start, stop, 0, args); \
+            else     hipExtLaunchKernelGGL((scan_lookback_kernel<ST, VEC, U, false, MAXT>), grid, block, 0, stream, start, stop, 0, args);\
         }                                                                                            \
         return hipGetLastError();                                                                    \
     }
@@ -50,11 +54,11 @@ hipError_t launch_scan(const ScanArgs &args, const Launch &l, bool rev, hipStrea
     if (l.ragged && l.vec == (VEC) && l.unroll == (U)) {                                             \
         constexpr int MAXT = max_threads_for_unroll(U);                                              \
         if (l.mode == kModeRow) {                                                                    \
-            if (rev) hipLaunchKernelGGL((scan_row_kernel<ST, VEC, U, true, MAXT, true>), grid, block, 0, stream, args);      \
-            else     hipLaunchKernelGGL((scan_row_kernel<ST, VEC, U, false, MAXT, true>), grid, block, 0, stream, args);     \
+            if (rev) hipExtLaunchKernelGGL((scan_row_kernel<ST, VEC, U, true, MAXT, true>), grid, block, 0, stream, start, stop, 0, args);      \
+            else     hipExtLaunchKernelGGL((scan_row_kernel<ST, VEC, U, false, MAXT, true>), grid, block, 0, stream, start, stop, 0, args);     \
         } else if (l.mode == kModeLookback) {                                                        \
-            if (rev) hipLaunchKernelGGL((scan_lookback_kernel<ST, VEC, U, true, MAXT, true>), grid, block, 0, stream, args); \
-            else     hipLaunchKernelGGL((scan_lookback_kernel<ST, VEC, U, false, MAXT, true>), grid, block, 0, stream, args);\
+            if (rev) hipExtLaunchKernelGGL((scan_lookback_kernel<ST, VEC, U, true, MAXT, true>), grid, block, 0, stream, start, stop, 0, args); \
+            else     hipExtLaunchKernelGGL((scan_lookback_kernel<ST, VEC, U, false, MAXT, true>), grid, block, 0, stream, start, stop, 0, args);\
         } else {                                                                                     \
             return hipErrorInvalidValue;                                                             \
         }                                                                                            \
@@ -63,7 +67,8 @@ hipError_t launch_scan(const ScanArgs &args, const Launch &l, bool rev, hipStrea
 
 #define SCANSCAM_DEFINE_LAUNCH(ST)                                                                   \
     template <>                                                                                      \
-    hipError_t launch_scan<ST>(const ScanArgs &args, const Launch &l, bool rev, hipStream_t stream)  \
+    hipError_t launch_scan<ST>(const ScanArgs &args, const Launch &l, bool rev, hipStream_t stream,  \
+                               hipEvent_t start, hipEvent_t stop)                                    \
     {                                                                                                \
         constexpr int FULL = 16 / (int)sizeof(ST);                                                   \
         const dim3 grid((unsigned)l.grid, (unsigned)l.grid_y), block((unsigned)(l.waves * kWave));   \

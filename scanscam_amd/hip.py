@@ -89,6 +89,10 @@ def _bind(path: str) -> ctypes.CDLL:
     lib.scanscam_scan_bwd_plan.restype = i32
     lib.scanscam_workspace_bytes_plan.argtypes = [i64, i64, i32, i32, plan_p]
     lib.scanscam_workspace_bytes_plan.restype = sz
+    lib.scanscam_scan_fwd_timed.argtypes = [p, p, p, i64, i64, i32, p, sz, p, plan_p, p, p]
+    lib.scanscam_scan_fwd_timed.restype = i32
+    lib.scanscam_scan_bwd_timed.argtypes = [p, p, p, p, p, i64, i64, i32, p, sz, p, plan_p, p, p]
+    lib.scanscam_scan_bwd_timed.restype = i32
     lib.scanscam_scan_fwd_cl.argtypes = [p, p, p, i64, i64, i64, i32, p, sz, p, plan_p]
     lib.scanscam_scan_fwd_cl.restype = i32
     lib.scanscam_scan_bwd_cl.argtypes = [p, p, p, p, p, i64, i64, i64, i32, p, sz, p, plan_p]
@@ -228,8 +232,53 @@ def scan_backward_out(gate: torch.Tensor, output: torch.Tensor, out_grad: torch.
         raise RuntimeError(f"scanscam_scan_bwd: {strerror(rc)}")
 
 
+class KernelEvents:
+    """A pair of HIP events for ``prepare_forward`` / ``prepare_backward``: the timed entry points bind
+    them to the scan kernel itself, so ``elapsed_ms()`` is the kernel's duration on the GPU without
+    the launch gaps and event packets that a ``torch.cuda.Event`` pair around a launch includes.
+    The events come straight from the HIP runtime (``libamdhip64``, already loaded by PyTorch).
+    """
+
+    _rt = None
+
+    @classmethod
+    def _runtime(cls):
+        if cls._rt is None:
+            rt = ctypes.CDLL("libamdhip64.so")
+            rt.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+            rt.hipEventDestroy.argtypes = [ctypes.c_void_p]
+            rt.hipEventSynchronize.argtypes = [ctypes.c_void_p]
+            rt.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+            cls._rt = rt
+        return cls._rt
+
+    def __init__(self) -> None:
+        rt = self._runtime()
+        self.start, self.stop = ctypes.c_void_p(), ctypes.c_void_p()
+        for ev in (self.start, self.stop):
+            rc = rt.hipEventCreate(ctypes.byref(ev))
+            if rc != 0:
+                raise RuntimeError(f"hipEventCreate failed with HIP error {rc}")
+
+    def elapsed_ms(self) -> float:
+        """Duration of the last launch that recorded into this pair (waits for it to finish)."""
+        rt = self._runtime()
+        ms = ctypes.c_float()
+        rc = rt.hipEventSynchronize(self.stop) or rt.hipEventElapsedTime(ctypes.byref(ms), self.start, self.stop)
+        if rc != 0:
+            raise RuntimeError(f"HIP event query failed with HIP error {rc}")
+        return float(ms.value)
+
+    def __del__(self) -> None:
+        rt = type(self)._rt
+        if rt is not None:
+            for ev in (self.start, self.stop):
+                if ev:
+                    rt.hipEventDestroy(ev)
+
+
 def prepare_forward(gate: torch.Tensor, value: torch.Tensor, out: torch.Tensor,
-                    plan: Optional[Plan] = None):
+                    plan: Optional[Plan] = None, events: Optional["KernelEvents"] = None):
     """A zero-argument callable that launches this exact forward scan again and again.
 
     All checks, the workspace and the argument marshalling are done once, so a
@@ -237,6 +286,8 @@ def prepare_forward(gate: torch.Tensor, value: torch.Tensor, out: torch.Tensor,
     fixed buffers (benchmarks, a captured step). The tensors and the workspace
     are kept alive by the callable; launches go to the stream that is current
     when it is called, on the device that was current when it was prepared.
+    With ``events`` every launch records the scan kernel's own start and end
+    on the GPU into them (``scanscam_scan_fwd_timed``).
     """
     L = lib()
     _check_rows(gate, value, out)
@@ -245,12 +296,15 @@ def prepare_forward(gate: torch.Tensor, value: torch.Tensor, out: torch.Tensor,
     ws, ws_ptr, ws_n = _workspace(rows, T, gate.dtype, FORWARD, plan, gate.device)
     args = (gate.data_ptr(), value.data_ptr(), out.data_ptr(), rows, T, code, ws_ptr, ws_n)
     plan_ref = ctypes.byref(plan) if plan is not None else None
-    keep = (gate, value, out, ws, plan)
-    fn = L.scanscam_scan_fwd_plan
+    keep = (gate, value, out, ws, plan, events)
     current_stream = torch.cuda.current_stream
+    if events is not None:
+        fn, tail = L.scanscam_scan_fwd_timed, (plan_ref, events.start, events.stop)
+    else:
+        fn, tail = L.scanscam_scan_fwd_plan, (plan_ref,)
 
     def launch(_keep=keep) -> None:
-        rc = fn(*args, current_stream().cuda_stream, plan_ref)
+        rc = fn(*args, current_stream().cuda_stream, *tail)
         if rc != 0:
             raise RuntimeError(f"scanscam_scan_fwd: {strerror(rc)}")
 
@@ -258,7 +312,8 @@ def prepare_forward(gate: torch.Tensor, value: torch.Tensor, out: torch.Tensor,
 
 
 def prepare_backward(gate: torch.Tensor, output: torch.Tensor, out_grad: torch.Tensor,
-                     gate_grad: torch.Tensor, value_grad: torch.Tensor, plan: Optional[Plan] = None):
+                     gate_grad: torch.Tensor, value_grad: torch.Tensor, plan: Optional[Plan] = None,
+                     events: Optional["KernelEvents"] = None):
     """The backward counterpart of ``prepare_forward``."""
     L = lib()
     _check_rows(gate, output, out_grad, gate_grad, value_grad)
@@ -268,12 +323,15 @@ def prepare_backward(gate: torch.Tensor, output: torch.Tensor, out_grad: torch.T
     args = (gate.data_ptr(), output.data_ptr(), out_grad.data_ptr(), gate_grad.data_ptr(),
             value_grad.data_ptr(), rows, T, code, ws_ptr, ws_n)
     plan_ref = ctypes.byref(plan) if plan is not None else None
-    keep = (gate, output, out_grad, gate_grad, value_grad, ws, plan)
-    fn = L.scanscam_scan_bwd_plan
+    keep = (gate, output, out_grad, gate_grad, value_grad, ws, plan, events)
     current_stream = torch.cuda.current_stream
+    if events is not None:
+        fn, tail = L.scanscam_scan_bwd_timed, (plan_ref, events.start, events.stop)
+    else:
+        fn, tail = L.scanscam_scan_bwd_plan, (plan_ref,)
 
     def launch(_keep=keep) -> None:
-        rc = fn(*args, current_stream().cuda_stream, plan_ref)
+        rc = fn(*args, current_stream().cuda_stream, *tail)
         if rc != 0:
             raise RuntimeError(f"scanscam_scan_bwd: {strerror(rc)}")
 

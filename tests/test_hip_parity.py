@@ -534,3 +534,29 @@ def test_more_than_2_pow_32_elements(gpu):
     b_tail[:, 0] += a[4, k] * h[4, k - 1]
     tail = hip.linear_scan_forward(a[4:5, k:].contiguous(), b_tail)
     assert float((tail - h[4:5, k:]).abs().max()) <= 1e-4
+
+
+def test_timed_entry_points(gpu):
+    # The timed variants launch the same kernels (bit-identical results) and leave the kernel's own
+    # duration in the caller's events: positive, and below what the whole call sequence takes.
+    g = torch.Generator(device=gpu).manual_seed(12)
+    for rows, T in [(1024, 4096), (2, 1 << 20), (4096, 64)]:  # row, look-back and small kernels
+        a = torch.rand((rows, T), generator=g, device=gpu)
+        b = torch.randn((rows, T), generator=g, device=gpu)
+        gh = torch.randn((rows, T), generator=g, device=gpu)
+        h, h2 = torch.empty_like(a), torch.empty_like(a)
+        ga, gb, ga2, gb2 = (torch.empty_like(a) for _ in range(4))
+        hip.prepare_forward(a, b, h)()
+        hip.prepare_backward(a, h, gh, ga, gb)()
+        ef, eb = hip.KernelEvents(), hip.KernelEvents()
+        fwd = hip.prepare_forward(a, b, h2, events=ef)
+        bwd = hip.prepare_backward(a, h, gh, ga2, gb2, events=eb)
+        for _ in range(3):
+            fwd()
+            bwd()
+        torch.cuda.synchronize()
+        assert torch.equal(h, h2) and torch.equal(ga, ga2) and torch.equal(gb, gb2)
+        tf, tb = ef.elapsed_ms(), eb.elapsed_ms()
+        print(f"timed [{rows}, {T}]: forward {tf * 1e3:.1f} us, backward {tb * 1e3:.1f} us", flush=True)
+        floor_ms = 12 * rows * T / 8e12 * 1e3  # no kernel is faster than the HBM peak
+        assert floor_ms <= tf < 5.0 and 20 / 12 * floor_ms <= tb < 5.0
