@@ -11,6 +11,7 @@
 #include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
+#include <string.h>
 
 #include "scanscam_hip.h"
 
@@ -123,6 +124,44 @@ static int check_case(const char *name, long rows, long T, long C, int channels_
            ws_bytes, eh, egb, ega);
     /* gates and values in [0,1) x [-1,1): |h|, |grad_b| stay small, so 1e-5 (2e-5 for the product) is ample */
     if (!(eh <= 1e-5) || !(egb <= 1e-5) || !(ega <= 2e-5)) failures++;
+
+    if (!channels_last) {
+        /* The same launch through the _plan and _timed variants: a resolved plan handed back in gives
+         * bit-identical output, and the caller's events hold the kernel's own duration. */
+        scanscam_plan plan;
+        hipEvent_t ev0, ev1;
+        float ms = -1.0f;
+        HIP_OK(hipEventCreate(&ev0));
+        HIP_OK(hipEventCreate(&ev1));
+        float *again = (float *)malloc(n * 4);
+        if (scanscam_resolve_plan(rows, T, SCANSCAM_F32, SCANSCAM_FORWARD, NULL, &plan) != SCANSCAM_OK) failures++;
+        if (scanscam_workspace_bytes_plan(rows, T, SCANSCAM_F32, SCANSCAM_FORWARD, &plan) > ws_bytes) failures++;
+        HIP_OK(hipMemset(o0, 0, n * 4));
+        if (scanscam_scan_fwd_plan(da, db, o0, rows, T, SCANSCAM_F32, ws, ws_bytes, stream, &plan) != SCANSCAM_OK) failures++;
+        HIP_OK(hipStreamSynchronize(stream));
+        HIP_OK(hipMemcpy(again, o0, n * 4, hipMemcpyDeviceToHost));
+        HIP_OK(hipMemset(o0, 0, n * 4));
+        if (scanscam_scan_fwd_timed(da, db, o0, rows, T, SCANSCAM_F32, ws, ws_bytes, stream, &plan, ev0, ev1) != SCANSCAM_OK)
+            failures++;
+        HIP_OK(hipEventSynchronize(ev1));
+        HIP_OK(hipEventElapsedTime(&ms, ev0, ev1));
+        HIP_OK(hipMemcpy(got, o0, n * 4, hipMemcpyDeviceToHost));
+        if (memcmp(got, again, n * 4) != 0 || worst(got, h, n) > 1e-5 || !(ms > 0.0f && ms < 100.0f)) failures++;
+        if (scanscam_scan_bwd_plan(da, dh, dgh, o1, o0, rows, T, SCANSCAM_F32, ws, ws_bytes, stream, NULL) != SCANSCAM_OK)
+            failures++;
+        HIP_OK(hipStreamSynchronize(stream));
+        HIP_OK(hipMemcpy(again, o0, n * 4, hipMemcpyDeviceToHost));
+        if (scanscam_scan_bwd_timed(da, dh, dgh, o1, o0, rows, T, SCANSCAM_F32, ws, ws_bytes, stream, NULL, ev0, ev1) !=
+            SCANSCAM_OK)
+            failures++;
+        HIP_OK(hipEventSynchronize(ev1));
+        HIP_OK(hipMemcpy(got, o0, n * 4, hipMemcpyDeviceToHost));
+        if (memcmp(got, again, n * 4) != 0 || worst(got, gb, n) > 1e-5) failures++;
+        printf("abi_check: %-28s _plan and _timed variants agree; forward kernel %.1f us\n", name, ms * 1e3);
+        free(again);
+        HIP_OK(hipEventDestroy(ev0));
+        HIP_OK(hipEventDestroy(ev1));
+    }
 
     hipFree(da); hipFree(db); hipFree(dgh); hipFree(dh); hipFree(o0); hipFree(o1);
     if (ws) hipFree(ws);
