@@ -98,8 +98,9 @@ int scanscam_scan_bwd(const void *a, const void *h, const void *gh, void *ga, vo
                       int64_t T, int dtype, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
- * Bytes of device workspace the two calls above need for this shape (0 for
- * most shapes; non-zero when long rows are split over workgroups). The
+ * Bytes of device workspace the call above of that direction needs for this
+ * shape (0 for most shapes; non-zero when rows are split over workgroups, which
+ * the two directions decide separately). The
  * reference's kernels need none, so this has no counterpart there. The
  * workspace need not be initialised; its contents are clobbered. Two calls
  * that may overlap in time need separate workspaces.

@@ -63,13 +63,39 @@ struct Resolved {
     int nch;
     int tiles_per_row;
     int counters;
+    int row_major;       // a counter's tickets walk its rows one after the other (see resolve)
     int64_t super_base;  // word offset of the super-tile descriptors
     size_t ws_bytes;
 };
 
-// Turns (shape, alignment, optional user plan) into a launch. `aligned16` says
+// Look-back tiles in chunks (8 waves x 4 chunks per wave) and the ticket order of the look-back kernel.
+// Tile-major: a counter's tickets visit tile 0 of each of its rows, then tile 1 of each, ...; few tiles of a
+// row are in flight together, so carries arrive with little waiting, at the price of as many separate spans of
+// memory being streamed at once as there are rows. Row-major: a counter's tickets finish one row before the
+// next, so the tiles in flight sweep memory in address order, which the memory system serves 5-8 points
+// faster (stream_probe order), while all tiles of a row are in flight together and wait for each other:
+// worth it when a row is only a few tiles long.
+constexpr int kTileChunks = 32;
+constexpr int kRowMajorCounters = 4;
+
+bool row_major_order(int64_t rows, int tiles_per_row) { return rows >= 256 && tiles_per_row <= 16; }
+
+// Many rows of moderate length: from two tiles per row on, the look-back kernel in row-major order beats one
+// workgroup walking each row, which streams as many separate spans as there are rows in flight and whose
+// last round of workgroups leaves CUs idle. Measured at 16 M to 64 M elements, 4-byte storage: backward +3 to
+// +12 points for 2 to 16 tiles per row, forward +1 to +8 for 2 to 14 (at 16 the forward pass loses); 16-bit
+// storage: backward +4 to +8 up to 8 tiles, forward nothing beyond 4. A problem of fewer than 2048 tiles is too
+// small to hide the extra launch that clears the workspace.
+bool prefer_row_major_lookback(int64_t rows, int nch, bool rev, int esize)
+{
+    const int tpr = (nch + kTileChunks - 1) / kTileChunks;
+    const int longest = rev ? (esize == 2 ? 8 : 16) : (esize == 2 ? 4 : 14);
+    return rows >= 256 && tpr >= 2 && tpr <= longest && rows * tpr >= 2048;
+}
+
+// Turns (shape, alignment, direction, optional user plan) into a launch. `aligned16` says
 // whether every tensor base is 16-byte aligned.
-int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool aligned16, Resolved *out)
+int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool aligned16, bool rev, Resolved *out)
 {
     const int esize = elem_size(dtype);
     if (esize == 0) return SCANSCAM_EDTYPE;
@@ -95,6 +121,7 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
     out->nch = nch;
     out->tiles_per_row = 0;
     out->counters = 1;
+    out->row_major = 0;
     out->super_base = 0;
     out->ws_bytes = 0;
     if (rows == 0 || T == 0) return SCANSCAM_OK;
@@ -105,6 +132,7 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
         // From 256 rows on, one 16-wave workgroup per row fills the chip as well as tiles over
         // workgroups do and needs no carry hand-off between workgroups.
         else if (nch >= 64 && rows < 256) l.mode = kModeLookback;
+        else if (prefer_row_major_lookback(rows, nch, rev, esize)) l.mode = kModeLookback;
         else l.mode = kModeRow;
     }
 
@@ -159,6 +187,9 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
         // One ticket counter per row up to kMaxCounters; when rows do not divide
         // evenly every counter gets the grid share of the fullest one.
         out->counters = (int)(rows < kMaxCounters ? rows : kMaxCounters);
+        // Row-major order: a few counters, so that their rows stay neighbours in memory.
+        out->row_major = row_major_order(rows, out->tiles_per_row) ? 1 : 0;
+        if (out->row_major) out->counters = kRowMajorCounters;
         const int64_t rows_per_counter = (rows + out->counters - 1) / out->counters;
         const int64_t tiles = rows * (int64_t)out->tiles_per_row;
         l.grid = (int64_t)out->counters * rows_per_counter * out->tiles_per_row;
@@ -250,7 +281,7 @@ int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y
     }
 
     Resolved r;
-    const int rc = resolve(plan, rows, T, dtype, aligned16, &r);
+    const int rc = resolve(plan, rows, T, dtype, aligned16, rev, &r);
     if (rc != SCANSCAM_OK) return rc;
 
     ScanArgs args;
@@ -271,6 +302,7 @@ int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y
     args.group = r.l.group;
     args.tiles_per_row = r.tiles_per_row;
     args.counters = r.counters;
+    args.row_major = r.row_major;
     args.desc_base = r.counters * kCounterStride;
     args.super_base = r.super_base;
     args.spin_limit = (plan && plan->spin_limit > 0) ? plan->spin_limit : scanscam::kSpinLimit;
@@ -482,14 +514,15 @@ int run_cl(bool rev, const void *a, const void *x, const void *h, void *y0, void
     return e == hipSuccess ? SCANSCAM_OK : SCANSCAM_ELAUNCH;
 }
 
-size_t workspace_for(int64_t rows, int64_t T, int dtype, const scanscam_plan *plan)
+size_t workspace_for(int64_t rows, int64_t T, int dtype, int direction, const scanscam_plan *plan)
 {
     // The caller's pointers are not known yet: cover both the 16-byte aligned
     // and the unaligned choice.
     size_t need = 0;
     for (int al = 0; al < 2; al++) {
         Resolved r;
-        if (resolve(plan, rows, T, dtype, al != 0, &r) == SCANSCAM_OK && r.ws_bytes > need) need = r.ws_bytes;
+        if (resolve(plan, rows, T, dtype, al != 0, direction == SCANSCAM_BACKWARD, &r) == SCANSCAM_OK && r.ws_bytes > need)
+            need = r.ws_bytes;
     }
     return need;
 }
@@ -512,8 +545,7 @@ int scanscam_scan_bwd(const void *a, const void *h, const void *gh, void *ga, vo
 
 size_t scanscam_workspace_bytes(int64_t rows, int64_t T, int dtype, int direction)
 {
-    (void)direction;
-    return workspace_for(rows, T, dtype, nullptr);
+    return workspace_for(rows, T, dtype, direction, nullptr);
 }
 
 int scanscam_scan_fwd_plan(const void *a, const void *b, void *h, int64_t rows, int64_t T, int dtype,
@@ -532,8 +564,7 @@ int scanscam_scan_bwd_plan(const void *a, const void *h, const void *gh, void *g
 size_t scanscam_workspace_bytes_plan(int64_t rows, int64_t T, int dtype, int direction,
                                      const scanscam_plan *plan)
 {
-    (void)direction;
-    return workspace_for(rows, T, dtype, plan);
+    return workspace_for(rows, T, dtype, direction, plan);
 }
 
 int scanscam_scan_fwd_timed(const void *a, const void *b, void *h, int64_t rows, int64_t T, int dtype,
@@ -619,10 +650,9 @@ int scanscam_scan_bwd_cl_strided(const void *a, const void *h, const void *gh, v
 int scanscam_resolve_plan(int64_t rows, int64_t T, int dtype, int direction, const scanscam_plan *plan,
                           scanscam_plan *out)
 {
-    (void)direction;
     if (!out) return SCANSCAM_EINVAL;
     Resolved r;
-    const int rc = resolve(plan, rows, T, dtype, true, &r);
+    const int rc = resolve(plan, rows, T, dtype, true, direction == SCANSCAM_BACKWARD, &r);
     if (rc != SCANSCAM_OK) return rc;
     out->mode = r.l.mode;
     out->vec = r.l.vec;

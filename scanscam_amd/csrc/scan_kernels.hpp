@@ -71,6 +71,7 @@ struct ScanArgs {
     int32_t group;          // SMALL: lanes per row (power of two, <= 64)
     int32_t tiles_per_row;  // LOOKBACK: tiles per row
     int32_t counters;       // LOOKBACK: number of ticket counters (row r uses counter r % counters)
+    int32_t row_major;      // LOOKBACK: a counter's tickets walk its rows one after the other
     int32_t desc_base;      // LOOKBACK: first tile-descriptor word of the workspace
     int64_t super_base;     // LOOKBACK: first super-tile-descriptor word of the workspace
     int32_t spin_limit;     // LOOKBACK: polls before a wait gives up
@@ -583,9 +584,16 @@ __global__ __launch_bounds__(MAXT) void scan_small_kernel(const ScanArgs p)
 // handed out by atomic tickets, so every tile a workgroup may wait for was
 // taken by a workgroup that is already running. A single counter would
 // serialise the whole grid on one address, so there are up to kMaxCounters of
-// them, each serving the rows r with r % counters == c: ticket k of a counter
-// works on its (k % rows_here)-th row, tile k / rows_here, which keeps the
-// tiles in flight at any moment spread over all rows.
+// them, each serving the rows r with r % counters == c. In tile-major order
+// ticket k of a counter works on its (k % rows_here)-th row, tile k / rows_here,
+// which keeps the tiles in flight at any moment spread over all rows: few
+// neighbours wait for each other. In row-major order (p.row_major, chosen by the
+// host for many rows of a few tiles each, with few counters) ticket k works on
+// tile k % tiles_per_row of the counter's (k / tiles_per_row)-th row, so the
+// tiles in flight cover consecutive rows: one sweep through memory in address
+// order, which the memory system serves faster than many separate spans.
+// Either way a tile only ever waits for tiles of its own row with smaller
+// tickets of the same counter.
 //
 // Carry protocol, two levels, run by wave 0 of the workgroup. 64 consecutive
 // tiles of a row form a super-tile. Let (A_q, B_q) be the aggregate of tile q
@@ -763,7 +771,7 @@ __global__ __launch_bounds__(MAXT) void scan_lookback_kernel(const ScanArgs p)
     const int nwaves = blockDim.x / kWave;
 
     // Counter c serves the rows r with r % counters == c; its tickets walk those
-    // rows round-robin, tile by tile.
+    // rows round-robin, tile by tile, or one row after the other.
     const int nctr = p.counters;
     const int ctr = blockIdx.x % nctr;
     if (threadIdx.x == 0)
@@ -773,8 +781,15 @@ __global__ __launch_bounds__(MAXT) void scan_lookback_kernel(const ScanArgs p)
     const unsigned ticket = __builtin_amdgcn_readfirstlane(lds_ticket);
     const int64_t rows_here = (p.rows - ctr + nctr - 1) / nctr;
     if ((int64_t)ticket >= rows_here * p.tiles_per_row) return;  // surplus workgroup of an uneven split
-    const int64_t row = ctr + (int64_t)nctr * (ticket % (uint64_t)rows_here);
-    const int tile = (int)(ticket / (uint64_t)rows_here);
+    int64_t row;
+    int tile;
+    if (p.row_major) {
+        row = ctr + (int64_t)nctr * (int64_t)(ticket / (unsigned)p.tiles_per_row);
+        tile = (int)(ticket % (unsigned)p.tiles_per_row);
+    } else {
+        row = ctr + (int64_t)nctr * (int64_t)(ticket % (uint64_t)rows_here);
+        tile = (int)(ticket / (uint64_t)rows_here);
+    }
     const int nvp = p.nch * kWave;
     const int chunk0 = (tile * nwaves + wave) * U;
 

@@ -298,21 +298,27 @@ def test_short_rows_automatic(gpu, rows, T):
 
 
 # One shape per branch of the automatic plan for rows longer than a chunk: (rows, T) -> the
-# (mode, waves per row, chunks per wave) the library reports for it.
+# (mode, waves per row, chunks per wave) the library reports for it, forward and backward.
+ROW, LOOKBACK = hip.MODE_ROW, hip.MODE_LOOKBACK
 AUTO_REGIMES = [
-    (2048, 1280, (hip.MODE_ROW, 4, 2)),
-    (2048, 4100, (hip.MODE_ROW, 8, 4)),       # 17 chunks: one step of an 8-wave tile
-    (2048, 12501, (hip.MODE_ROW, 16, 4)),     # 49 chunks, element-aligned rows
-    (300, 4100, (hip.MODE_ROW, 16, 1)),
-    (300, 16640, (hip.MODE_ROW, 16, 4)),      # few rows, 65 chunks
-    (255, 16640, (hip.MODE_LOOKBACK, 0, 4)),
+    (2048, 1280, (ROW, 4, 2), None),
+    (2048, 4100, (ROW, 8, 4), None),          # 17 chunks: one step of an 8-wave tile
+    (2048, 12501, (LOOKBACK, 0, 4), None),    # 49 chunks = 2 tiles, element-aligned rows: tiles in row-major order
+    (700, 20000, (LOOKBACK, 0, 4), None),     # 3 tiles per row, 2100 tiles
+    (256, 131072, (ROW, 16, 4), (LOOKBACK, 0, 4)),  # 16 tiles per row: only the backward pass gains
+    (600, 20000, (ROW, 16, 4), None),         # 1800 tiles: too small a problem for the look-back launch
+    (300, 4100, (ROW, 16, 1), None),
+    (300, 16640, (ROW, 16, 4), None),         # few rows, 65 chunks
+    (255, 16640, (LOOKBACK, 0, 4), None),     # fewer than 256 rows: tiles in tile-major order
 ]
 
 
-@pytest.mark.parametrize("rows,T,expect", AUTO_REGIMES)
-def test_automatic_plan_regimes(gpu, rows, T, expect):
+@pytest.mark.parametrize("rows,T,expect,expect_bwd", AUTO_REGIMES)
+def test_automatic_plan_regimes(gpu, rows, T, expect, expect_bwd):
     plan = hip.resolve_plan(rows, T, torch.float32, hip.FORWARD)
     assert (plan.mode, plan.waves_per_row, plan.unroll) == expect, plan
+    plan = hip.resolve_plan(rows, T, torch.float32, hip.BACKWARD)
+    assert (plan.mode, plan.waves_per_row, plan.unroll) == (expect_bwd or expect), plan
     g = seeded(rows + T)
     a = torch.rand((rows, T), generator=g)
     b = torch.randn((rows, T), generator=g)
@@ -560,3 +566,42 @@ def test_timed_entry_points(gpu):
         print(f"timed [{rows}, {T}]: forward {tf * 1e3:.1f} us, backward {tb * 1e3:.1f} us", flush=True)
         floor_ms = 12 * rows * T / 8e12 * 1e3  # no kernel is faster than the HBM peak
         assert floor_ms <= tf < 5.0 and 20 / 12 * floor_ms <= tb < 5.0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16, torch.float16])
+def test_lookback_row_major_ticket_order(gpu, dtype):
+    # From 256 rows on, rows of at most 16 tiles are handed out row after row by 4 ticket counters
+    # (rows of one counter are 4 apart). Forced here with small tiles: whole and partial last tiles,
+    # element-aligned rows, a row count that the counters do not divide, and two-level strided views.
+    full = full_vec(dtype)
+    bar = bar_for(dtype)
+    g = seeded(17)
+    chunk = 64 * full
+    for rows, T, unroll, waves in [(259, 11 * chunk + 3, 2, 1), (257, 16 * chunk, 1, 1), (300, 7 * 8 * chunk - full, 2, 4),
+                                   (256, 2 * 16 * chunk, 4, 4)]:
+        plan = hip.Plan(mode=hip.MODE_LOOKBACK, vec=full, unroll=unroll, waves=waves)
+        a = torch.rand((rows, T), generator=g, dtype=torch.float64).to(dtype)
+        b = torch.randn((rows, T), generator=g, dtype=torch.float64).to(dtype)
+        gh = torch.randn((rows, T), generator=g, dtype=torch.float64).to(dtype)
+        print(f"case row-major {dtype} rows={rows} T={T} {plan}", flush=True)
+        h = oracle.fwd(upcast(a), upcast(b))
+        got = run_fwd(gpu, a, b, plan)
+        assert rel_err(to_np(got), h) <= bar
+        ga, gb = oracle.bwd(upcast(a), upcast(got.cpu()), upcast(gh))
+        got_ga, got_gb = run_bwd(gpu, a, got, gh, plan)
+        assert rel_err(to_np(got_gb), gb) <= bar
+        assert rel_err(to_np(got_ga), ga, prev_abs(to_np(got))) <= bar
+    # halves of x[3, 2*90, T]: 270 rows in two levels
+    T = 6 * chunk
+    x = torch.randn((3, 180, T), generator=g, dtype=torch.float64)
+    x[:, :90] = torch.sigmoid(x[:, :90])
+    x = x.to(dtype).to(gpu)
+    a, b = x.chunk(2, dim=1)
+    plan = hip.Plan(mode=hip.MODE_LOOKBACK, vec=full, unroll=1, waves=1)
+    got = hip.scan_forward(a, b, plan)
+    h = oracle.fwd(upcast(a.cpu()), upcast(b.cpu()))
+    assert rel_err(to_np(got), h) <= bar
+    ga, gb = oracle.bwd(upcast(a.cpu()), upcast(got.cpu()), upcast(b.cpu()))
+    got_ga, got_gb = hip.scan_backward(a, got, b, plan)
+    assert rel_err(to_np(got_gb), gb) <= bar
+    assert rel_err(to_np(got_ga), ga, prev_abs(to_np(got))) <= bar
