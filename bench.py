@@ -22,6 +22,7 @@ Prints ONE JSON line. Besides the contract fields it carries
   cpu_baseline  the reference's single-threaded CPU loop on the same tensors,
                 timed on this host (oracle/_ref if it was built, else the C
                 restatement in oracle/);
+  long_rows     many rows of 16K to 96K elements (long-context shapes);
   configs       forward and forward+backward GB/s of the other four synthetic
                 configurations (buffer sets rotated so that the 256 MB
                 Infinity Cache cannot serve them; timed as batches of
@@ -212,6 +213,37 @@ def reference_grid(dev, args, hip, torch):
         "fwd_GBps": round(12 * n / (times[0] * 1e-3) / 1e9, 1), "bwd_GBps": round(20 * n / (times[1] * 1e-3) / 1e9, 1),
         "note": "includes the wrapper's output allocation; working set fits the Infinity Cache",
     }
+    return out
+
+
+def long_rows(dev, args, hip, torch):
+    """Many rows of 8K to 128K elements (long-context shapes), 64 M elements each, fp32 and bf16.
+
+    From two tiles per row on these run on the look-back kernel with its tiles handed out row after row;
+    mean microseconds per launch over back-to-back launches (each tensor is 268 MB / 134 MB, beyond the
+    Infinity Cache).
+    """
+    out = {}
+    for dtype in (torch.float32, torch.bfloat16):
+        for rows, T in ((4096, 16384), (2048, 32768), (1365, 49152), (682, 98304)):
+            g = torch.Generator(device=dev).manual_seed(0)
+            a = torch.rand((rows, T), generator=g, device=dev).to(dtype)
+            b = torch.randn((rows, T), generator=g, device=dev).to(dtype)
+            gh = torch.randn((rows, T), generator=g, device=dev).to(dtype)
+            s = object.__new__(DeviceSet)
+            s.a, s.b, s.gh = a, b, gh
+            s.h, s.ga, s.gb = (torch.empty_like(a) for _ in range(3))
+            f_ms, b_ms = time_batches([s], max(20, args.steps // 2), max(3, args.warmup // 2), hip, torch)
+            n, esize = a.numel(), a.element_size()
+            out[f"{rows}x{T}_{str(dtype).replace('torch.', '')}"] = {
+                "fwd_us": round(f_ms * 1e3, 1), "bwd_us": round(b_ms * 1e3, 1),
+                "fwd_frac": round(FWD_BYTES[esize] * n / (f_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                "bwd_frac": round(BWD_BYTES[esize] * n / (b_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                "plan_fwd": repr(hip.resolve_plan(rows, T, dtype, hip.FORWARD)),
+                "plan_bwd": repr(hip.resolve_plan(rows, T, dtype, hip.BACKWARD)),
+            }
+            del s, a, b, gh
+            torch.cuda.empty_cache()
     return out
 
 
@@ -451,6 +483,7 @@ def main():
     if not args.no_configs:
         out["reference_grid"] = reference_grid(dev, args, hip, torch)
         out["strided_views"] = strided_views(dev, args, hip, torch)
+        out["long_rows"] = long_rows(dev, args, hip, torch)
 
     if not args.no_cpu:
         # 16-bit workloads: the reference has no 16-bit path, so its loop runs on the exact fp32 upcast.

@@ -82,15 +82,21 @@ bool row_major_order(int64_t rows, int tiles_per_row) { return rows >= 256 && ti
 
 // Many rows of moderate length: from two tiles per row on, the look-back kernel in row-major order beats one
 // workgroup walking each row, which streams as many separate spans as there are rows in flight and whose
-// last round of workgroups leaves CUs idle. Measured at 16 M to 64 M elements, 4-byte storage: backward +3 to
-// +12 points for 2 to 16 tiles per row, forward +1 to +8 for 2 to 14 (at 16 the forward pass loses); 16-bit
-// storage: backward +4 to +8 up to 8 tiles, forward nothing beyond 4. A problem of fewer than 2048 tiles is too
-// small to hide the extra launch that clears the workspace.
+// last round of workgroups leaves CUs idle. Measured at 16 M to 64 M elements: the backward pass gains +2 to
+// +15 points of peak for 2 to 16 tiles per row, whatever the storage type; the forward pass +1 to +8 up to 6
+// tiles (4 for 16-bit storage, nothing lost), and beyond that, up to 14 tiles, only where the row kernel's
+// 16-wave workgroups (one per CU) do not come out in full rounds (rows = 512 or 1024 do: there it keeps the
+// forward pass). A problem of fewer than 2048 tiles is too small to hide the extra launch that clears the
+// workspace.
+constexpr int kComputeUnits = 256;  // MI355X
+
 bool prefer_row_major_lookback(int64_t rows, int nch, bool rev, int esize)
 {
     const int tpr = (nch + kTileChunks - 1) / kTileChunks;
-    const int longest = rev ? (esize == 2 ? 8 : 16) : (esize == 2 ? 4 : 14);
-    return rows >= 256 && tpr >= 2 && tpr <= longest && rows * tpr >= 2048;
+    if (rows < 256 || tpr < 2 || tpr > 16 || rows * tpr < 2048) return false;
+    if (rev || tpr <= (esize == 2 ? 4 : 6)) return true;
+    const int64_t rounds = (rows + kComputeUnits - 1) / kComputeUnits;
+    return tpr <= 14 && rows * 100 < rounds * kComputeUnits * 93;  // last round less than 93 % useful overall
 }
 
 // Turns (shape, alignment, direction, optional user plan) into a launch. `aligned16` says

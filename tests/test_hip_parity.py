@@ -307,6 +307,8 @@ AUTO_REGIMES = [
     (700, 20000, (LOOKBACK, 0, 4), None),     # 3 tiles per row, 2100 tiles
     (256, 131072, (ROW, 16, 4), (LOOKBACK, 0, 4)),  # 16 tiles per row: only the backward pass gains
     (600, 20000, (ROW, 16, 4), None),         # 1800 tiles: too small a problem for the look-back launch
+    (300, 81920, (LOOKBACK, 0, 4), None),     # 10 tiles per row, and 300 rows fill 256 CUs 1.17 times: forward too
+    (512, 81920, (ROW, 16, 4), (LOOKBACK, 0, 4)),  # two full rounds of row workgroups: the forward pass keeps them
     (300, 4100, (ROW, 16, 1), None),
     (300, 16640, (ROW, 16, 4), None),         # few rows, 65 chunks
     (255, 16640, (LOOKBACK, 0, 4), None),     # fewer than 256 rows: tiles in tile-major order
