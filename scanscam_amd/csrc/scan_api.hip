@@ -87,16 +87,20 @@ bool row_major_order(int64_t rows, int tiles_per_row) { return rows >= 256 && ti
 // tiles (4 for 16-bit storage, nothing lost), and beyond that, up to 14 tiles, only where the row kernel's
 // 16-wave workgroups (one per CU) do not come out in full rounds (rows = 512 or 1024 do: there it keeps the
 // forward pass). A problem of fewer than 2048 tiles is too small to hide the extra launch that clears the
-// workspace.
+// workspace. Rows of more than 16 tiles go to the look-back kernel (in tile-major order) only where the row
+// kernel's rounds do not come out.
 constexpr int kComputeUnits = 256;  // MI355X
 
-bool prefer_row_major_lookback(int64_t rows, int nch, bool rev, int esize)
+bool prefer_lookback_for_many_rows(int64_t rows, int nch, bool rev, int esize)
 {
     const int tpr = (nch + kTileChunks - 1) / kTileChunks;
-    if (rows < 256 || tpr < 2 || tpr > 16 || rows * tpr < 2048) return false;
-    if (rev || tpr <= (esize == 2 ? 4 : 6)) return true;
+    if (rows < 256 || tpr < 2 || rows * tpr < 2048) return false;
     const int64_t rounds = (rows + kComputeUnits - 1) / kComputeUnits;
-    return tpr <= 14 && rows * 100 < rounds * kComputeUnits * 93;  // last round less than 93 % useful overall
+    const bool ragged_rounds = rows * 100 < rounds * kComputeUnits * 93;  // the row kernel's CUs idle > 7 % of the time
+    // Longer rows (tile-major order): only where the row kernel's rounds do not come out (+2 to +13 points).
+    if (tpr > 16) return ragged_rounds;
+    if (rev || tpr <= (esize == 2 ? 4 : 6)) return true;
+    return tpr <= 14 && ragged_rounds;
 }
 
 // Turns (shape, alignment, direction, optional user plan) into a launch. `aligned16` says
@@ -138,7 +142,7 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
         // From 256 rows on, one 16-wave workgroup per row fills the chip as well as tiles over
         // workgroups do and needs no carry hand-off between workgroups.
         else if (nch >= 64 && rows < 256) l.mode = kModeLookback;
-        else if (prefer_row_major_lookback(rows, nch, rev, esize)) l.mode = kModeLookback;
+        else if (prefer_lookback_for_many_rows(rows, nch, rev, esize)) l.mode = kModeLookback;
         else l.mode = kModeRow;
     }
 

@@ -310,6 +310,7 @@ AUTO_REGIMES = [
     (300, 81920, (LOOKBACK, 0, 4), None),     # 10 tiles per row, and 300 rows fill 256 CUs 1.17 times: forward too
     (512, 81920, (ROW, 16, 4), (LOOKBACK, 0, 4)),  # two full rounds of row workgroups: the forward pass keeps them
     (300, 4100, (ROW, 16, 1), None),
+    (270, 140000, (LOOKBACK, 0, 4), None),    # 18 tiles per row, 270 rows on 256 CUs: tile-major look-back
     (300, 16640, (ROW, 16, 4), None),         # few rows, 65 chunks
     (255, 16640, (LOOKBACK, 0, 4), None),     # fewer than 256 rows: tiles in tile-major order
 ]
