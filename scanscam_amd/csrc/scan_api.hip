@@ -399,9 +399,12 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         l->vec = 1;
     } else {
         // A workgroup owns 64*vec channels of one batch element. Enough of them: 16-byte loads.
-        // Not enough, but enough with one channel per lane: narrower loads beat a second pass
-        // over the data. Fewer still: 16-byte loads and time split over workgroups (below).
-        l->vec = (batch * groups(full) >= 256 || batch * groups(1) < 256) ? full : 1;
+        // Not enough: one channel per lane, which gives full/1 times as many workgroups; if even those
+        // are too few, time is split over workgroups as well (below), and there too the narrow lanes
+        // win: more, narrower carry chains (fp32 1.1-1.7 times faster than 16-byte lanes, measured from
+        // [1, 262144, 256] to [8, 4096, 512]; 16-bit storage 2.5-16 times, its 16-byte lanes leave
+        // 8 times fewer chains).
+        l->vec = batch * groups(full) >= 256 ? full : 1;
     }
     if (l->vec != 1 && l->vec != full) return SCANSCAM_EPLAN;
     if (l->vec == full && full != 1 && !vec_possible) return SCANSCAM_EPLAN;
@@ -414,7 +417,9 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     if (u.mode == kModeLookback || (u.mode == SCANSCAM_MODE_AUTO && rowgroups < 256)) l->kind = 2;
     if (u.mode == kModeSmall) return SCANSCAM_EPLAN;
 
-    l->steps = u.unroll ? u.unroll : (l->vec == 1 || (l->kind != 0 && full <= 4) ? 8 : 4);
+    // Steps per wave per tile: with one channel per lane and tiles over workgroups, 16 (8 measured 1.2-1.4
+    // times slower: twice as many tiles pay the carry wait).
+    l->steps = u.unroll ? u.unroll : (l->vec == 1 ? (l->kind != 0 ? 16 : 8) : ((l->kind != 0 && full <= 4) ? 8 : 4));
     const bool steps_ok = (l->vec == full) ? (l->steps == 2 || l->steps == 4 || l->steps == 8)
                                            : (l->steps == 4 || l->steps == 8 || l->steps == 16);
     if (!steps_ok) return SCANSCAM_EPLAN;
@@ -432,7 +437,9 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     } else {
         const int64_t segments = (T + l->steps - 1) / l->steps;  // no more waves than segments of time
         l->waves = segments < max_waves ? pow2_ceil(segments) : max_waves;
-        if (l->kind != 0 && l->waves > 8) l->waves = 8;  // shorter tiles: more of them to hand out
+        // Tiles over workgroups: 8 waves (shorter tiles, more of them to hand out), 16 when there are very
+        // few carry chains to spread the workgroups over.
+        if (l->kind != 0 && l->waves > 8 && rowgroups > 16) l->waves = 8;
         while (l->waves > max_waves) l->waves >>= 1;
     }
     if (l->waves < 1 || l->waves > max_waves) return SCANSCAM_EPLAN;
