@@ -140,8 +140,10 @@ int scanscam_scan_bwd_timed(const void *a, const void *h, const void *gh, void *
  * output, outGrad, gateGradOut, valueGradOut, channelsPerBlock), :687-723. The
  * reference's trailing tuning argument has its counterpart in `plan` (NULL =
  * automatic): vec = channels per lane (16/sizeof(storage) or 1), unroll = time
- * steps per wave per tile (2, 4, 8 for the full vector; 4, 8, 16 for vec 1),
- * waves = waves per workgroup (1..16). When batch * C is too small to fill the
+ * steps per wave per tile (2, 4, 8 for the full vector; 4, 8, 16 for vec 1;
+ * with at most 32 * vec channels a wave holds several time steps per load and
+ * `unroll` counts those loads), waves = waves per workgroup (1..16). When
+ * batch * C is too small to fill the
  * GPU, time is also cut into tiles over workgroups, carried by a look-back
  * chain, which needs a workspace (scanscam_workspace_bytes_cl, same rules as
  * above); mode = SCANSCAM_MODE_ROW forbids that split, SCANSCAM_MODE_LOOKBACK

@@ -405,6 +405,11 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         // [1, 262144, 256] to [8, 4096, 512]; 16-bit storage 2.5-16 times, its 16-byte lanes leave
         // 8 times fewer chains).
         l->vec = batch * groups(full) >= 256 ? full : 1;
+        // Few channels (the packed kernel, below): a wide lane leaves more steps per instruction to scan
+        // across with lane shuffles, which costs more than the wider loads gain -- except where C is not a
+        // power of two and one channel per lane would leave a quarter of 32 lanes idle (fp32 [256, 8192, 24]:
+        // 177 / 235 us with 16-byte lanes, 209 / 320 with 4-byte lanes; [512, 4096, 8]: 66 / 80 against 44 / 67).
+        if (C <= 32 && (esize == 2 || pow2_ceil(C) <= 16 || is_pow2((int)C))) l->vec = 1;
     }
     if (l->vec != 1 && l->vec != full) return SCANSCAM_EPLAN;
     if (l->vec == full && full != 1 && !vec_possible) return SCANSCAM_EPLAN;
@@ -419,7 +424,16 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
 
     // Steps per wave per tile: with one channel per lane and tiles over workgroups, 16 (8 measured 1.2-1.4
     // times slower: twice as many tiles pay the carry wait).
+    // Few channels: a time step fills `group` lanes only, and a wave holds 64 / group consecutive steps
+    // per instruction (the packed kernel; a workgroup then owns a whole batch element).
+    l->group = kWave;
+    if (l->kind == 0 && groups(l->vec) == 1) {
+        const int g = pow2_ceil((C + l->vec - 1) / l->vec);
+        if (g < kWave) l->group = g;
+    }
+
     l->steps = u.unroll ? u.unroll : (l->vec == 1 ? (l->kind != 0 ? 16 : 8) : ((l->kind != 0 && full <= 4) ? 8 : 4));
+    if (!u.unroll && l->group <= 16 && l->vec == 1) l->steps = 4;  // packed, 4 or more steps per instruction
     const bool steps_ok = (l->vec == full) ? (l->steps == 2 || l->steps == 4 || l->steps == 8)
                                            : (l->steps == 4 || l->steps == 8 || l->steps == 16);
     if (!steps_ok) return SCANSCAM_EPLAN;
@@ -435,7 +449,8 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     if (u.waves) {
         l->waves = u.waves;
     } else {
-        const int64_t segments = (T + l->steps - 1) / l->steps;  // no more waves than segments of time
+        const int64_t wave_steps = (int64_t)l->steps * (kWave / l->group);
+        const int64_t segments = (T + wave_steps - 1) / wave_steps;  // no more waves than segments of time
         l->waves = segments < max_waves ? pow2_ceil(segments) : max_waves;
         // Tiles over workgroups: 8 waves (shorter tiles, more of them to hand out), 16 when there are very
         // few carry chains to spread the workgroups over.
@@ -508,6 +523,7 @@ int run_cl(bool rev, const void *a, const void *x, const void *h, void *y0, void
     args.T = (int32_t)T;
     args.C = (int32_t)C;
     args.segments = l.segments;
+    args.group = l.group;
     args.ws = nullptr;
     args.spin_limit = (plan && plan->spin_limit > 0) ? plan->spin_limit : scanscam::kSpinLimit;
 

@@ -21,7 +21,9 @@
 // A workgroup owns 64*VEC channels of one batch element. When that gives too
 // few workgroups to fill the GPU, time is also cut into tiles over workgroups
 // (scan_cl_lookback_kernel), with a decoupled look-back chain that carries one
-// affine pair per channel from tile to tile.
+// affine pair per channel from tile to tile. When C is so small that a time
+// step does not fill half a wave, a wave holds several consecutive time steps
+// instead (scan_cl_packed_kernel) and scans across them with lane moves.
 #pragma once
 
 #include "scan_kernels.hpp"
@@ -40,6 +42,7 @@ struct ClArgs {
     int32_t T;
     int32_t C;
     int32_t segments;   // look-back kernel: tiles per (batch element, channel group)
+    int32_t group;      // packed kernel: lanes per time step (power of two below 64)
     uint64_t *ws;       // look-back kernel: ticket counters + published pairs
     int32_t spin_limit; // look-back kernel: polls before a wait gives up
 };
@@ -233,6 +236,141 @@ __global__ __launch_bounds__(MAXT) void scan_cl_kernel(const ClArgs p)
         CT *lds_A = lds + (it & 1) * 2 * plane;
         cl_tile<ST, VEC, S, REV, true, CT>(ln, p.T, it * tile_steps, p.T, wave, W, lane, lds_A, lds_A + plane,
                                            unused, carry);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Few channels (C <= 32*VEC): a time step fills only G = pow2 >= C/VEC lanes, so
+// a wave holds 64/G consecutive time steps per instruction: lane = (step in the
+// instruction, channel vector), and every load and store instruction still
+// covers one contiguous span (64/G steps of C channels). The recurrence along
+// time is then a scan ACROSS lanes at stride G (a lane never folds in time by
+// itself: its S instructions are 64/G steps apart). Per instruction: an
+// inclusive scan of the affine pairs over the lanes of one channel vector, on
+// lane shuffles at distances G, 2G, ... 32; instruction to instruction the
+// total (held by the last step's lanes) is composed onto a running pair; wave
+// to wave through LDS, tile to tile in registers, as in scan_cl_kernel. Every
+// element's output is then one FMA: inclusive pair applied to the value entering
+// the wave. A workgroup owns one batch element.
+// LDS: two buffers (tiles alternate) of A and B, each [W][VEC][G] values.
+// ---------------------------------------------------------------------------
+template <typename ST, int VEC, int S, bool REV, int MAXT>
+__global__ __launch_bounds__(MAXT) void scan_cl_packed_kernel(const ClArgs p)
+{
+    using CT = typename ComputeOf<ST>::type;
+    using V = Vec<ST, VEC>;
+    using raw_t = typename V::raw_t;
+    extern __shared__ double lds_raw[];
+    CT *lds = reinterpret_cast<CT *>(lds_raw);
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int W = blockDim.x / kWave;
+    const int G = p.group;
+    const int subs = kWave / G;       // time steps per instruction
+    const int cl = lane & (G - 1);    // channel vector of this lane
+    const int sub = lane / G;         // its step inside the instruction
+    const ClLane<ST> ln = cl_lane<ST, VEC>(p, blockIdx.x, 0, cl);
+
+    const int wave_steps = S * subs;
+    const int tile_steps = W * wave_steps;
+    const int ntiles = (p.T + tile_steps - 1) / tile_steps;
+    const int plane = W * VEC * G;
+    CT carry[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; k++) carry[k] = CT(0);
+
+    for (int it = 0; it < ntiles; it++) {
+        CT *lds_A = lds + (it & 1) * 2 * plane, *lds_B = lds_A + plane;
+        // All loads first, unconditionally (masked lanes read offset 0 of their own column).
+        raw_t ra[S], rx[S], rh[REV ? S : 1];
+        bool ok[S], a_ok[S], h_ok[S];
+        int tt[S];
+#pragma unroll
+        for (int s = 0; s < S; s++) {
+            const int tau = it * tile_steps + (wave * S + s) * subs + sub;  // scan position
+            const int t = REV ? p.T - 1 - tau : tau;
+            tt[s] = t;
+            ok[s] = ln.c_ok && tau < p.T;
+            a_ok[s] = ok[s] && (!REV || t + 1 < p.T);  // backward gate a[t+1], 0 past the end
+            h_ok[s] = ok[s] && t > 0;                   // h[-1] = 0
+            ra[s] = V::load(ln.a + (a_ok[s] ? (int64_t)(REV ? t + 1 : t) * ln.pa : 0));
+            rx[s] = V::load(ln.x + (ok[s] ? (int64_t)t * ln.px : 0));
+            if (REV) rh[s] = V::load(ln.h + (h_ok[s] ? (int64_t)(t - 1) * ln.ph : 0));
+        }
+        // PA/PB: the pair of everything in this wave's span up to and including the lane's step of
+        // instruction s; (RA, RB): instructions 0..s-1 composed (the same in every lane of a channel).
+        CT PA[S][VEC], PB[S][VEC], RA[VEC], RB[VEC];
+#pragma unroll
+        for (int k = 0; k < VEC; k++) {
+            RA[k] = CT(1);
+            RB[k] = CT(0);
+        }
+#pragma unroll
+        for (int s = 0; s < S; s++) {
+            CT fa[VEC], fx[VEC];
+            V::unpack(ra[s], fa);
+            V::unpack(rx[s], fx);
+#pragma unroll
+            for (int k = 0; k < VEC; k++) {
+                CT A = ok[s] ? (a_ok[s] ? fa[k] : CT(0)) : CT(1);
+                CT B = ok[s] ? fx[k] : CT(0);
+                for (int off = G; off < kWave; off <<= 1) {
+                    const CT A1 = __shfl_up(A, off, kWave), B1 = __shfl_up(B, off, kWave);
+                    if (lane >= off) {
+                        B = fma_(A, B1, B);
+                        A = A * A1;
+                    }
+                }
+                const CT TA = __shfl(A, kWave - G + cl, kWave), TB = __shfl(B, kWave - G + cl, kWave);
+                PB[s][k] = fma_(A, RB[k], B);
+                PA[s][k] = A * RA[k];
+                RB[k] = fma_(TA, RB[k], TB);
+                RA[k] = TA * RA[k];
+            }
+        }
+        CT mine[VEC];
+#pragma unroll
+        for (int k = 0; k < VEC; k++) mine[k] = carry[k];
+        if (W > 1) {
+            if (sub == 0) {
+#pragma unroll
+                for (int k = 0; k < VEC; k++) {
+                    lds_A[(wave * VEC + k) * G + cl] = RA[k];
+                    lds_B[(wave * VEC + k) * G + cl] = RB[k];
+                }
+            }
+            __syncthreads();
+            for (int q = 0; q < W; q++) {
+#pragma unroll
+                for (int k = 0; k < VEC; k++) {
+                    const CT Aq = lds_A[(q * VEC + k) * G + cl], Bq = lds_B[(q * VEC + k) * G + cl];
+                    if (q == wave) mine[k] = carry[k];
+                    carry[k] = fma_(Aq, carry[k], Bq);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < VEC; k++) carry[k] = fma_(RA[k], carry[k], RB[k]);
+        }
+#pragma unroll
+        for (int s = 0; s < S; s++) {
+            CT out[VEC];
+#pragma unroll
+            for (int k = 0; k < VEC; k++) out[k] = fma_(PA[s][k], mine[k], PB[s][k]);
+            if (!REV) {
+                if (ok[s]) V::store(ln.y0 + (int64_t)tt[s] * ln.py0, V::pack(out));
+            } else {
+                CT fh[VEC], ga[VEC];
+                V::unpack(rh[s], fh);
+#pragma unroll
+                for (int k = 0; k < VEC; k++) ga[k] = out[k] * (h_ok[s] ? fh[k] : CT(0));
+                if (ok[s]) {
+                    V::store(ln.y0 + (int64_t)tt[s] * ln.py0, V::pack(out));
+                    V::store(ln.y1 + (int64_t)tt[s] * ln.py1, V::pack(ga));
+                }
+            }
+        }
     }
 }
 

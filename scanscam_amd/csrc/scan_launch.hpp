@@ -90,6 +90,7 @@ struct ClLaunch {
     int steps;
     int waves;
     int kind;       // 0: a workgroup walks all of T; 2: tiles over workgroups with a look-back chain
+    int group;      // kind 0: lanes per time step; below 64: the packed kernel for few channels
     int segments;   // kind 2: tiles per row-group
     int64_t grid;
     size_t lds_bytes;
@@ -107,6 +108,9 @@ hipError_t launch_scan_cl(const ClArgs &args, const ClLaunch &l, bool rev, hipSt
         if (l.kind == 2) {                                                                             \
             if (rev) hipLaunchKernelGGL((scan_cl_lookback_kernel<ST, VEC, S, true, MAXT>), grid, block, l.lds_bytes, stream, args);  \
             else     hipLaunchKernelGGL((scan_cl_lookback_kernel<ST, VEC, S, false, MAXT>), grid, block, l.lds_bytes, stream, args); \
+        } else if (l.group < kWave) {                                                                  \
+            if (rev) hipLaunchKernelGGL((scan_cl_packed_kernel<ST, VEC, S, true, MAXT>), grid, block, l.lds_bytes, stream, args);  \
+            else     hipLaunchKernelGGL((scan_cl_packed_kernel<ST, VEC, S, false, MAXT>), grid, block, l.lds_bytes, stream, args); \
         } else {                                                                                       \
             if (rev) hipLaunchKernelGGL((scan_cl_kernel<ST, VEC, S, true, MAXT>), grid, block, l.lds_bytes, stream, args);  \
             else     hipLaunchKernelGGL((scan_cl_kernel<ST, VEC, S, false, MAXT>), grid, block, l.lds_bytes, stream, args); \

@@ -178,3 +178,33 @@ def test_expired_wait_is_reported_and_every_wave_exits(gpu):
     else:
         assert torch.equal(out, good)
     assert torch.equal(hip.transposed_linear_scan_forward(x, y, plan=hip.Plan(mode=hip.MODE_LOOKBACK, vec=1, unroll=4, waves=2)), good)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16])
+def test_few_channels_packed_kernel(gpu, dtype):
+    # C <= 32 with enough batch elements: a wave holds several consecutive time steps per instruction and
+    # scans across them with lane shuffles. Every lane-group width (1 ... 32 lanes per step), channel
+    # counts that do not fill the group, 16-byte and single-channel lanes, lengths that end inside an
+    # instruction, inside a wave's span and inside a tile.
+    full = 16 // torch.empty(0, dtype=dtype).element_size()
+    bar = {torch.float32: 1e-5, torch.float64: 1e-13}.get(dtype, 1e-2)
+    g = torch.Generator().manual_seed(23)
+    for C, T in [(1, 700), (2, 129), (3, 1000), (5, 64), (8, 4097), (12, 333), (16, 2048), (24, 515), (31, 77), (32, 1030)]:
+        shape = (257, T, C)
+        a = torch.rand(shape, generator=g, dtype=torch.float64).to(dtype)
+        b = torch.randn(shape, generator=g, dtype=torch.float64).to(dtype)
+        gh = torch.randn(shape, generator=g, dtype=torch.float64).to(dtype)
+        h = oracle.fwd(as_rows(a), as_rows(b))
+        hs = torch.from_numpy(h).mT.contiguous().to(dtype)
+        ga, gb = oracle.bwd(as_rows(a), as_rows(hs), as_rows(gh))
+        plans = [None]
+        if C % full == 0:
+            plans += [hip.Plan(vec=full, unroll=4, mode=hip.MODE_ROW), hip.Plan(vec=full, unroll=2, waves=3, mode=hip.MODE_ROW)]
+        plans += [hip.Plan(vec=1, unroll=16, waves=2, mode=hip.MODE_ROW)]
+        for plan in plans:
+            print(f"case cl packed {dtype} shape={shape} {plan}", flush=True)
+            got_h = hip.transposed_linear_scan_forward(a.to(gpu), b.to(gpu), plan=plan)
+            got_ga, got_gb = hip.transposed_linear_scan_backward(a.to(gpu), hs.to(gpu), gh.to(gpu), plan=plan)
+            assert rel_err(as_rows(got_h), h) <= bar, (plan, shape)
+            assert rel_err(as_rows(got_gb), gb) <= bar, (plan, shape)
+            assert rel_err(as_rows(got_ga), ga, prev_abs(as_rows(hs))) <= bar, (plan, shape)
