@@ -246,8 +246,9 @@ __global__ __launch_bounds__(MAXT) void scan_cl_kernel(const ClArgs p)
 // covers one contiguous span (64/G steps of C channels). The recurrence along
 // time is then a scan ACROSS lanes at stride G (a lane never folds in time by
 // itself: its S instructions are 64/G steps apart). Per instruction: an
-// inclusive scan of the affine pairs over the lanes of one channel vector, on
-// lane shuffles at distances G, 2G, ... 32; instruction to instruction the
+// inclusive scan of the affine pairs over the lanes of one channel vector (DPP
+// moves inside each row of 16 lanes, two shuffles across rows); instruction to
+// instruction the
 // total (held by the last step's lanes) is composed onto a running pair; wave
 // to wave through LDS, tile to tile in registers, as in scan_cl_kernel. Every
 // element's output is then one FMA: inclusive pair applied to the value entering
@@ -315,11 +316,49 @@ __global__ __launch_bounds__(MAXT) void scan_cl_packed_kernel(const ClArgs p)
             for (int k = 0; k < VEC; k++) {
                 CT A = ok[s] ? (a_ok[s] ? fa[k] : CT(0)) : CT(1);
                 CT B = ok[s] ? fx[k] : CT(0);
-                for (int off = G; off < kWave; off <<= 1) {
-                    const CT A1 = __shfl_up(A, off, kWave), B1 = __shfl_up(B, off, kWave);
-                    if (lane >= off) {
-                        B = fma_(A, B1, B);
-                        A = A * A1;
+                // Two ways to the same inclusive scan over the steps of one instruction. Measured, the backward
+                // pass with one channel per lane is 15 % faster on plain shuffles at distances G, 2G, ... 32;
+                // everything else 8-20 % faster with the ladder below.
+                if (REV && VEC == 1) {
+                    for (int off = G; off < kWave; off <<= 1) {
+                        const CT A1 = __shfl_up(A, off, kWave), B1 = __shfl_up(B, off, kWave);
+                        if (lane >= off) {
+                            B = fma_(A, B1, B);
+                            A = A * A1;
+                        }
+                    }
+                } else {
+                    // Inside each row of 16 lanes: DPP moves at distances G, 2G, ... 8 (lanes without a
+                    // source in their row receive the identity).
+#define SCANSCAM_ROW_STEP(OFF)                                  \
+    if (G <= (OFF)) {                                           \
+        const CT A1 = dpp_move<0x110 + (OFF), 0xf>(CT(1), A);   \
+        const CT B1 = dpp_move<0x110 + (OFF), 0xf>(CT(0), B);   \
+        B = fma_(A, B1, B);                                     \
+        A = A * A1;                                             \
+    }
+                    SCANSCAM_ROW_STEP(1)
+                    SCANSCAM_ROW_STEP(2)
+                    SCANSCAM_ROW_STEP(4)
+                    SCANSCAM_ROW_STEP(8)
+#undef SCANSCAM_ROW_STEP
+                    // Across rows: rows 1 and 3 take the total of the row before (held by its last lanes of
+                    // the same channel vector), then rows 2 and 3 the total of rows 0-1.
+                    if (G <= 16) {
+                        const int src = ((lane & ~15) - G + cl) & (kWave - 1);  // rows 0 and 2 discard what they read
+                        const CT A1 = __shfl(A, src, kWave), B1 = __shfl(B, src, kWave);
+                        if (lane & 16) {
+                            B = fma_(A, B1, B);
+                            A = A * A1;
+                        }
+                    }
+                    {
+                        const int src = 32 - G + cl;
+                        const CT A1 = __shfl(A, src, kWave), B1 = __shfl(B, src, kWave);
+                        if (lane & 32) {
+                            B = fma_(A, B1, B);
+                            A = A * A1;
+                        }
                     }
                 }
                 const CT TA = __shfl(A, kWave - G + cl, kWave), TB = __shfl(B, kWave - G + cl, kWave);
