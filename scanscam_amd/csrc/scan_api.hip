@@ -384,7 +384,7 @@ int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y
 }
 
 // Channels-last: choice of vector width, steps per wave and waves per workgroup.
-int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, int dtype, bool aligned16,
+int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, int dtype, bool aligned16, bool aligned4,
                scanscam::ClLaunch *l)
 {
     const int esize = elem_size(dtype);
@@ -392,27 +392,32 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     scanscam_plan u = {0, 0, 0, 0, 0, 0};
     if (user) u = *user;
     const bool vec_possible = aligned16 && (C % full == 0);
+    // The narrow lane: one channel, or two for 16-bit storage (4 bytes, like one fp32 channel).
+    const bool pair_possible = esize == 2 && aligned4 && (C % 2 == 0);
     auto groups = [&](int vec) { return (C + (int64_t)kWave * vec - 1) / ((int64_t)kWave * vec); };
+    // Pairs halve the number of workgroups: not where single channels just reach 256 of them and pairs do not.
+    const int narrow = pair_possible && (batch * groups(2) >= 256 || batch * groups(1) < 256) ? 2 : 1;
     if (u.vec) {
         l->vec = u.vec;
     } else if (!vec_possible) {
-        l->vec = 1;
+        l->vec = narrow;
     } else {
         // A workgroup owns 64*vec channels of one batch element. Enough of them: 16-byte loads.
-        // Not enough: one channel per lane, which gives full/1 times as many workgroups; if even those
+        // Not enough: narrow lanes, which give full/narrow times as many workgroups; if even those
         // are too few, time is split over workgroups as well (below), and there too the narrow lanes
         // win: more, narrower carry chains (fp32 1.1-1.7 times faster than 16-byte lanes, measured from
         // [1, 262144, 256] to [8, 4096, 512]; 16-bit storage 2.5-16 times, its 16-byte lanes leave
         // 8 times fewer chains).
-        l->vec = batch * groups(full) >= 256 ? full : 1;
+        l->vec = batch * groups(full) >= 256 ? full : narrow;
         // Few channels (the packed kernel, below): a wide lane leaves more steps per instruction to scan
         // across with lane shuffles, which costs more than the wider loads gain -- except where C is not a
         // power of two and one channel per lane would leave a quarter of 32 lanes idle (fp32 [256, 8192, 24]:
         // 177 / 235 us with 16-byte lanes, 209 / 320 with 4-byte lanes; [512, 4096, 8]: 66 / 80 against 44 / 67).
-        if (C <= 32 && (esize == 2 || pow2_ceil(C) <= 16 || is_pow2((int)C))) l->vec = 1;
+        if (C <= 32 && (esize == 2 || pow2_ceil(C) <= 16 || is_pow2((int)C))) l->vec = narrow;
     }
-    if (l->vec != 1 && l->vec != full) return SCANSCAM_EPLAN;
-    if (l->vec == full && full != 1 && !vec_possible) return SCANSCAM_EPLAN;
+    if (l->vec != 1 && l->vec != full && !(l->vec == 2 && esize == 2)) return SCANSCAM_EPLAN;
+    if (l->vec == full && !vec_possible) return SCANSCAM_EPLAN;
+    if (l->vec == 2 && esize == 2 && !pair_possible) return SCANSCAM_EPLAN;
     // Too few (batch element, channel group) pairs to fill the GPU: cut time into tiles over
     // workgroups as well. kind 0: one workgroup walks all of T. kind 2: tiles by ticket with a
     // look-back chain of per-channel pairs (mode = SCANSCAM_MODE_LOOKBACK forces it,
@@ -432,8 +437,9 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         if (g < kWave) l->group = g;
     }
 
-    l->steps = u.unroll ? u.unroll : (l->vec == 1 ? (l->kind != 0 ? 16 : 8) : ((l->kind != 0 && full <= 4) ? 8 : 4));
-    if (!u.unroll && l->group <= 16 && l->vec == 1) l->steps = 4;  // packed, 4 or more steps per instruction
+    const bool narrow_lane = l->vec < full;
+    l->steps = u.unroll ? u.unroll : (narrow_lane ? (l->kind != 0 ? 16 : 8) : ((l->kind != 0 && full <= 4) ? 8 : 4));
+    if (!u.unroll && l->group <= 16 && narrow_lane) l->steps = 4;  // packed, 4 or more steps per instruction
     const bool steps_ok = (l->vec == full) ? (l->steps == 2 || l->steps == 4 || l->steps == 8)
                                            : (l->steps == 4 || l->steps == 8 || l->steps == 16);
     if (!steps_ok) return SCANSCAM_EPLAN;
@@ -496,7 +502,7 @@ int run_cl(bool rev, const void *a, const void *x, const void *h, void *y0, void
     const int src[5] = {0, 1, rev ? 2 : 0, 3, rev ? 4 : 3};
     const int full = 16 / esize;
     int64_t sB[5], sT[5];
-    bool aligned16 = true;
+    bool aligned16 = true, aligned4 = true;  // aligned4: what two-channel lanes of 16-bit storage need
     for (int k = 0; k < 5; k++) {
         const scanscam_strides *t = st[src[k]];
         sB[k] = batch == 1 ? 0 : (t ? t->outer : T * C);
@@ -504,9 +510,10 @@ int run_cl(bool rev, const void *a, const void *x, const void *h, void *y0, void
         if (sB[k] < 0 || sT[k] < 0 || sT[k] >= kMaxT) return SCANSCAM_EINVAL;
         if (!aligned_to(ptrs[k], (size_t)esize)) return SCANSCAM_EALIGN;
         aligned16 = aligned16 && aligned_to(ptrs[k], 16) && sB[k] % full == 0 && sT[k] % full == 0;
+        aligned4 = aligned4 && aligned_to(ptrs[k], 4) && sB[k] % 2 == 0 && sT[k] % 2 == 0;
     }
     scanscam::ClLaunch l;
-    const int rc = resolve_cl(plan, batch, T, C, dtype, aligned16, &l);
+    const int rc = resolve_cl(plan, batch, T, C, dtype, aligned16, aligned4, &l);
     if (rc != SCANSCAM_OK) return rc;
 
     scanscam::ClArgs args;
@@ -635,9 +642,10 @@ size_t scanscam_workspace_bytes_cl(int64_t batch, int64_t T, int64_t C, int dtyp
     (void)direction;
     if (elem_size(dtype) == 0 || batch <= 0 || T <= 0 || C <= 0 || T >= kMaxT || C >= kMaxT) return 0;
     size_t need = 0;
-    for (int al = 0; al < 2; al++) {
+    for (int al = 0; al < 3; al++) {
         scanscam::ClLaunch l;
-        if (resolve_cl(plan, batch, T, C, dtype, al != 0, &l) == SCANSCAM_OK && l.ws_bytes > need) need = l.ws_bytes;
+        // al: 0 = element-aligned only, 1 = 4-byte aligned (16-bit pairs), 2 = 16-byte aligned
+        if (resolve_cl(plan, batch, T, C, dtype, al == 2, al >= 1, &l) == SCANSCAM_OK && l.ws_bytes > need) need = l.ws_bytes;
     }
     return need;
 }

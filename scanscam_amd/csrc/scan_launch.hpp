@@ -130,6 +130,11 @@ hipError_t launch_scan_cl(const ClArgs &args, const ClLaunch &l, bool rev, hipSt
         SCANSCAM_CL_CASE(ST, 1, 4)                                                                     \
         SCANSCAM_CL_CASE(ST, 1, 8)                                                                     \
         SCANSCAM_CL_CASE(ST, 1, 16)                                                                    \
+        if constexpr (sizeof(ST) == 2) { /* 16-bit storage: lanes of two channels (4 bytes) */         \
+            SCANSCAM_CL_CASE(ST, 2, 4)                                                                 \
+            SCANSCAM_CL_CASE(ST, 2, 8)                                                                 \
+            SCANSCAM_CL_CASE(ST, 2, 16)                                                                \
+        }                                                                                              \
         return hipErrorInvalidValue;                                                                   \
     }
 

@@ -81,7 +81,7 @@ def test_forced_plans(gpu, dtype):
         ga, gb = oracle.bwd(as_rows(a), as_rows(hs), as_rows(gh))
         cases.append((shape, a.to(gpu), b.to(gpu), gh.to(gpu), hs.to(gpu), h, ga, gb, prev_abs(as_rows(hs))))
     n = 0
-    for vec in (full, 1):
+    for vec in ((full, 2, 1) if full == 8 else (full, 1)):  # 16-bit storage also has lanes of two channels
         for steps in ((2, 4, 8) if vec == full else (4, 8, 16)):
             csize = 8 if dtype == torch.float64 else 4
             max_waves = min(16, 65536 // (4 * vec * 64 * csize), (512 if (vec > 1 and steps >= 8) else 1024) // 64)
@@ -92,7 +92,7 @@ def test_forced_plans(gpu, dtype):
                              for waves in sorted({1, 2, lb_waves})]
             for plan in shapes_plans:
                 for shape, a, b, gh, hs, h, ga, gb, hp in cases:
-                    if vec != 1 and shape[-1] % full != 0:
+                    if vec != 1 and shape[-1] % vec != 0:
                         continue
                     print(f"case cl forced {dtype} shape={shape} {plan}", flush=True)
                     got_h = hip.transposed_linear_scan_forward(a, b, plan=plan)
