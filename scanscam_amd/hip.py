@@ -244,7 +244,27 @@ class KernelEvents:
     @classmethod
     def _runtime(cls):
         if cls._rt is None:
-            rt = ctypes.CDLL("libamdhip64.so")
+            rt = None
+            # The events must come from the runtime instance the library launches with: the copy of
+            # libamdhip64 that is already mapped into this process (PyTorch's), else the loader's choice.
+            candidates = []
+            try:
+                with open("/proc/self/maps") as maps:
+                    for line in maps:
+                        path = line.split()[-1]
+                        if "libamdhip64.so" in path and path not in candidates:
+                            candidates.append(path)
+            except OSError:
+                pass
+            candidates.append("libamdhip64.so")
+            for path in candidates:
+                try:
+                    rt = ctypes.CDLL(path)
+                    break
+                except OSError:
+                    continue
+            if rt is None:
+                raise RuntimeError("scanscam_amd.hip.KernelEvents: libamdhip64.so not found")
             rt.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
             rt.hipEventDestroy.argtypes = [ctypes.c_void_p]
             rt.hipEventSynchronize.argtypes = [ctypes.c_void_p]
