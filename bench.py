@@ -26,7 +26,9 @@ Prints ONE JSON line. Besides the contract fields it carries
   configs       forward and forward+backward GB/s of the other four synthetic
                 configurations (buffer sets rotated so that the 256 MB
                 Infinity Cache cannot serve them; timed as batches of
-                back-to-back launches, gaps included).
+                back-to-back launches, gaps included). Where a launch is
+                shorter than the host's call (under 25 us), the *_graph_*
+                fields give the same launches replayed from a HIP graph.
 """
 import argparse
 import json
@@ -46,6 +48,8 @@ MEASURED_TRAFFIC = {"fwd": 805.37e6, "bwd": 1347.53e6}
 METRIC = "scan HBM GB/s and % of MI355X peak, fwd and fwd+bwd, fp32 [B,C,T]"
 FWD_BYTES = {4: 12, 2: 6}
 BWD_BYTES = {4: 20, 2: 10}
+# Launches shorter than this are paced by the host's call; they are also timed replaying from a HIP graph.
+GRAPH_BELOW_MS = 0.025
 
 
 # --workload: name -> (configuration number for make_config, description)
@@ -171,6 +175,37 @@ def time_batches(sets, launches, warmup, hip, torch):
     return out[0], out[1]
 
 
+def time_graph(sets, replays, hip, torch):
+    """Mean ms per launch of each direction when the launches replay from a HIP graph.
+
+    One launch per buffer set is captured (a kernel of a few microseconds is otherwise
+    paced by the host's call, not by the GPU); two events bracket `replays` replays.
+    """
+    out = []
+    for d in (0, 1):
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            calls = [(hip.prepare_forward(s.a, s.b, s.h), hip.prepare_backward(s.a, s.h, s.gh, s.ga, s.gb))[d]
+                     for s in sets]
+            calls[0]()
+            side.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                for c in calls:
+                    c()
+        torch.cuda.synchronize()
+        graph.replay()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(replays):
+            graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        out.append(e0.elapsed_time(e1) / (replays * len(sets)))
+        del graph
+    return out[0], out[1]
+
+
 def reference_grid(dev, args, hip, torch):
     """The shapes the reference's own timing tests use, fp32 N(0,1) inputs.
 
@@ -192,6 +227,12 @@ def reference_grid(dev, args, hip, torch):
             "fwd_us": round(f_ms * 1e3, 2), "bwd_us": round(b_ms * 1e3, 2),
             "fwd_GBps": round(12 * n / (f_ms * 1e-3) / 1e9, 1), "bwd_GBps": round(20 * n / (b_ms * 1e-3) / 1e9, 1),
         }
+        if f_ms < GRAPH_BELOW_MS:
+            gf_ms, gb_ms = time_graph(sets, max(4, 4 * args.steps // nsets), hip, torch)
+            out["x".join(map(str, shape))].update(
+                fwd_graph_us=round(gf_ms * 1e3, 2), bwd_graph_us=round(gb_ms * 1e3, 2),
+                fwd_graph_GBps=round(12 * n / (gf_ms * 1e-3) / 1e9, 1),
+                bwd_graph_GBps=round(20 * n / (gb_ms * 1e-3) / 1e9, 1))
         del sets, first
         torch.cuda.empty_cache()
     # Channels-last: logical [8, 512, 4096] stored [8, 4096, 512].
@@ -481,6 +522,15 @@ def main():
                                       / HBM_PEAK_GBPS, 4),
                 "elements_per_s_fwd_bwd": round(cn / ((f_ms + b_ms) * 1e-3)),
             }
+            if f_ms < GRAPH_BELOW_MS:
+                # Launch-bound from the host: the same launches replayed from a HIP graph.
+                gf_ms, gb_ms = time_graph(csets, max(4, 4 * args.steps // nsets), hip, torch)
+                others[key].update(
+                    fwd_graph_ms=round(gf_ms, 4),
+                    fwd_graph_frac=round(FWD_BYTES[esize] * cn / (gf_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                    fwd_bwd_graph_ms=round(gf_ms + gb_ms, 4),
+                    fwd_bwd_graph_frac=round((FWD_BYTES[esize] + BWD_BYTES[esize]) * cn / ((gf_ms + gb_ms) * 1e-3)
+                                             / 1e9 / HBM_PEAK_GBPS, 4))
             del csets, first
             torch.cuda.empty_cache()
         out["configs"] = others
