@@ -260,7 +260,7 @@ __device__ __forceinline__ void wave_scan(CT &A, CT &B, int j)
 // multiple of VEC, bases need not be 16-byte aligned): vectors are loaded and
 // stored element-aligned, and the last vector of a row may hold fewer than VEC
 // elements (`count`), the rest being masked to the identity.
-template <typename ST, int VEC, int U, bool REV, bool GROUPED, bool CHAIN, bool RAGGED = false>
+template <typename ST, int VEC, int U, bool REV, bool GROUPED, bool CHAIN, bool RAGGED = false, bool LEAN = false>
 struct WaveTile {
     using V = Vec<ST, VEC>;
     using raw_t = typename V::raw_t;
@@ -310,7 +310,13 @@ struct WaveTile {
     CT edge_a[REV ? U : 1];  // a[(m+1)*VEC] for the first lane of a group
     CT edge_h[REV ? U : 1];  // h[m*VEC - 1] for the last lane of a group
 
-    CT g[U][VEC], v[U][VEC];
+    // LEAN, for 16-bit storage with 8 elements per vector: the (gate, value) pairs are not kept from
+    // reduce() to apply() (64 fp32 registers per lane at U = 4, 96 with h[t-1] in the backward pass)
+    // but built a second time from the packed vectors, which take half the registers. It pays where
+    // waves wait between the two (the look-back kernel: more waves per SIMD cover the wait) and
+    // costs 1-2 % where they do not (the row kernel).
+    static constexpr bool REBUILD = LEAN && sizeof(ST) == 2 && VEC == 8;
+    CT g[REBUILD ? 1 : U][VEC], v[REBUILD ? 1 : U][VEC];
     CT PA[U], PB[U];
 
     __device__ __forceinline__ void load(const ScanArgs &p, int j, int jlast)
@@ -351,12 +357,10 @@ struct WaveTile {
         }
     }
 
-    // Builds (gate, value) per element in scan order and reduces them.
-    __device__ __forceinline__ void reduce(int j, int jlast, CT (&hp)[REV ? U : 1][VEC])
+    // Backward with CHAIN: a[first element] and h[last element] of every chunk's vectors, for the
+    // lanes at the borders between the chunks of this wave.
+    __device__ __forceinline__ void borders(CT (&first_a)[REV ? U : 1], CT (&last_h)[REV ? U : 1]) const
     {
-        // Backward: a[first element] and h[last element] of every chunk's vectors,
-        // for the lanes at the borders between the chunks of this wave.
-        CT first_a[REV ? U : 1], last_h[REV ? U : 1];
         if (REV && CHAIN) {
 #pragma unroll
             for (int u = 0; u < U; u++) {
@@ -367,58 +371,91 @@ struct WaveTile {
                 last_h[u] = valid[u] ? t[VEC - 1] : CT(0);
             }
         }
+    }
+
+    // (gate, value) per element of chunk u in scan order, and for the backward pass h[t-1].
+    __device__ __forceinline__ void build(int u, int j, int jlast, const CT (&first_a)[REV ? U : 1],
+                                          const CT (&last_h)[REV ? U : 1], CT (&G)[VEC], CT (&X)[VEC],
+                                          CT (&HP)[VEC]) const
+    {
+        CT fa[VEC], fx[VEC];
+        V::unpack(ra[u], fa);
+        V::unpack(rx[u], fx);
+#pragma unroll
+        for (int k = 0; k < VEC; k++) {  // lanes outside the row hold a = 0, x = 0
+            fa[k] = valid[u] ? fa[k] : CT(0);
+            fx[k] = valid[u] ? fx[k] : CT(0);
+        }
+        if (!REV) {
+#pragma unroll
+            for (int k = 0; k < VEC; k++) {
+                const bool in_row = RAGGED ? (valid[u] && k < count[u]) : valid[u];
+                G[k] = in_row ? fa[k] : CT(1);
+                X[k] = fx[k];  // zero-filled where invalid
+            }
+        } else {
+            CT fh[VEC];
+            V::unpack(rh[u], fh);
+#pragma unroll
+            for (int k = 0; k < VEC; k++) fh[k] = valid[u] ? fh[k] : CT(0);
+            // Scan order k <-> time t0 + VEC-1-k. gate = a[t+1], value = gh[t],
+            // hp = h[t-1]. Invalid lanes hold a = 0, so a neighbour past the
+            // end of the row reads as gate 0, which is what t = T-1 needs.
+            CT a_next = lane_prev(fa[0], CT(0));        // lane-1 holds vector m+1
+            CT h_prev = lane_next(fh[VEC - 1], CT(0));  // lane+1 holds vector m-1
+            CT border_a = edge_a[u], border_h = edge_h[u];
+            if (CHAIN && u > 0) border_a = read_lane(first_a[u - 1], kWave - 1);
+            if (CHAIN && u + 1 < U) border_h = read_lane(last_h[u + 1], 0);
+            a_next = (j == 0) ? border_a : a_next;
+            h_prev = (j == jlast) ? border_h : h_prev;
+#pragma unroll
+            for (int k = 0; k < VEC; k++) {
+                const CT gk = (k == 0) ? a_next : fa[(VEC - k) % VEC];
+                // Scan position k is element VEC-1-k of the vector; past the row's end it is the identity
+                // (its a and gh read as 0, so the element below it sees gate 0, as t = T-1 must).
+                const bool in_row = RAGGED ? (valid[u] && VEC - 1 - k < count[u]) : valid[u];
+                G[k] = in_row ? gk : CT(1);
+                X[k] = fx[VEC - 1 - k];
+                HP[k] = (k == VEC - 1) ? h_prev : fh[(VEC - 2 - k) < 0 ? 0 : (VEC - 2 - k)];
+            }
+        }
+    }
+
+    // Builds (gate, value) per element in scan order and reduces them.
+    __device__ __forceinline__ void reduce(int j, int jlast, CT (&hp)[REV ? U : 1][VEC])
+    {
+        CT first_a[REV ? U : 1], last_h[REV ? U : 1];
+        borders(first_a, last_h);
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            CT fa[VEC], fx[VEC];
-            V::unpack(ra[u], fa);
-            V::unpack(rx[u], fx);
-#pragma unroll
-            for (int k = 0; k < VEC; k++) {  // lanes outside the row hold a = 0, x = 0
-                fa[k] = valid[u] ? fa[k] : CT(0);
-                fx[k] = valid[u] ? fx[k] : CT(0);
-            }
-            if (!REV) {
+            CT G[VEC], X[VEC], HP[VEC];
+            build(u, j, jlast, first_a, last_h, G, X, HP);
+            if (!REBUILD) {
 #pragma unroll
                 for (int k = 0; k < VEC; k++) {
-                    const bool in_row = RAGGED ? (valid[u] && k < count[u]) : valid[u];
-                    g[u][k] = in_row ? fa[k] : CT(1);
-                    v[u][k] = fx[k];  // zero-filled where invalid
-                }
-            } else {
-                CT fh[VEC];
-                V::unpack(rh[u], fh);
-#pragma unroll
-                for (int k = 0; k < VEC; k++) fh[k] = valid[u] ? fh[k] : CT(0);
-                // Scan order k <-> time t0 + VEC-1-k. gate = a[t+1], value = gh[t],
-                // hp = h[t-1]. Invalid lanes hold a = 0, so a neighbour past the
-                // end of the row reads as gate 0, which is what t = T-1 needs.
-                CT a_next = lane_prev(fa[0], CT(0));        // lane-1 holds vector m+1
-                CT h_prev = lane_next(fh[VEC - 1], CT(0));  // lane+1 holds vector m-1
-                CT border_a = edge_a[u], border_h = edge_h[u];
-                if (CHAIN && u > 0) border_a = read_lane(first_a[u - 1], kWave - 1);
-                if (CHAIN && u + 1 < U) border_h = read_lane(last_h[u + 1], 0);
-                a_next = (j == 0) ? border_a : a_next;
-                h_prev = (j == jlast) ? border_h : h_prev;
-#pragma unroll
-                for (int k = 0; k < VEC; k++) {
-                    const CT gk = (k == 0) ? a_next : fa[(VEC - k) % VEC];
-                    // Scan position k is element VEC-1-k of the vector; past the row's end it is the identity
-                    // (its a and gh read as 0, so the element below it sees gate 0, as t = T-1 must).
-                    const bool in_row = RAGGED ? (valid[u] && VEC - 1 - k < count[u]) : valid[u];
-                    g[u][k] = in_row ? gk : CT(1);
-                    v[u][k] = fx[VEC - 1 - k];
-                    hp[u][k] = (k == VEC - 1) ? h_prev : fh[(VEC - 2 - k) < 0 ? 0 : (VEC - 2 - k)];
+                    g[u][k] = G[k];
+                    v[u][k] = X[k];
+                    if (REV) hp[u][k] = HP[k];
                 }
             }
-            CT A = g[u][0], B = v[u][0];
+            CT A = G[0], B = X[0];
 #pragma unroll
             for (int k = 1; k < VEC; k++) {
-                B = fma_(g[u][k], B, v[u][k]);
-                A = A * g[u][k];
+                B = fma_(G[k], B, X[k]);
+                A = A * G[k];
             }
             wave_scan<GROUPED, CT>(A, B, j);
             PA[u] = A;
             PB[u] = B;
+        }
+        if (REBUILD) {
+            // The packed vectors pass through an empty asm statement, so that the compiler
+            // cannot carry their unpacked form over to apply() instead of unpacking again.
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                asm volatile("" : "+v"(ra[u]), "+v"(rx[u]));
+                if (REV) asm volatile("" : "+v"(rh[u]));
+            }
         }
     }
 
@@ -435,13 +472,26 @@ struct WaveTile {
         }
     }
 
-    __device__ __forceinline__ void apply(const ScanArgs &p, CT carry, int j,
+    __device__ __forceinline__ void apply(const ScanArgs &p, CT carry, int j, int jlast,
                                           const CT (&hp)[REV ? U : 1][VEC])
     {
         ST *y0 = static_cast<ST *>(p.y0);
         ST *y1 = static_cast<ST *>(p.y1);
+        CT first_a[REV ? U : 1], last_h[REV ? U : 1];
+        if (REBUILD) borders(first_a, last_h);
 #pragma unroll
         for (int u = 0; u < U; u++) {
+            CT G[VEC], X[VEC], HP[VEC];
+            if (REBUILD) {
+                build(u, j, jlast, first_a, last_h, G, X, HP);
+            } else {
+#pragma unroll
+                for (int k = 0; k < VEC; k++) {
+                    G[k] = g[u][k];
+                    X[k] = v[u][k];
+                    if (REV) HP[k] = hp[u][k];
+                }
+            }
             // Map of everything before this lane inside the chunk.
             CT EA = lane_prev(PA[u], CT(1));
             CT EB = lane_prev(PB[u], CT(0));
@@ -454,7 +504,7 @@ struct WaveTile {
             CT out[VEC];
 #pragma unroll
             for (int k = 0; k < VEC; k++) {
-                acc = fma_(g[u][k], acc, v[u][k]);
+                acc = fma_(G[k], acc, X[k]);
                 out[k] = acc;
             }
             if (CHAIN && u + 1 < U)
@@ -466,7 +516,7 @@ struct WaveTile {
 #pragma unroll
                 for (int k = 0; k < VEC; k++) {
                     gb[VEC - 1 - k] = out[k];
-                    ga[VEC - 1 - k] = out[k] * hp[u][k];
+                    ga[VEC - 1 - k] = out[k] * HP[k];
                 }
                 if (valid[u]) {
                     put(y0 + at<3>(p, u), V::pack(gb), u);
@@ -543,7 +593,7 @@ __global__ __launch_bounds__(MAXT) void scan_row_kernel(const ScanArgs p)
             w.total(WA, WB);
             row_carry = fma_(WA, row_carry, WB);
         }
-        w.apply(p, carry, lane, hp);
+        w.apply(p, carry, lane, kWave - 1, hp);
     }
 }
 
@@ -576,7 +626,7 @@ __global__ __launch_bounds__(MAXT) void scan_small_kernel(const ScanArgs p)
     }
     w.load(p, j, G - 1);
     w.reduce(j, G - 1, hp);
-    w.apply(p, CT(0), j, hp);
+    w.apply(p, CT(0), j, G - 1, hp);
 }
 
 // ---------------------------------------------------------------------------
@@ -793,7 +843,7 @@ __global__ __launch_bounds__(MAXT) void scan_lookback_kernel(const ScanArgs p)
     const int nvp = p.nch * kWave;
     const int chunk0 = (tile * nwaves + wave) * U;
 
-    WaveTile<ST, VEC, U, REV, false, true, RAGGED> w;
+    WaveTile<ST, VEC, U, REV, false, true, RAGGED, true> w;
     const int64_t group = row / p.n1;
     w.set_row(p, group, row - group * p.n1);
     CT hp[REV ? U : 1][VEC];
@@ -832,7 +882,7 @@ __global__ __launch_bounds__(MAXT) void scan_lookback_kernel(const ScanArgs p)
 
     CT carry = lds_carry;
     for (int q = 0; q < wave; q++) carry = fma_(lds_A[q], carry, lds_B[q]);
-    w.apply(p, carry, lane, hp);
+    w.apply(p, carry, lane, kWave - 1, hp);
 }
 
 }  // namespace scanscam
