@@ -23,6 +23,8 @@ Prints ONE JSON line. Besides the contract fields it carries
                 timed on this host (oracle/_ref if it was built, else the C
                 restatement in oracle/);
   long_rows     many rows of 16K to 96K elements (long-context shapes);
+  autograd_op   the same step through the op a model calls,
+                scanscam_amd.scan(a, b).backward(grad_h), outputs allocated per call;
   configs       forward and forward+backward GB/s of the other four synthetic
                 configurations (buffer sets rotated so that the 256 MB
                 Infinity Cache cannot serve them; timed as batches of
@@ -204,6 +206,36 @@ def time_graph(sets, replays, hip, torch):
         out.append(e0.elapsed_time(e1) / (replays * len(sets)))
         del graph
     return out[0], out[1]
+
+
+def autograd_step(s, shape, steps, warmup, torch):
+    """Wall milliseconds per step of the op a model calls: h = scan(a, b); h.backward(grad_h).
+
+    The same kernels as the timed region, plus what the autograd function adds per call: the
+    allocation of h and of the two gradients from torch's caching allocator, the autograd graph,
+    the checks and the plan look-up.
+    """
+    import scanscam_amd
+
+    a = s.a.view(shape).requires_grad_()
+    b = s.b.view(shape).requires_grad_()
+    gh = s.gh.view(shape)
+
+    def step():
+        a.grad = b.grad = None
+        scanscam_amd.scan(a, b).backward(gh)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+    a.requires_grad_(False)
+    b.requires_grad_(False)
+    return wall * 1e3
 
 
 def reference_grid(dev, args, hip, torch):
@@ -491,6 +523,13 @@ def main():
             "avg_ms": round(fwd_ms, 4),
             "min_ms": round(fwd_min, 4),
         },
+    }
+    op_ms = autograd_step(first, tuple(a.shape), args.steps, args.warmup, torch)
+    out["autograd_op"] = {
+        "call": "scanscam_amd.scan(a, b).backward(grad_h), outputs allocated per call",
+        "ms_per_step": round(op_ms, 4),
+        "GBps": round(step_bytes * n / (op_ms * 1e-3) / 1e9, 1),
+        "frac": round(step_bytes * n / (op_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
     }
     del sets, first
 
