@@ -26,7 +26,8 @@ Prints ONE JSON line. Besides the contract fields it carries
   autograd_op   the same step through the op a model calls,
                 scanscam_amd.scan(a, b).backward(grad_h), outputs allocated per call;
   configs       forward and forward+backward GB/s of the other four synthetic
-                configurations (buffer sets rotated so that the 256 MB
+                configurations and of configuration 2's bytes in float64
+                ([8, 2048, 2048]) (buffer sets rotated so that the 256 MB
                 Infinity Cache cannot serve them; timed as batches of
                 back-to-back launches, gaps included). Where a launch is
                 shorter than the host's call (under 25 us), the *_graph_*
@@ -48,8 +49,8 @@ HBM_PEAK_GBPS = 8000.0
 # counters read for a copy kernel of known size (profiles/scan_row_f32_fwd_bwd_8x2048x4096_pmc_traffic.txt).
 MEASURED_TRAFFIC = {"fwd": 805.37e6, "bwd": 1347.53e6}
 METRIC = "scan HBM GB/s and % of MI355X peak, fwd and fwd+bwd, fp32 [B,C,T]"
-FWD_BYTES = {4: 12, 2: 6}
-BWD_BYTES = {4: 20, 2: 10}
+FWD_BYTES = {8: 24, 4: 12, 2: 6}
+BWD_BYTES = {8: 40, 4: 20, 2: 10}
 # Launches shorter than this are paced by the host's call; they are also timed replaying from a HIP graph.
 GRAPH_BELOW_MS = 0.025
 
@@ -93,6 +94,10 @@ def make_config(n, torch):
     elif n == 6:
         shape = (1, 2048, 32768)
         a, b = torch.sigmoid(torch.randn(shape)), torch.randn(shape)
+    elif n == 20:  # configuration 2's bytes in float64 (the reference's other storage type): half its T
+        shape = (8, 2048, 2048)
+        a, b = torch.sigmoid(torch.randn(shape)), torch.randn(shape)
+        dtype = torch.float64
     else:
         raise ValueError(n)
     gh = torch.randn(shape)
@@ -535,7 +540,7 @@ def main():
 
     if not args.no_configs:
         others = {}
-        for key, cfg in (("1", 1), ("3", 3), ("4_bf16", 4), ("4_f16", 40), ("5", 5)):
+        for key, cfg in (("1", 1), ("3", 3), ("4_bf16", 4), ("4_f16", 40), ("5", 5), ("2_f64_half_T", 20)):
             ca, cb, cgh = make_config(cfg, torch)
             esize = ca.element_size()
             cn = ca.numel()
