@@ -457,6 +457,53 @@ def test_nonfinite_rows_do_not_leak_into_other_rows(gpu):
     assert np.all(np.isnan(h[4, 7:]))
 
 
+@pytest.mark.parametrize("T,plan", [
+    (64, None),                                                         # small kernel
+    (1024, None),                                                       # row kernel, one wave per row
+    (20000, None),                                                      # row kernel, 16 waves per row
+    (20000, hip.Plan(mode=hip.MODE_LOOKBACK, vec=4, unroll=1, waves=2)),  # look-back, 40 tiles per row
+])
+def test_backward_nonfinite_gradients_follow_the_reference(gpu, T, plan):
+    # The reference forms grad_a[0] as grad_b[0] * 0.0, a multiplication (src/scanscam_cpu.hpp:70-74: h[-1] is
+    # the value 0, not a skipped term), so an infinite or NaN grad_b[0] gives NaN there, and an infinite
+    # upstream gradient reaches every earlier time step through the gates. Gates just below 1 keep the
+    # sign of everything and keep products of gates over any span away from underflow (a parallel scan
+    # multiplies an infinite carry by the product of a whole span's gates, and 0 * inf would be NaN where
+    # the sequential loop, gate by gate, keeps inf), so the pattern of inf / NaN is fixed by the recurrence,
+    # not by the order of association; finite elements must still meet the fp32 bar. Gates 1 - x with
+    # x up to 2e-6: in fp32 the product (1 - x)(1 - y) loses its x*y term whenever that is below half the
+    # spacing 6e-8 of the numbers under 1, always in the same direction, so products of many gates that
+    # close to 1 come out low. A scan over pairs, which multiplies gates with each other, then ends a sum
+    # of 20 000 positive terms low by 1e-5 (relative) for x up to 2e-5 and by 3e-5 for x up to 1e-4 -- a
+    # plain Hillis-Steele scan in numpy does the same -- while the sequential loop never multiplies two
+    # gates. With x up to 2e-6 the effect is below 2e-6.
+    g = seeded(1200 + T)
+    rows = 6
+    a = 1.0 - 2e-6 * torch.rand((rows, T), generator=g)
+    b = torch.randn((rows, T), generator=g)
+    gh = torch.randn((rows, T), generator=g).abs()
+    gh[1, T // 2] = float("inf")     # everything at and before T/2 becomes +inf; grad_a[1, 0] = inf * 0 = NaN
+    gh[3, 0] = float("inf")          # only t = 0: grad_b = inf, grad_a = NaN
+    gh[4, T - 1] = float("nan")      # the whole row
+    h = oracle.fwd(a.numpy(), b.numpy())
+    wga, wgb = oracle.bwd(a.numpy(), h, gh.numpy())
+    ga, gb = (to_np(x) for x in run_bwd(gpu, a, torch.from_numpy(h), gh, plan))
+    for got, want in ((gb, wgb), (ga, wga)):
+        assert np.array_equal(np.isnan(got), np.isnan(want))
+        assert np.array_equal(np.isposinf(got), np.isposinf(want))
+        assert np.array_equal(np.isneginf(got), np.isneginf(want))
+    assert np.isnan(wga[1, 0]) and np.isnan(wga[3, 0]) and np.isposinf(wgb[3, 0]) and np.all(np.isnan(wgb[4]))
+    # Finite values against the float64 recurrence: with gates this close to 1 a row is nearly a running
+    # sum of T positive terms, which the fp32 sequential loop itself only holds to a few 1e-5.
+    h64 = h.astype(np.float64)
+    xga, xgb = oracle.bwd(a.double().numpy(), h64, gh.double().numpy())
+    for r in (0, 2, 5):
+        assert rel_err(gb[r], xgb[r]) <= FP32_BAR
+        assert rel_err(ga[r], xga[r], prev_abs(h)[r]) <= FP32_BAR
+    fin = np.isfinite(wgb[1])
+    assert rel_err(gb[1][fin], xgb[1][fin]) <= FP32_BAR
+
+
 @pytest.mark.parametrize("shape", [(32, 1025), (32, 4100), (3, 300001), (4, 64), (16, 2, 5)])
 def test_float64(gpu, shape):
     # The reference also dispatches double (src/scanscam_cpu.hpp:43): fp64 storage and arithmetic.
