@@ -6,7 +6,9 @@ Same surface as the reference's ``scanscam/op.py:9-55``: ``scan`` applies
 ``(grad_gate, grad_value)``. Dispatch is by device and layout as in
 ``op.py:27-35``: GPU tensors run the HIP kernels (the channels-last ones when the
 last two dimensions are transposed in memory, the row ones otherwise; strided
-views are not copied first), everything else the tensor-level loop. Two
+views are not copied first), float32 / float64 CPU tensors the native host loop
+(``scanscam_amd/cpu.py``) when its library is built, everything else the
+tensor-level loop. Two
 defects of the reference are not reproduced: its backward for transposed
 inputs calls a three-argument wrapper with four arguments (``op.py:46-48``),
 and its CPU backward drops its result (``op.py:52-53``); both return the
@@ -16,7 +18,7 @@ from typing import Any, Tuple
 
 import torch
 
-from . import hip
+from . import cpu, hip
 from .baseline import naive_linear_scan_backward, naive_linear_scan_forward
 
 
@@ -52,6 +54,8 @@ class Scan(torch.autograd.Function):
             # of leading dimensions, and strided views of either layout, are taken as they are
             # where the reference's wrappers would copy them first (cuda.py:36-37).
             output = hip.scan_forward(gate, value)
+        elif cpu.supports(gate) and cpu.supports(value):
+            output = cpu.simple_linear_scan_forward(gate, value)
         else:
             output = naive_linear_scan_forward(gate, value)
         ctx.save_for_backward(gate, output)
@@ -64,4 +68,6 @@ class Scan(torch.autograd.Function):
             # Channels-last when gate and output are: what op.py:45-49 of the reference means to
             # do (its call has one argument too many).
             return hip.scan_backward(gate, output, output_grad)
+        if cpu.supports(gate) and cpu.supports(output) and cpu.supports(output_grad):
+            return cpu.simple_linear_scan_backward(gate, output, output_grad)
         return naive_linear_scan_backward(gate, output, output_grad)
