@@ -22,6 +22,8 @@ Prints ONE JSON line. Besides the contract fields it carries
   cpu_baseline  the reference's single-threaded CPU loop on the same tensors,
                 timed on this host (oracle/_ref if it was built, else the C
                 restatement in oracle/);
+  host_library  the package's own loop for CPU tensors on the same tensors
+                (not the baseline: several rows side by side, several threads);
   long_rows     many rows of 16K to 96K elements (long-context shapes);
   autograd_op   the same step through the op a model calls,
                 scanscam_amd.scan(a, b).backward(grad_h), outputs allocated per call;
@@ -433,6 +435,43 @@ def cpu_baseline(a, b, gh, reps):
     }
 
 
+def host_library(a, b, gh, reps):
+    """The package's own loop for CPU tensors (libscanscam_cpu.so) on the same tensors.
+
+    Bit-identical to the reference's loop per row; 8 rows side by side per thread, slabs of rows over
+    threads. Outputs pre-allocated and touched, as for cpu_baseline. Reported beside it, not part of it.
+    """
+    import torch
+
+    from scanscam_amd import cpu
+
+    if not cpu.has_cpu_ops:
+        return None
+    T = a.shape[-1]
+    n = a.numel()
+    a2, b2, gh2 = (x.reshape(-1, T).contiguous() for x in (a, b, gh))
+    rows = a2.shape[0]
+    h, ga, gb = torch.zeros_like(a2), torch.zeros_like(a2), torch.zeros_like(a2)
+    suffix = cpu._SUFFIX[a2.dtype]
+    f, g = getattr(cpu._lib, f"scanscam_cpu_fwd_{suffix}"), getattr(cpu._lib, f"scanscam_cpu_bwd_{suffix}")
+    times = {"fwd": [], "bwd": []}
+    for rep in range(reps + 1):
+        for name, fn, tensors in (("fwd", f, (a2, b2, h)), ("bwd", g, (a2, h, gh2, ga, gb))):
+            t0 = time.perf_counter()
+            cpu._run(fn, tensors, rows, T)
+            dt = time.perf_counter() - t0
+            if rep > 0:
+                times[name].append(dt)
+    tf, tb = statistics.median(times["fwd"]), statistics.median(times["bwd"])
+    return {
+        "value": round(32 * n / (tf + tb) / 1e9, 3),
+        "unit": "GB/s",
+        "threads": len(cpu._slabs(rows, T)),
+        "fwd_s": round(tf, 4),
+        "bwd_s": round(tb, 4),
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -587,6 +626,7 @@ def main():
     if not args.no_cpu:
         # 16-bit workloads: the reference has no 16-bit path, so its loop runs on the exact fp32 upcast.
         out["cpu_baseline"] = cpu_baseline(a.float(), b.float(), gh.float(), reps=5)
+        out["host_library"] = host_library(a.float(), b.float(), gh.float(), reps=5)
 
     print(json.dumps(out))
 
