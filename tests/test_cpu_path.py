@@ -72,6 +72,32 @@ def test_bit_identical_to_the_reference_loop(shape, dtype):
     assert np.array_equal(ga.numpy(), wga)
 
 
+# The reference's CPU test grid (scanscam/cpu_test.py:11-48): N(0,1) gates and values, each shape
+# contiguous and with its last two dimensions transposed in memory (x.mT.contiguous().mT), forward
+# against the tensor-level loop at atol 1e-4 and backward as a plain function of three unrelated
+# tensors (gate, output, out_grad).
+REFERENCE_CPU_GRID = [(32, 5), (16, 2, 5), (32, 64), (1, 1024), (32, 1024), (32, 1025), (1, 1025)]
+
+
+@pytest.mark.parametrize("permute", [False, True])
+@pytest.mark.parametrize("shape", REFERENCE_CPU_GRID)
+def test_reference_cpu_grid(shape, permute):
+    from scanscam_amd.baseline import naive_linear_scan_backward, naive_linear_scan_forward
+
+    x, y, z = inputs(shape, torch.float32, 77 + sum(shape))
+    if permute:
+        x, y, z = (t.mT.contiguous().mT for t in (x, y, z))
+        assert not x.is_contiguous() or 1 in shape[-2:]
+    out = cpu.simple_linear_scan_forward(x, y)
+    assert out.shape == x.shape
+    assert torch.allclose(out, naive_linear_scan_forward(x, y), atol=1e-4)
+    ga, gb = cpu.simple_linear_scan_backward(x, y, z)
+    wa, wb = naive_linear_scan_backward(x, y, z)
+    # N(0,1) gates: values grow along a row; the bar of the reference's test, scaled by the row's size.
+    scale = max(1.0, float(wb.abs().max()), float(wa.abs().max()))
+    assert torch.allclose(ga, wa, atol=1e-4 * scale) and torch.allclose(gb, wb, atol=1e-4 * scale)
+
+
 def test_golden_vectors():
     # The fixtures written from the reference's own build (tests/golden/make_golden.py).
     z = np.load(os.path.join(ROOT, "tests", "golden", "scan_golden.npz"))
