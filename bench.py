@@ -11,7 +11,7 @@ backward reads a, h, grad_h and writes grad_a, grad_b = 20 B).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-configs] [--workload N]
 
---workload runs another of the synthetic configurations (1, 3, 4, 4f16, 5; or `long`) through the same timed
+--workload runs another of the synthetic configurations (1, 3, 4, 4f16, 5; or `long`, `long16`) through the same timed
 region instead of configuration 2 (used for the rocprofv3 summaries under profiles/).
 
 Prints ONE JSON line. Besides the contract fields it carries
@@ -68,6 +68,8 @@ WORKLOADS = {
     "4f16": (40, "configs[3]: forward + backward scan, fp16 storage / fp32 arithmetic, [B=16, C=1024, T=2048], "
                  "a=sigmoid(N(2,1)), b ~ N(0,0.5)"),
     "5": (5, "configs[4]: forward + backward fp32 scan, many short rows [B=256, C=512, T=64], a ~ U(0,1), b ~ N(0,1)"),
+    "long16": (60, "long-context shape in bf16 storage / fp32 arithmetic (not one of the five configurations): "
+                   "forward + backward scan, [B=1, C=2048, T=32768], a=sigmoid(N(0,1)), b ~ N(0,1)"),
     "long": (6, "long-context shape (not one of the five configurations): forward + backward fp32 scan, "
                 "[B=1, C=2048, T=32768], a=sigmoid(N(0,1)), b ~ N(0,1)"),
 }
@@ -93,9 +95,10 @@ def make_config(n, torch):
     elif n == 5:
         shape = (256, 512, 64)
         a, b = torch.rand(shape), torch.randn(shape)
-    elif n == 6:
+    elif n in (6, 60):
         shape = (1, 2048, 32768)
         a, b = torch.sigmoid(torch.randn(shape)), torch.randn(shape)
+        dtype = torch.float32 if n == 6 else torch.bfloat16
     elif n == 20:  # configuration 2's bytes in float64 (the reference's other storage type): half its T
         shape = (8, 2048, 2048)
         a, b = torch.sigmoid(torch.randn(shape)), torch.randn(shape)
