@@ -58,6 +58,16 @@ def test_header_is_plain_c():
                         "-o", os.path.join(d, "t.o")], check=True)
 
 
+def test_plain_c_consumer():
+    # tests/c_abi/cpu_abi_check: C99, no torch, no Python; built by `make -C tests/c_abi`.
+    import subprocess
+
+    binary = os.path.join(ROOT, "tests", "c_abi", "cpu_abi_check")
+    assert os.path.exists(binary), "tests/c_abi/cpu_abi_check is not built: run `make -C tests/c_abi`"
+    done = subprocess.run([binary], capture_output=True, text=True, timeout=120)
+    assert done.returncode == 0 and "cpu_abi_check: ok" in done.stdout, done.stdout + done.stderr
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape", SHAPES)
 def test_bit_identical_to_the_reference_loop(shape, dtype):
