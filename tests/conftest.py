@@ -8,8 +8,23 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 
+BUILT = [
+    os.path.join(ROOT, "scanscam_amd", "libscanscam_hip.so"),
+    os.path.join(ROOT, "scanscam_amd", "libscanscam_cpu.so"),
+    os.path.join(ROOT, "oracle", "libscan_oracle.so"),
+    os.path.join(ROOT, "tests", "c_abi", "abi_check"),
+    os.path.join(ROOT, "tests", "c_abi", "cpu_abi_check"),
+]
+
+
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    # The tests load what is built; a tree in which something was never built (a fresh clone:
+    # libraries are not committed) is built once here.
+    if not all(os.path.exists(p) for p in BUILT):
+        import __graft_entry__
+
+        __graft_entry__.build()
 
 
 @pytest.fixture(scope="session")
