@@ -401,6 +401,16 @@ def blocked_linear_scan_backward(
     return linear_scan_backward(x, y, z)
 
 
+# The reference keeps two earlier kernels beside the blocked one (one thread per row, and its
+# coalesced variant; cuda.py:16-31, 43-53) behind wrappers with the same contract. They compute the
+# same function, so here the names lead to the one implementation.
+simple_linear_scan_forward = blocked_linear_scan_forward
+coalesced_linear_scan_forward = blocked_linear_scan_forward
+simple_linear_scan_backward = blocked_linear_scan_backward
+# The probe scanscam/op.py reads from its GPU wrapper module (cuda.py:7-13).
+has_cuda_ops = has_hip_ops
+
+
 def _workspace_cl(L, batch: int, T: int, C: int, dtype: torch.dtype, direction: int, plan_ref,
                   device: torch.device) -> Tuple[Optional[torch.Tensor], int, int]:
     n = int(L.scanscam_workspace_bytes_cl(batch, T, C, _dtype_code(dtype), direction, plan_ref))

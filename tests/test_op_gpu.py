@@ -93,6 +93,28 @@ def test_wrapper_names_of_the_reference(gpu):
         hip.blocked_linear_scan_forward(a.long(), b.long())
 
 
+def test_reference_module_and_function_names(gpu):
+    # A test written for the reference (scanscam/cuda_test.py:19-126: each wrapper of scanscam.cuda
+    # against the tensor-level loop, N(0,1) inputs, atol 1e-4) runs against scanscam_amd.cuda unchanged.
+    from scanscam_amd import cuda
+    from scanscam_amd.baseline import naive_linear_scan_backward, naive_linear_scan_forward
+
+    assert cuda.has_cuda_ops
+    g = torch.Generator().manual_seed(5)
+    x, y, z = (torch.randn((16, 2, 5), generator=g).to(gpu) for _ in range(3))
+    want = naive_linear_scan_forward(x, y)
+    for fn in (cuda.simple_linear_scan_forward, cuda.coalesced_linear_scan_forward, cuda.blocked_linear_scan_forward):
+        assert torch.allclose(fn(x, y), want, atol=1e-4)
+    wa, wb = naive_linear_scan_backward(x, y, z)
+    for fn in (cuda.simple_linear_scan_backward, cuda.blocked_linear_scan_backward):
+        ga, gb = fn(x, y, z)
+        assert torch.allclose(ga, wa, atol=1e-4) and torch.allclose(gb, wb, atol=1e-4)
+    xt, yt, zt = (t.mT.contiguous() for t in (x, y, z))  # stored [B, T, C]
+    assert torch.allclose(cuda.transposed_linear_scan_forward(xt, yt, 8).mT, want, atol=1e-4)
+    ga, gb = cuda.transposed_linear_scan_backward(xt, yt, zt, 8)
+    assert torch.allclose(ga.mT, wa, atol=1e-4) and torch.allclose(gb.mT, wb, atol=1e-4)
+
+
 def test_runs_on_the_current_stream(gpu):
     s = torch.cuda.Stream(device=gpu)
     a = torch.rand(64, 4096, device=gpu)
