@@ -17,7 +17,10 @@ region instead of configuration 2 (used for the rocprofv3 summaries under profil
 Prints ONE JSON line. Besides the contract fields it carries
   roofline      the dominant kernel (backward) against the 8 TB/s HBM peak, its
                 duration measured with HIP events on the launch stream, bound to
-                the kernel itself (start and end of the kernel on the GPU);
+                the kernel itself (start and end of the kernel on the GPU): the
+                average over ten launches of the timed region, and in
+                `after_region` median, minimum and mean over 50 or more further
+                launches that all carry events;
   roofline_fwd  the same for the forward kernel;
   cpu_baseline  the reference's single-threaded CPU loop on the same tensors,
                 timed on this host (oracle/_ref if it was built, else the C
@@ -162,6 +165,28 @@ def time_kernels(sets, steps, warmup, hip, torch):
     fwd = [t[2].elapsed_ms() for t in timed.values()]
     bwd = [t[3].elapsed_ms() for t in timed.values()]
     return wall, statistics.fmean(fwd), statistics.fmean(bwd), min(fwd), min(bwd)
+
+
+def kernel_statistics(sets, launches, hip, torch):
+    """After the timed region: `launches` more steps, every launch with its own bound events.
+
+    Returns {"fwd": (median ms, min ms, mean ms), "bwd": ...} over all of them.
+    """
+    runs = []
+    for i in range(launches):
+        s = sets[i % len(sets)]
+        ef, eb = hip.KernelEvents(), hip.KernelEvents()
+        runs.append((hip.prepare_forward(s.a, s.b, s.h, events=ef),
+                     hip.prepare_backward(s.a, s.h, s.gh, s.ga, s.gb, events=eb), ef, eb))
+    for f, b, _, _ in runs:
+        f()
+        b()
+    torch.cuda.synchronize()
+    out = {}
+    for name, k in (("fwd", 2), ("bwd", 3)):
+        ms = [r[k].elapsed_ms() for r in runs]
+        out[name] = (statistics.median(ms), min(ms), statistics.fmean(ms))
+    return out
 
 
 def time_batches(sets, launches, warmup, hip, torch):
@@ -512,6 +537,7 @@ def main():
     nsets = max(1, min(64, -(-(1 << 30) // (6 * n * esize)))) if 6 * n * esize < (1 << 30) else 1
     sets = [first] + [first.clone(torch) for _ in range(nsets - 1)]
     wall, fwd_ms, bwd_ms, fwd_min, bwd_min = time_kernels(sets, args.steps, max(args.warmup, nsets), hip, torch)
+    stats = kernel_statistics(sets, max(50, args.steps), hip, torch)
     step_bytes = FWD_BYTES[esize] + BWD_BYTES[esize]
     fwd_gbps = FWD_BYTES[esize] * n / (fwd_ms * 1e-3) / 1e9
     bwd_gbps = BWD_BYTES[esize] * n / (bwd_ms * 1e-3) / 1e9
@@ -561,6 +587,8 @@ def main():
             "bytes_per_launch": BWD_BYTES[esize] * n,
             "avg_ms": round(bwd_ms, 4),
             "min_ms": round(bwd_min, 4),
+            "after_region": {"launches": max(50, args.steps), "median_ms": round(stats["bwd"][0], 4),
+                             "min_ms": round(stats["bwd"][1], 4), "mean_ms": round(stats["bwd"][2], 4)},
         },
         "roofline_fwd": {
             "kernel": kernel % "false" + " (forward)",
@@ -573,6 +601,8 @@ def main():
             "bytes_per_launch": FWD_BYTES[esize] * n,
             "avg_ms": round(fwd_ms, 4),
             "min_ms": round(fwd_min, 4),
+            "after_region": {"launches": max(50, args.steps), "median_ms": round(stats["fwd"][0], 4),
+                             "min_ms": round(stats["fwd"][1], 4), "mean_ms": round(stats["fwd"][2], 4)},
         },
     }
     op_ms = autograd_step(first, tuple(a.shape), args.steps, args.warmup, torch)
