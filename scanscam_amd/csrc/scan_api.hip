@@ -437,8 +437,14 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         if (g < kWave) l->group = g;
     }
 
+    // 16-bit storage moves half as many bytes per step of a narrow lane. Where there is only about one
+    // workgroup per CU (fewer than 512 of them) that leaves too little in flight, and a workgroup that walks
+    // all of T takes 16 steps per wave as well: forward +5 to +11 points of peak (bf16 [16, 4096, 1024]
+    // 48 -> 59 %, [128, 2048, 256] 56 -> 67 %), backward -2 to +4. With more workgroups, or rows too short to
+    // fill such tiles, it costs 2 to 10 points; fp32 gains nothing from it.
     const bool narrow_lane = l->vec < full;
-    l->steps = u.unroll ? u.unroll : (narrow_lane ? (l->kind != 0 ? 16 : 8) : ((l->kind != 0 && full <= 4) ? 8 : 4));
+    const bool long_steps = l->kind != 0 || (esize == 2 && rowgroups < 512 && T >= 1024);
+    l->steps = u.unroll ? u.unroll : (narrow_lane ? (long_steps ? 16 : 8) : ((l->kind != 0 && full <= 4) ? 8 : 4));
     if (!u.unroll && l->group <= 16 && narrow_lane) l->steps = 4;  // packed, 4 or more steps per instruction
     const bool steps_ok = (l->vec == full) ? (l->steps == 2 || l->steps == 4 || l->steps == 8)
                                            : (l->steps == 4 || l->steps == 8 || l->steps == 16);
