@@ -95,6 +95,13 @@ bool prefer_lookback_for_many_rows(int64_t rows, int nch, bool rev, int esize)
 {
     const int tpr = (nch + kTileChunks - 1) / kTileChunks;
     if (rows < 256 || tpr < 2 || rows * tpr < 2048) return false;
+    // Rows of two tiles whose second tile is mostly empty: the look-back kernel's workgroups for those tiles
+    // idle, and the row kernel with one workgroup fitted to the row (resolve: up to 16 waves x 4 chunks, one
+    // step) is faster -- fp32 [6710, 10000] (40 chunks = 1.25 tiles): 138 / 243 us against 149 / 254. The
+    // backward pass gains more from the look-back order and gives it up later (from 30 % of the two tiles'
+    // chunks unused; forward from 20 %). Rows of three tiles would take the row kernel two steps: not faster.
+    const int unused_pct = (tpr * kTileChunks - nch) * 100 / (tpr * kTileChunks);
+    if (tpr == 2 && unused_pct > (rev ? 30 : 20)) return false;
     const int64_t rounds = (rows + kComputeUnits - 1) / kComputeUnits;
     const bool ragged_rounds = rows * 100 < rounds * kComputeUnits * 93;  // the row kernel's CUs idle > 7 % of the time
     // Longer rows (tile-major order): only where the row kernel's rounds do not come out (+2 to +13 points).
@@ -171,18 +178,25 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
                 l.unroll = (l.vec == full && nch <= 8) ? 2 : 4;
                 l.wpr = 4;
                 l.waves = 4;
-            } else {
-                // Longer rows: a workgroup tile (waves x chunks per wave) that covers the row in one
-                // step, or in as few as possible -- each further step waits for the carry of the last.
+            } else if (nch <= 32) {
                 l.unroll = 4;
-                l.wpr = l.waves = nch <= 48 ? 8 : 16;
+                l.wpr = l.waves = 8;
+            } else {
+                // Longer rows: a workgroup tile (waves x 4 chunks) that covers the row in one step, or
+                // in as few as 16 waves allow -- each further step waits for the carry of the last --
+                // with just the waves those steps need: a row of 36 chunks takes 9 waves, not 8 waves
+                // twice or 16 waves of which 7 idle (fp32 [7456, 9000]: 138 / 250 us against 145 / 258).
+                // Below 33 chunks the fit gains nothing over 4 or 8 waves (measured).
+                l.unroll = 4;
+                const int steps = (nch + 63) / 64;
+                l.wpr = l.waves = (nch + steps * 4 - 1) / (steps * 4);
             }
         } else {
             if (!l.unroll) l.unroll = 4;
             if (!l.waves) l.waves = l.wpr ? l.wpr : 4;
             if (!l.wpr) l.wpr = l.waves;
         }
-        if (!is_pow2(l.wpr) || l.wpr > l.waves || l.waves % l.wpr != 0) return SCANSCAM_EPLAN;
+        if (l.wpr < 1 || l.wpr > l.waves || l.waves % l.wpr != 0) return SCANSCAM_EPLAN;
         const int rows_per_wg = l.waves / l.wpr;
         l.grid = (rows + rows_per_wg - 1) / rows_per_wg;
     } else if (l.mode == kModeLookback) {

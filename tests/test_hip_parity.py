@@ -235,6 +235,10 @@ def plans_for(dtype):
                     if waves % wpr == 0:
                         out.append(hip.Plan(mode=hip.MODE_ROW, vec=vec, unroll=unroll, waves=waves, waves_per_row=wpr))
                 out.append(hip.Plan(mode=hip.MODE_LOOKBACK, vec=vec, unroll=unroll, waves=waves))
+    # Workgroups fitted to a row: any number of waves per row, several such rows per workgroup.
+    for waves, wpr in ((3, 3), (9, 9), (13, 13), (15, 5), (12, 3), (6, 2)):
+        out.append(hip.Plan(mode=hip.MODE_ROW, vec=full, unroll=4, waves=waves, waves_per_row=wpr))
+        out.append(hip.Plan(mode=hip.MODE_ROW, vec=1, unroll=1, waves=waves, waves_per_row=wpr))
     return out
 
 
@@ -329,7 +333,9 @@ ROW, LOOKBACK = hip.MODE_ROW, hip.MODE_LOOKBACK
 AUTO_REGIMES = [
     (2048, 1280, (ROW, 4, 2), None),
     (2048, 4100, (ROW, 8, 4), None),          # 17 chunks: one step of an 8-wave tile
-    (2048, 12501, (LOOKBACK, 0, 4), None),    # 49 chunks = 2 tiles, element-aligned rows: tiles in row-major order
+    (2048, 10000, (ROW, 10, 4), None),        # 40 chunks = 1.25 tiles: one workgroup of 10 waves per row instead
+    (2048, 12501, (ROW, 13, 4), (LOOKBACK, 0, 4)),  # 49 chunks, 23 % of two tiles unused: only the backward pass stays
+    (2048, 14001, (LOOKBACK, 0, 4), None),    # 55 chunks = 2 tiles, element-aligned rows: tiles in row-major order
     (700, 20000, (LOOKBACK, 0, 4), None),     # 3 tiles per row, 2100 tiles
     (256, 131072, (ROW, 16, 4), (LOOKBACK, 0, 4)),  # 16 tiles per row: only the backward pass gains
     (600, 20000, (ROW, 16, 4), None),         # 1800 tiles: too small a problem for the look-back launch
