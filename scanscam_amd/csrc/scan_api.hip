@@ -81,33 +81,26 @@ constexpr int kRowMajorCounters = 4;
 bool row_major_order(int64_t rows, int tiles_per_row) { return rows >= 256 && tiles_per_row <= 16; }
 
 // Many rows of moderate length: from two tiles per row on, the look-back kernel in row-major order beats one
-// workgroup walking each row, which streams as many separate spans as there are rows in flight and whose
-// last round of workgroups leaves CUs idle. Measured at 16 M to 64 M elements: the backward pass gains +2 to
-// +15 points of peak for 2 to 16 tiles per row, whatever the storage type; the forward pass +1 to +8 up to 6
-// tiles (4 for 16-bit storage, nothing lost), and beyond that, up to 14 tiles, only where the row kernel's
-// 16-wave workgroups (one per CU) do not come out in full rounds (rows = 512 or 1024 do: there it keeps the
-// forward pass). A problem of fewer than 2048 tiles is too small to hide the extra launch that clears the
-// workspace. Rows of more than 16 tiles go to the look-back kernel (in tile-major order) only where the row
-// kernel's rounds do not come out.
+// workgroup walking each row, which streams as many separate spans as there are rows in flight, leaves CUs
+// idle in its last round of workgroups, and whose 16-wave steps seldom divide a row. Measured at 16 M to 128 M
+// elements, fp32 and bf16, with tiles fitted to the row (resolve): 2 to 15 tiles per row gain +2 to +20 % forward
+// and +9 to +30 % backward, also where the row kernel's workgroups come out in full rounds of 256; rows of 8
+// tiles (4 exact steps of the row kernel) tie forward. At 16 tiles the forward pass of the row kernel (8 exact
+// steps) is 5-8 % faster and keeps the shape unless its rounds do not come out; the backward pass still gains
+// 4-6 %. A problem of fewer than 2048 tiles is too small to hide the extra launch that clears the workspace.
+// Rows of more than 16 tiles go to the look-back kernel (in tile-major order) only where the row kernel's
+// rounds do not come out.
 constexpr int kComputeUnits = 256;  // MI355X
 
-bool prefer_lookback_for_many_rows(int64_t rows, int nch, bool rev, int esize)
+bool prefer_lookback_for_many_rows(int64_t rows, int nch, bool rev)
 {
     const int tpr = (nch + kTileChunks - 1) / kTileChunks;
     if (rows < 256 || tpr < 2 || rows * tpr < 2048) return false;
-    // Rows of two tiles whose second tile is mostly empty: the look-back kernel's workgroups for those tiles
-    // idle, and the row kernel with one workgroup fitted to the row (resolve: up to 16 waves x 4 chunks, one
-    // step) is faster -- fp32 [6710, 10000] (40 chunks = 1.25 tiles): 138 / 243 us against 149 / 254. The
-    // backward pass gains more from the look-back order and gives it up later (from 30 % of the two tiles'
-    // chunks unused; forward from 20 %). Rows of three tiles would take the row kernel two steps: not faster.
-    const int unused_pct = (tpr * kTileChunks - nch) * 100 / (tpr * kTileChunks);
-    if (tpr == 2 && unused_pct > (rev ? 30 : 20)) return false;
     const int64_t rounds = (rows + kComputeUnits - 1) / kComputeUnits;
     const bool ragged_rounds = rows * 100 < rounds * kComputeUnits * 93;  // the row kernel's CUs idle > 7 % of the time
-    // Longer rows (tile-major order): only where the row kernel's rounds do not come out (+2 to +13 points).
-    if (tpr > 16) return ragged_rounds;
-    if (rev || tpr <= (esize == 2 ? 4 : 6)) return true;
-    return tpr <= 14 && ragged_rounds;
+    if (rev && tpr <= 16) return true;
+    if (tpr <= 15) return true;
+    return ragged_rounds;
 }
 
 // Turns (shape, alignment, direction, optional user plan) into a launch. `aligned16` says
@@ -149,7 +142,7 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
         // From 256 rows on, one 16-wave workgroup per row fills the chip as well as tiles over
         // workgroups do and needs no carry hand-off between workgroups.
         else if (nch >= 64 && rows < 256) l.mode = kModeLookback;
-        else if (prefer_lookback_for_many_rows(rows, nch, rev, esize)) l.mode = kModeLookback;
+        else if (prefer_lookback_for_many_rows(rows, nch, rev)) l.mode = kModeLookback;
         else l.mode = kModeRow;
     }
 
@@ -169,24 +162,17 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
                 l.unroll = (l.vec == full) ? pow2_ceil(nch) : (nch == 1 ? 1 : 4);
                 l.wpr = 1;
                 l.waves = 4;
-            } else if (rows < 2048 && nch >= 16) {
-                // Few rows: as many waves per row as a workgroup holds.
-                l.unroll = nch >= 64 ? 4 : 1;
-                l.wpr = 16;
-                l.waves = 16;
             } else if (nch <= 16) {
                 l.unroll = (l.vec == full && nch <= 8) ? 2 : 4;
                 l.wpr = 4;
                 l.waves = 4;
-            } else if (nch <= 32) {
-                l.unroll = 4;
-                l.wpr = l.waves = 8;
             } else {
                 // Longer rows: a workgroup tile (waves x 4 chunks) that covers the row in one step, or
                 // in as few as 16 waves allow -- each further step waits for the carry of the last --
                 // with just the waves those steps need: a row of 36 chunks takes 9 waves, not 8 waves
                 // twice or 16 waves of which 7 idle (fp32 [7456, 9000]: 138 / 250 us against 145 / 258).
-                // Below 33 chunks the fit gains nothing over 4 or 8 waves (measured).
+                // Few rows as well: fewer steps count for more than more waves per row ([300, 16640]:
+                // 15.5 / 23.9 us with 9 waves x 4 chunks x 2 steps, 18.8 / 27.1 with 16 waves x 4 x 2).
                 l.unroll = 4;
                 const int steps = (nch + 63) / 64;
                 l.wpr = l.waves = (nch + steps * 4 - 1) / (steps * 4);
@@ -206,6 +192,12 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
         // longest for each other: 64 chunks there.
         l.unroll = u.unroll ? u.unroll : 4;
         l.waves = u.waves ? u.waves : (rows <= 16 && l.unroll <= 4 ? 16 : 8);
+        if (!u.waves && !u.unroll && rows > 16) {
+            // As many tiles as 8-wave tiles would take, but with only the waves they need: 75 chunks are 3
+            // tiles of 7 waves (84 chunk slots), not of 8 (96).
+            const int tiles = (nch + kTileChunks - 1) / kTileChunks;
+            l.waves = (nch + tiles * l.unroll - 1) / (tiles * l.unroll);
+        }
         const int tile_chunks = l.waves * l.unroll;
         out->tiles_per_row = (nch + tile_chunks - 1) / tile_chunks;
         // One ticket counter per row up to kMaxCounters; when rows do not divide

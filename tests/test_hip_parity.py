@@ -332,24 +332,30 @@ def test_short_rows_automatic(gpu, rows, T):
 ROW, LOOKBACK = hip.MODE_ROW, hip.MODE_LOOKBACK
 AUTO_REGIMES = [
     (2048, 1280, (ROW, 4, 2), None),
-    (2048, 4100, (ROW, 8, 4), None),          # 17 chunks: one step of an 8-wave tile
-    (2048, 10000, (ROW, 10, 4), None),        # 40 chunks = 1.25 tiles: one workgroup of 10 waves per row instead
-    (2048, 12501, (ROW, 13, 4), (LOOKBACK, 0, 4)),  # 49 chunks, 23 % of two tiles unused: only the backward pass stays
-    (2048, 14001, (LOOKBACK, 0, 4), None),    # 55 chunks = 2 tiles, element-aligned rows: tiles in row-major order
+    (2048, 4100, (ROW, 5, 4), None),          # 17 chunks: one step of a 5-wave workgroup
+    (2048, 10000, (LOOKBACK, 0, 4), None),    # 40 chunks = 2 tiles of 5 waves
+    (2048, 12501, (LOOKBACK, 0, 4), None),    # 49 chunks = 2 tiles of 7 waves, element-aligned rows: row-major order
     (700, 20000, (LOOKBACK, 0, 4), None),     # 3 tiles per row, 2100 tiles
     (256, 131072, (ROW, 16, 4), (LOOKBACK, 0, 4)),  # 16 tiles per row: only the backward pass gains
-    (600, 20000, (ROW, 16, 4), None),         # 1800 tiles: too small a problem for the look-back launch
-    (300, 81920, (LOOKBACK, 0, 4), None),     # 10 tiles per row, and 300 rows fill 256 CUs 1.17 times: forward too
-    (512, 81920, (ROW, 16, 4), (LOOKBACK, 0, 4)),  # two full rounds of row workgroups: the forward pass keeps them
-    (300, 4100, (ROW, 16, 1), None),
+    (600, 20000, (ROW, 10, 4), None),         # 1800 tiles: too small for the look-back launch; 79 chunks = 2 steps of 10 waves
+    (300, 81920, (LOOKBACK, 0, 4), None),     # 10 tiles per row
+    (512, 81920, (LOOKBACK, 0, 4), None),     # also where the row kernel's workgroups come out in full rounds
+    (300, 4100, (ROW, 5, 4), None),
     (270, 140000, (LOOKBACK, 0, 4), None),    # 18 tiles per row, 270 rows on 256 CUs: tile-major look-back
-    (300, 16640, (ROW, 16, 4), None),         # few rows, 65 chunks
+    (512, 140000, (ROW, 16, 4), None),        # 18 tiles per row in full rounds: the row kernel
+    (300, 16640, (ROW, 9, 4), None),          # few rows, 65 chunks: 2 steps of 9 waves
     (255, 16640, (LOOKBACK, 0, 4), None),     # fewer than 256 rows: tiles in tile-major order
 ]
 
 
 @pytest.mark.parametrize("rows,T,expect,expect_bwd", AUTO_REGIMES)
 def test_automatic_plan_regimes(gpu, rows, T, expect, expect_bwd):
+    if (rows, T) == (2048, 10000):
+        # Tiles and row workgroups are fitted to the row: 40 chunks are 2 look-back tiles of 5 waves, or,
+        # with the row kernel forced, one workgroup of 10 waves.
+        assert hip.resolve_plan(rows, T, torch.float32, hip.FORWARD).waves == 5
+        forced = hip.resolve_plan(rows, T, torch.float32, hip.FORWARD, hip.Plan(mode=ROW))
+        assert (forced.waves, forced.waves_per_row, forced.unroll) == (10, 10, 4)
     plan = hip.resolve_plan(rows, T, torch.float32, hip.FORWARD)
     assert (plan.mode, plan.waves_per_row, plan.unroll) == expect, plan
     plan = hip.resolve_plan(rows, T, torch.float32, hip.BACKWARD)
