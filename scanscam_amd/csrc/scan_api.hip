@@ -64,6 +64,7 @@ struct Resolved {
     int tiles_per_row;
     int counters;
     int row_major;       // a counter's tickets walk its rows one after the other (see resolve)
+    int line_shift;      // chunks laid out from the 128-byte line border before each row's start (see resolve)
     int64_t super_base;  // word offset of the super-tile descriptors
     size_t ws_bytes;
 };
@@ -103,9 +104,11 @@ bool prefer_lookback_for_many_rows(int64_t rows, int nch, bool rev)
     return ragged_rounds;
 }
 
-// Turns (shape, alignment, direction, optional user plan) into a launch. `aligned16` says
+// Turns (shape, alignment, direction, optional user plan) into a launch. `aligned128` says whether every
+// row of every tensor starts on a 128-byte line border; `aligned16` says
 // whether every tensor base is 16-byte aligned.
-int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool aligned16, bool rev, Resolved *out)
+int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool aligned16, bool aligned128, bool rev,
+            Resolved *out)
 {
     const int esize = elem_size(dtype);
     if (esize == 0) return SCANSCAM_EDTYPE;
@@ -126,7 +129,17 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
     if (l.ragged && !ragged_possible) return SCANSCAM_EPLAN;
 
     const int64_t chunk = (int64_t)kWave * l.vec;
-    const int64_t nch64 = (T + chunk - 1) / chunk;
+    // Rows that start inside a 128-byte line, longer than one chunk: the ROW and LOOKBACK kernels lay their
+    // chunks out from the line border before each row's start, so that a wave's loads and stores cover
+    // whole lines (fp32 [23140, 2900], rows 16-byte aligned only: 129 / 220 us, 136 / 250 us without). A row
+    // then takes up to one line's worth of vector slots more, which is not worth a fifth chunk for rows of
+    // up to four (one wave per row: [67108, 1000] 128 us forward without, 150 with).
+    const int64_t lead = 128 / ((int64_t)l.vec * esize) - 1;
+    const int64_t nvec = (T + l.vec - 1) / l.vec;
+    const int64_t nch_plain = (T + chunk - 1) / chunk, nch_lines = (nvec + lead + kWave - 1) / kWave;
+    out->line_shift = (!aligned128 && !l.ragged && T > chunk && u.mode != kModeSmall &&
+                       (nch_plain > 4 || nch_lines <= 4)) ? 1 : 0;
+    const int64_t nch64 = out->line_shift ? nch_lines : nch_plain;
     const int nch = (int)nch64;
     out->nch = nch;
     out->tiles_per_row = 0;
@@ -138,7 +151,7 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
 
     l.mode = u.mode;
     if (l.mode == SCANSCAM_MODE_AUTO) {
-        if (T <= chunk) l.mode = kModeSmall;
+        if (T <= chunk) l.mode = kModeSmall;  // (line_shift is 0 here)
         // From 256 rows on, one 16-wave workgroup per row fills the chip as well as tiles over
         // workgroups do and needs no carry hand-off between workgroups.
         else if (nch >= 64 && rows < 256) l.mode = kModeLookback;
@@ -289,15 +302,17 @@ int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y
 
     // 16-byte vectors need every row of every tensor to start on a 16-byte border.
     const int full = 16 / esize;
-    bool aligned16 = true;
+    bool aligned16 = true, aligned128 = true;
+    const int line = 128 / esize;  // elements per 128-byte line
     for (int k = 0; k < 5; k++) {
         if (!used[k]) continue;
         if (!aligned_to(ptrs[k], (size_t)esize)) return SCANSCAM_EALIGN;
         aligned16 = aligned16 && aligned_to(ptrs[k], 16) && s0[k] % full == 0 && s1[k] % full == 0;
+        aligned128 = aligned128 && aligned_to(ptrs[k], 128) && s0[k] % line == 0 && s1[k] % line == 0;
     }
 
     Resolved r;
-    const int rc = resolve(plan, rows, T, dtype, aligned16, rev, &r);
+    const int rc = resolve(plan, rows, T, dtype, aligned16, aligned128, rev, &r);
     if (rc != SCANSCAM_OK) return rc;
 
     ScanArgs args;
@@ -319,6 +334,7 @@ int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y
     args.tiles_per_row = r.tiles_per_row;
     args.counters = r.counters;
     args.row_major = r.row_major;
+    args.line_shift = r.line_shift;
     args.desc_base = r.counters * kCounterStride;
     args.super_base = r.super_base;
     args.spin_limit = (plan && plan->spin_limit > 0) ? plan->spin_limit : scanscam::kSpinLimit;
@@ -571,9 +587,10 @@ size_t workspace_for(int64_t rows, int64_t T, int dtype, int direction, const sc
     // The caller's pointers are not known yet: cover both the 16-byte aligned
     // and the unaligned choice.
     size_t need = 0;
-    for (int al = 0; al < 2; al++) {
+    for (int al = 0; al < 3; al++) {  // element-aligned, 16-byte aligned, 128-byte aligned rows
         Resolved r;
-        if (resolve(plan, rows, T, dtype, al != 0, direction == SCANSCAM_BACKWARD, &r) == SCANSCAM_OK && r.ws_bytes > need)
+        if (resolve(plan, rows, T, dtype, al >= 1, al == 2, direction == SCANSCAM_BACKWARD, &r) == SCANSCAM_OK &&
+            r.ws_bytes > need)
             need = r.ws_bytes;
     }
     return need;
@@ -705,7 +722,10 @@ int scanscam_resolve_plan(int64_t rows, int64_t T, int dtype, int direction, con
 {
     if (!out) return SCANSCAM_EINVAL;
     Resolved r;
-    const int rc = resolve(plan, rows, T, dtype, true, direction == SCANSCAM_BACKWARD, &r);
+    // Dense tensors on allocation borders: rows start on line borders exactly when a row is whole lines.
+    const int esize = elem_size(dtype);
+    const bool lines = esize != 0 && (T * esize) % 128 == 0;
+    const int rc = resolve(plan, rows, T, dtype, true, lines, direction == SCANSCAM_BACKWARD, &r);
     if (rc != SCANSCAM_OK) return rc;
     out->mode = r.l.mode;
     out->vec = r.l.vec;

@@ -72,6 +72,7 @@ struct ScanArgs {
     int32_t tiles_per_row;  // LOOKBACK: tiles per row
     int32_t counters;       // LOOKBACK: number of ticket counters (row r uses counter r % counters)
     int32_t row_major;      // LOOKBACK: a counter's tickets walk its rows one after the other
+    int32_t line_shift;     // ROW, LOOKBACK: chunks are laid out from the 128-byte line border before each row's start
     int32_t desc_base;      // LOOKBACK: first tile-descriptor word of the workspace
     int64_t super_base;     // LOOKBACK: first super-tile-descriptor word of the workspace
     int32_t spin_limit;     // LOOKBACK: polls before a wait gives up
@@ -282,6 +283,17 @@ struct WaveTile {
     {
 #pragma unroll
         for (int k = 0; k < 5; k++) base[k] = group * p.s0[k] + row * p.s1[k];
+    }
+    // Rows that start inside a 128-byte line (a row length that is no multiple of it): laying the
+    // chunks out from the line border before the row's start keeps every load and store instruction of
+    // a wave on whole lines. Returns how many vectors lie between that border and the row's start (in
+    // tensor a; the other tensors of a dense call share it). Vector m of the row is then slot
+    // m + shift of the chunks; slots before the row and past its end are masked like any other.
+    __device__ __forceinline__ int line_shift(const ScanArgs &p) const
+    {
+        if (RAGGED || GROUPED || !p.line_shift) return 0;
+        const uint64_t byte = (uint64_t)reinterpret_cast<uintptr_t>(p.a) + (uint64_t)base[0] * sizeof(ST);
+        return (int)((byte & 127u) / (VEC * sizeof(ST)));
     }
     template <int K> __device__ __forceinline__ int64_t at(const ScanArgs &p, int u) const
     {
@@ -558,13 +570,14 @@ __global__ __launch_bounds__(MAXT) void scan_row_kernel(const ScanArgs p)
     w.set_row(p, blockIdx.y, row_ok ? row : 0);
     CT hp[REV ? U : 1][VEC];
     CT row_carry = CT(0);
+    const int shift = w.line_shift(p);
 
     for (int it = 0; it < ntiles; it++) {
         const int chunk0 = (it * wpr + wr) * U;
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            const int s = (chunk0 + u) * kWave + lane;  // vector index in scan order
-            const int m = REV ? nvp - 1 - s : s;
+            const int s = (chunk0 + u) * kWave + lane;  // slot in scan order
+            const int m = (REV ? nvp - 1 - s : s) - shift;  // vector index in the row
             w.m[u] = m;
             w.valid[u] = row_ok && m >= 0 && (int64_t)m * VEC < p.T;
             w.col[u] = w.valid[u] ? m * VEC : 0;
@@ -847,10 +860,11 @@ __global__ __launch_bounds__(MAXT) void scan_lookback_kernel(const ScanArgs p)
     const int64_t group = row / p.n1;
     w.set_row(p, group, row - group * p.n1);
     CT hp[REV ? U : 1][VEC];
+    const int shift = w.line_shift(p);
 #pragma unroll
     for (int u = 0; u < U; u++) {
         const int s = (chunk0 + u) * kWave + lane;
-        const int m = REV ? nvp - 1 - s : s;
+        const int m = (REV ? nvp - 1 - s : s) - shift;
         w.m[u] = m;
         w.valid[u] = m >= 0 && (int64_t)m * VEC < p.T;
         w.col[u] = w.valid[u] ? m * VEC : 0;

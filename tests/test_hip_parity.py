@@ -372,6 +372,40 @@ def test_automatic_plan_regimes(gpu, rows, T, expect, expect_bwd):
     assert rel_err(to_np(got_ga), ga, prev_abs(h)) <= FP32_BAR
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float64])
+def test_rows_that_start_inside_a_cache_line(gpu, dtype):
+    # Rows of a length that is a multiple of 16 bytes but not of 128: every row starts at another place
+    # inside a 128-byte line, and the row and look-back kernels lay their chunks out from the line
+    # border before it (slots before the row's start are masked). Dense tensors and views at every
+    # 16-byte offset of a line, both directions, automatic and forced plans.
+    full = full_vec(dtype)
+    bar = bar_for(dtype)
+    g = seeded(91)
+    chunk = 64 * full
+    plans = [None, hip.Plan(mode=hip.MODE_ROW, vec=full, unroll=2, waves=3, waves_per_row=3),
+             hip.Plan(mode=hip.MODE_ROW, vec=1, unroll=4, waves=4, waves_per_row=2),
+             hip.Plan(mode=hip.MODE_LOOKBACK, vec=full, unroll=1, waves=2),
+             hip.Plan(mode=hip.MODE_LOOKBACK, vec=full, unroll=4, waves=5)]
+    for rows, T in [(37, 4 * chunk + 5 * full), (9, 11 * chunk + full), (300, 40 * chunk + 3 * full), (3, 130 * chunk - full)]:
+        for off in (0, full, 3 * full, 7 * full):
+            def view(fn):
+                buf = fn((rows * T + 8 * full,), generator=g, dtype=torch.float64).to(dtype).to(gpu)
+                return buf[off:off + rows * T].view(rows, T)
+            a, b, gh = view(torch.rand), view(torch.randn), view(torch.randn)
+            h = oracle.fwd(upcast(a.cpu()), upcast(b.cpu()))
+            hs = torch.from_numpy(h).to(dtype).to(gpu)
+            ga, gb = oracle.bwd(upcast(a.cpu()), upcast(hs.cpu()), upcast(gh.cpu()))
+            hp = prev_abs(upcast(hs.cpu()))
+            for plan in plans:
+                if rows >= 300 and plan is not None and plan.vec == 1:
+                    continue
+                print(f"case lines {dtype} rows={rows} T={T} offset={off} {plan}", flush=True)
+                assert rel_err(to_np(hip.linear_scan_forward(a, b, plan)), h) <= bar
+                got_ga, got_gb = hip.linear_scan_backward(a, hs, gh, plan)
+                assert rel_err(to_np(got_gb), gb) <= bar
+                assert rel_err(to_np(got_ga), ga, hp) <= bar
+
+
 def test_unaligned_base_pointers(gpu):
     # Views that start 4 bytes into an allocation: the library must fall back to
     # element-wise loads, not fault or misread.
