@@ -176,8 +176,11 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
                 l.wpr = 1;
                 l.waves = 4;
             } else if (nch <= 16) {
-                l.unroll = (l.vec == full && nch <= 8) ? 2 : 4;
-                l.wpr = 4;
+                // 4 waves per workgroup. 5-6 chunks: 2 chunks per wave; 7-8: 4 chunks per wave and two
+                // rows per workgroup (fp32 [32768, 2048] 122 / 211 us against 124 / 215 with 2 chunks per
+                // wave and one row, bf16 [16384, 4096] 63.2 / 109.5 against 65.0 / 111.3); 9-16: one row.
+                l.unroll = (l.vec == full && nch <= 6) ? 2 : 4;
+                l.wpr = (l.vec == full && (nch == 7 || nch == 8)) ? 2 : 4;
                 l.waves = 4;
             } else {
                 // Longer rows: a workgroup tile (waves x 4 chunks) that covers the row in one step, or
