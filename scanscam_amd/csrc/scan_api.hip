@@ -134,11 +134,11 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
     // whole lines (fp32 [23140, 2900], rows 16-byte aligned only: 129 / 220 us, 136 / 250 us without). A row
     // then takes up to one line's worth of vector slots more, which is not worth a fifth chunk for rows of
     // up to four (one wave per row: [67108, 1000] 128 us forward without, 150 with).
-    const int64_t lead = 128 / ((int64_t)l.vec * esize) - 1;
-    const int64_t nvec = (T + l.vec - 1) / l.vec;
-    const int64_t nch_plain = (T + chunk - 1) / chunk, nch_lines = (nvec + lead + kWave - 1) / kWave;
-    out->line_shift = (!aligned128 && !l.ragged && T > chunk && u.mode != kModeSmall &&
-                       (nch_plain > 4 || nch_lines <= 4)) ? 1 : 0;
+    // (Element-aligned rows: the border is counted in elements, and the vectors then sit on 16-byte borders.)
+    const int64_t lead = l.ragged ? 128 / esize - 1 : 128 / ((int64_t)l.vec * esize) - 1;
+    const int64_t nvec = l.ragged ? (T + lead + l.vec - 1) / l.vec : (T + l.vec - 1) / l.vec + lead;
+    const int64_t nch_plain = (T + chunk - 1) / chunk, nch_lines = (nvec + kWave - 1) / kWave;
+    out->line_shift = (!aligned128 && T > chunk && u.mode != kModeSmall && (nch_plain > 4 || nch_lines <= 4)) ? 1 : 0;
     const int64_t nch64 = out->line_shift ? nch_lines : nch_plain;
     const int nch = (int)nch64;
     out->nch = nch;
@@ -182,6 +182,8 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
                 l.unroll = (l.vec == full && nch <= 6) ? 2 : 4;
                 l.wpr = (l.vec == full && (nch == 7 || nch == 8)) ? 2 : 4;
                 l.waves = 4;
+                // Element-aligned rows of 9-12 chunks: 3 waves (bf16 [16380, 4097]: 76 / 123 us, 96 / 149 with 4).
+                if (l.ragged && nch > 8 && nch <= 12) l.wpr = l.waves = 3;
             } else {
                 // Longer rows: a workgroup tile (waves x 4 chunks) that covers the row in one step, or
                 // in as few as 16 waves allow -- each further step waits for the carry of the last --

@@ -139,20 +139,21 @@ template <typename ST, int VEC> struct Vec {
     {
         __builtin_nontemporal_store(r, reinterpret_cast<raw_unaligned_t *>(p));
     }
-    // The first n (< VEC) elements only, the rest zero: the partial vector at the end of a row.
-    static __device__ __forceinline__ raw_t load_head(const ST *p, int n)
+    // The components whose bit is set in `inside` only, the rest zero: the partial vector at the start
+    // or the end of a row (the others lie outside the row and are neither read nor written).
+    static __device__ __forceinline__ raw_t load_part(const ST *p, uint32_t inside)
     {
         Elems<ST, VEC> e;
 #pragma unroll
-        for (int k = 0; k < VEC; k++) e.e[k] = (k < n) ? p[k] : (ST)0.0f;
+        for (int k = 0; k < VEC; k++) e.e[k] = ((inside >> k) & 1u) ? p[k] : (ST)0.0f;
         return __builtin_bit_cast(raw_t, e);
     }
-    static __device__ __forceinline__ void store_head(ST *p, raw_t r, int n)
+    static __device__ __forceinline__ void store_part(ST *p, raw_t r, uint32_t inside)
     {
         const Elems<ST, VEC> e = __builtin_bit_cast(Elems<ST, VEC>, r);
 #pragma unroll
         for (int k = 0; k < VEC; k++)
-            if (k < n) p[k] = e.e[k];
+            if ((inside >> k) & 1u) p[k] = e.e[k];
     }
     // For data that is read a second time soon: left to the caches' normal policy.
     static __device__ __forceinline__ raw_t load_cached(const ST *p) { return *reinterpret_cast<const raw_t *>(p); }
@@ -259,20 +260,21 @@ __device__ __forceinline__ void wave_scan(CT &A, CT &B, int j)
 // ---------------------------------------------------------------------------
 // With RAGGED, rows may start at any element (their length need not be a
 // multiple of VEC, bases need not be 16-byte aligned): vectors are loaded and
-// stored element-aligned, and the last vector of a row may hold fewer than VEC
-// elements (`count`), the rest being masked to the identity.
+// stored element-aligned, and the first and the last vector of a row may hold
+// fewer than VEC of its elements (bit mask `inside`), the rest being masked to
+// the identity.
 template <typename ST, int VEC, int U, bool REV, bool GROUPED, bool CHAIN, bool RAGGED = false, bool LEAN = false>
 struct WaveTile {
     using V = Vec<ST, VEC>;
     using raw_t = typename V::raw_t;
     using CT = typename ComputeOf<ST>::type;
+    static constexpr uint32_t kAll = (1u << VEC) - 1u;  // all components of a vector
 
     // Where this lane's vector of chunk u lives. Lanes without a vector point at element 0 of an
     // existing row (col = 0), which is always readable.
     int32_t col[U];  // first element of the vector inside its row (m*VEC)
-    int32_t m[U];    // vector index inside the row
     bool valid[U];   // inside the row (and the row exists)
-    int32_t count[RAGGED ? U : 1];  // RAGGED: elements of the vector inside the row (1..VEC)
+    uint32_t inside[RAGGED ? U : 1];  // RAGGED: bit k set = component k of the vector lies inside the row
     // Start of the row in tensor k = 0..4 (a, x, h, y0, y1), in elements. The ROW and LOOKBACK kernels
     // have one row per wave (wave-uniform); in the SMALL kernel `base` is the start of the group and
     // the row of chunk u, which differs from lane to lane, is added per access.
@@ -289,11 +291,30 @@ struct WaveTile {
     // a wave on whole lines. Returns how many vectors lie between that border and the row's start (in
     // tensor a; the other tensors of a dense call share it). Vector m of the row is then slot
     // m + shift of the chunks; slots before the row and past its end are masked like any other.
+    // With RAGGED (rows start at any element) the shift is counted in elements: the vectors then start
+    // on 16-byte borders of tensor a, and the first vector of a row may lie partly before its start.
     __device__ __forceinline__ int line_shift(const ScanArgs &p) const
     {
-        if (RAGGED || GROUPED || !p.line_shift) return 0;
+        if (GROUPED || !p.line_shift) return 0;
         const uint64_t byte = (uint64_t)reinterpret_cast<uintptr_t>(p.a) + (uint64_t)base[0] * sizeof(ST);
-        return (int)((byte & 127u) / (VEC * sizeof(ST)));
+        return (int)((byte & 127u) / ((RAGGED ? 1 : VEC) * sizeof(ST)));
+    }
+
+    // Places slot q of the chunks (a vector index counted from the row's line border) in the row.
+    __device__ __forceinline__ void place(int u, int q, int shift, bool row_ok, int T)
+    {
+        if (!RAGGED) {
+            const int m = q - shift;
+            valid[u] = row_ok && m >= 0 && (int64_t)m * VEC < T;
+            col[u] = valid[u] ? m * VEC : 0;
+        } else {
+            const int64_t x0 = (int64_t)q * VEC - shift;  // element of the row at component 0
+            const int64_t l = x0 < 0 ? -x0 : 0, h = T - x0;
+            const int lo = (int)(l < VEC ? l : VEC), hi = (int)(h < 0 ? 0 : (h < VEC ? h : VEC));
+            valid[u] = row_ok && q >= 0 && lo < hi;
+            inside[u] = valid[u] ? ((kAll >> (VEC - hi)) & (kAll << lo) & kAll) : 0u;
+            col[u] = valid[u] ? (int32_t)x0 : 0;
+        }
     }
     template <int K> __device__ __forceinline__ int64_t at(const ScanArgs &p, int u) const
     {
@@ -305,16 +326,16 @@ struct WaveTile {
     __device__ __forceinline__ raw_t fetch(const ST *p, int u) const
     {
         if (!RAGGED) return V::load(p);
-        return count[u] >= VEC ? V::load_unaligned(p) : V::load_head(p, count[u]);
+        return inside[u] == kAll ? V::load_unaligned(p) : V::load_part(p, inside[u]);
     }
     __device__ __forceinline__ void put(ST *p, raw_t r, int u) const
     {
         if (!RAGGED) {
             V::store(p, r);
-        } else if (count[u] >= VEC) {
+        } else if (inside[u] == kAll) {
             V::store_unaligned(p, r);
         } else {
-            V::store_head(p, r, count[u]);
+            V::store_part(p, r, inside[u]);
         }
     }
 
@@ -363,8 +384,8 @@ struct WaveTile {
                 // inner ones are taken from the neighbouring chunk's registers in reduce().
                 const bool need_a = !CHAIN || u == 0;
                 const bool need_h = !CHAIN || u == U - 1;
-                if (need_a && valid[u] && j == 0 && (m[u] + 1) * VEC < p.T) edge_a[u] = (CT)a[at<0>(p, u) + VEC];
-                if (need_h && valid[u] && j == jlast && m[u] > 0) edge_h[u] = (CT)h[at<2>(p, u) - 1];
+                if (need_a && valid[u] && j == 0 && col[u] + VEC < p.T) edge_a[u] = (CT)a[at<0>(p, u) + VEC];
+                if (need_h && valid[u] && j == jlast && col[u] > 0) edge_h[u] = (CT)h[at<2>(p, u) - 1];
             }
         }
     }
@@ -401,7 +422,7 @@ struct WaveTile {
         if (!REV) {
 #pragma unroll
             for (int k = 0; k < VEC; k++) {
-                const bool in_row = RAGGED ? (valid[u] && k < count[u]) : valid[u];
+                const bool in_row = RAGGED ? ((inside[u] >> k) & 1u) != 0 : valid[u];
                 G[k] = in_row ? fa[k] : CT(1);
                 X[k] = fx[k];  // zero-filled where invalid
             }
@@ -425,7 +446,7 @@ struct WaveTile {
                 const CT gk = (k == 0) ? a_next : fa[(VEC - k) % VEC];
                 // Scan position k is element VEC-1-k of the vector; past the row's end it is the identity
                 // (its a and gh read as 0, so the element below it sees gate 0, as t = T-1 must).
-                const bool in_row = RAGGED ? (valid[u] && VEC - 1 - k < count[u]) : valid[u];
+                const bool in_row = RAGGED ? ((inside[u] >> (VEC - 1 - k)) & 1u) != 0 : valid[u];
                 G[k] = in_row ? gk : CT(1);
                 X[k] = fx[VEC - 1 - k];
                 HP[k] = (k == VEC - 1) ? h_prev : fh[(VEC - 2 - k) < 0 ? 0 : (VEC - 2 - k)];
@@ -577,11 +598,7 @@ __global__ __launch_bounds__(MAXT) void scan_row_kernel(const ScanArgs p)
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const int s = (chunk0 + u) * kWave + lane;  // slot in scan order
-            const int m = (REV ? nvp - 1 - s : s) - shift;  // vector index in the row
-            w.m[u] = m;
-            w.valid[u] = row_ok && m >= 0 && (int64_t)m * VEC < p.T;
-            w.col[u] = w.valid[u] ? m * VEC : 0;
-            if (RAGGED) w.count[u] = p.T - m * VEC;
+            w.place(u, REV ? nvp - 1 - s : s, shift, row_ok, p.T);
         }
         w.load(p, lane, kWave - 1);
         w.reduce(lane, kWave - 1, hp);
@@ -632,7 +649,6 @@ __global__ __launch_bounds__(MAXT) void scan_small_kernel(const ScanArgs p)
     for (int u = 0; u < U; u++) {
         const int64_t row = row0 + (int64_t)u * rows_per_chunk;
         const int m = REV ? G - 1 - j : j;
-        w.m[u] = m;
         w.valid[u] = row < p.rows && m * VEC < p.T;
         w.rowi[u] = w.valid[u] ? row : 0;
         w.col[u] = w.valid[u] ? m * VEC : 0;
@@ -864,11 +880,7 @@ __global__ __launch_bounds__(MAXT) void scan_lookback_kernel(const ScanArgs p)
 #pragma unroll
     for (int u = 0; u < U; u++) {
         const int s = (chunk0 + u) * kWave + lane;
-        const int m = (REV ? nvp - 1 - s : s) - shift;
-        w.m[u] = m;
-        w.valid[u] = m >= 0 && (int64_t)m * VEC < p.T;
-        w.col[u] = w.valid[u] ? m * VEC : 0;
-        if (RAGGED) w.count[u] = p.T - m * VEC;
+        w.place(u, REV ? nvp - 1 - s : s, shift, true, p.T);
     }
     w.load(p, lane, kWave - 1);
     w.reduce(lane, kWave - 1, hp);

@@ -334,7 +334,7 @@ AUTO_REGIMES = [
     (2048, 1280, (ROW, 4, 2), None),
     (2048, 4100, (ROW, 5, 4), None),          # 17 chunks: one step of a 5-wave workgroup
     (2048, 10000, (LOOKBACK, 0, 4), None),    # 40 chunks = 2 tiles of 5 waves
-    (2048, 12501, (LOOKBACK, 0, 4), None),    # 49 chunks = 2 tiles of 7 waves, element-aligned rows: row-major order
+    (2048, 12501, (LOOKBACK, 0, 4), None),    # element-aligned rows, 50 chunks = 2 tiles of 7 waves, row-major order
     (700, 20000, (LOOKBACK, 0, 4), None),     # 3 tiles per row, 2100 tiles
     (256, 131072, (ROW, 16, 4), (LOOKBACK, 0, 4)),  # 16 tiles per row: only the backward pass gains
     (600, 20000, (ROW, 10, 4), None),         # 1800 tiles: too small for the look-back launch; 79 chunks = 2 steps of 10 waves
