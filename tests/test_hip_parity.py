@@ -312,7 +312,7 @@ def test_empty_inputs(gpu):
         assert ga.shape == a.shape and gb.shape == a.shape
 
 
-@pytest.mark.parametrize("T", [1, 2, 3, 4, 63, 64, 65, 255, 256, 257, 260])
+@pytest.mark.parametrize("T", [1, 2, 3, 4, 63, 64, 65, 229, 231, 250, 255, 256, 257, 260])
 @pytest.mark.parametrize("rows", [1, 2, 129])
 def test_short_rows_automatic(gpu, rows, T):
     g = seeded(rows * 1000 + T)
@@ -325,6 +325,27 @@ def test_short_rows_automatic(gpu, rows, T):
     got_ga, got_gb = run_bwd(gpu, a, torch.from_numpy(h), gh)
     assert rel_err(to_np(got_gb), gb) <= FP32_BAR
     assert rel_err(to_np(got_ga), ga, prev_abs(h)) <= FP32_BAR
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float64])
+@pytest.mark.parametrize("T", [29, 57, 59, 461, 463, 500, 511])
+def test_short_element_aligned_rows_other_types(gpu, dtype, T):
+    # Rows of odd length around the border (nine tenths of a chunk: 461 elements of 16-bit storage, 116 of
+    # float64... the float64 lengths here are 29, 57, 59) from which 16-byte lanes with a masked end take
+    # over from one element per lane.
+    rows = 131
+    g = seeded(4000 + T)
+    a = torch.rand((rows, T), generator=g, dtype=torch.float64).to(dtype)
+    b = torch.randn((rows, T), generator=g, dtype=torch.float64).to(dtype)
+    gh = torch.randn((rows, T), generator=g, dtype=torch.float64).to(dtype)
+    bar = bar_for(dtype)
+    h = oracle.fwd(upcast(a), upcast(b))
+    assert rel_err(to_np(run_fwd(gpu, a, b)), h) <= bar
+    hs = torch.from_numpy(h).to(dtype)
+    ga, gb = oracle.bwd(upcast(a), upcast(hs), upcast(gh))
+    got_ga, got_gb = run_bwd(gpu, a, hs, gh)
+    assert rel_err(to_np(got_gb), gb) <= bar
+    assert rel_err(to_np(got_ga), ga, prev_abs(upcast(hs))) <= bar
 
 
 # One shape per branch of the automatic plan for rows longer than a chunk: (rows, T) -> the
