@@ -119,13 +119,14 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
 
     Launch &l = out->l;
     l = Launch{0, 0, 0, 0, 1, 64, 0, false, 1};
-    // The full 16-byte vector needs rows that start on 16-byte borders -- or, for rows longer than one
-    // chunk, the element-aligned ("ragged") variants of the ROW and LOOKBACK kernels.
+    // The full 16-byte vector needs rows that start on 16-byte borders -- or the element-aligned ("ragged")
+    // variants of the kernels: ROW and LOOKBACK for rows of at least nine tenths of a chunk (on shorter rows
+    // most of their lanes would idle), SMALL for rows of 4 vectors to one chunk (shorter ones lose nothing
+    // with one element per lane).
     const bool vec_aligned = aligned16 && (T % full == 0);
-    // (Rows within a tenth of a chunk of its length too: 16-byte lanes with a masked end beat one element per
-    // lane there -- bf16 [134217, 500] 236 / 331 us -> 98 / 147 us, fp32 [268435, 250] 143 / 285 -> 131 / 244 --
-    // but not on shorter rows, where most of the lanes would idle.)
-    const bool ragged_possible = full > 1 && T * 10 >= (int64_t)kWave * full * 9 && u.mode != kModeSmall;
+    const bool small_rows = u.mode == kModeSmall || (u.mode == SCANSCAM_MODE_AUTO && T <= (int64_t)kWave * full);
+    const bool ragged_possible = full > 1 && (small_rows ? (T >= 4 * full && T <= (int64_t)kWave * full)
+                                                         : T * 10 >= (int64_t)kWave * full * 9);
     l.vec = u.vec ? u.vec : ((vec_aligned || ragged_possible) ? full : 1);
     if (l.vec != 1 && l.vec != full) return SCANSCAM_EPLAN;
     l.ragged = l.vec == full && full != 1 && !vec_aligned;
@@ -141,7 +142,7 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
     const int64_t lead = l.ragged ? 128 / esize - 1 : 128 / ((int64_t)l.vec * esize) - 1;
     const int64_t nvec = l.ragged ? (T + lead + l.vec - 1) / l.vec : (T + l.vec - 1) / l.vec + lead;
     const int64_t nch_plain = (T + chunk - 1) / chunk, nch_lines = (nvec + kWave - 1) / kWave;
-    out->line_shift = (!aligned128 && (T > chunk || l.ragged) && u.mode != kModeSmall && (nch_plain > 4 || nch_lines <= 4)) ? 1 : 0;
+    out->line_shift = (!aligned128 && !small_rows && (T > chunk || l.ragged) && (nch_plain > 4 || nch_lines <= 4)) ? 1 : 0;
     const int64_t nch64 = out->line_shift ? nch_lines : nch_plain;
     const int nch = (int)nch64;
     out->nch = nch;
@@ -154,7 +155,7 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
 
     l.mode = u.mode;
     if (l.mode == SCANSCAM_MODE_AUTO) {
-        if (T <= chunk && !l.ragged) l.mode = kModeSmall;  // (line_shift is 0 here)
+        if (T <= chunk) l.mode = kModeSmall;  // (line_shift is 0 here)
         // From 256 rows on, one 16-wave workgroup per row fills the chip as well as tiles over
         // workgroups do and needs no carry hand-off between workgroups.
         else if (nch >= 64 && rows < 256) l.mode = kModeLookback;

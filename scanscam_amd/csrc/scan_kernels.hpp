@@ -629,9 +629,11 @@ __global__ __launch_bounds__(MAXT) void scan_row_kernel(const ScanArgs p)
 
 // ---------------------------------------------------------------------------
 // SMALL kernel: rows no longer than one chunk. `group` lanes hold one row, a
-// wave holds U * 64 / group rows, and nothing is carried anywhere.
+// wave holds U * 64 / group rows, and nothing is carried anywhere. With RAGGED
+// the rows start at any element: a lane's vector is loaded element-aligned and
+// the last vector of a row is partial.
 // ---------------------------------------------------------------------------
-template <typename ST, int VEC, int U, bool REV, int MAXT>
+template <typename ST, int VEC, int U, bool REV, int MAXT, bool RAGGED = false>
 __global__ __launch_bounds__(MAXT) void scan_small_kernel(const ScanArgs p)
 {
     using CT = typename ComputeOf<ST>::type;
@@ -642,16 +644,14 @@ __global__ __launch_bounds__(MAXT) void scan_small_kernel(const ScanArgs p)
     const int64_t wave_id = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
     const int64_t row0 = wave_id * (U * rows_per_chunk) + lane / G;
 
-    WaveTile<ST, VEC, U, REV, true, false> w;
+    WaveTile<ST, VEC, U, REV, true, false, RAGGED> w;
     w.set_row(p, blockIdx.y, 0);
     CT hp[REV ? U : 1][VEC];
 #pragma unroll
     for (int u = 0; u < U; u++) {
         const int64_t row = row0 + (int64_t)u * rows_per_chunk;
-        const int m = REV ? G - 1 - j : j;
-        w.valid[u] = row < p.rows && m * VEC < p.T;
+        w.place(u, REV ? G - 1 - j : j, 0, row < p.rows, p.T);
         w.rowi[u] = w.valid[u] ? row : 0;
-        w.col[u] = w.valid[u] ? m * VEC : 0;
     }
     w.load(p, j, G - 1);
     w.reduce(j, G - 1, hp);

@@ -49,7 +49,7 @@ hipError_t launch_scan(const ScanArgs &args, const Launch &l, bool rev, hipStrea
         return hipGetLastError();                                                                    \
     }
 
-// The same for rows that are only element-aligned (ROW and LOOKBACK, full vector, U = 2 or 4).
+// The same for rows that are only element-aligned (full vector, U = 2 or 4).
 #define SCANSCAM_RAGGED_CASE(ST, VEC, U)                                                             \
     if (l.ragged && l.vec == (VEC) && l.unroll == (U)) {                                             \
         constexpr int MAXT = max_threads_for_unroll(U);                                              \
@@ -60,7 +60,8 @@ hipError_t launch_scan(const ScanArgs &args, const Launch &l, bool rev, hipStrea
             if (rev) hipExtLaunchKernelGGL((scan_lookback_kernel<ST, VEC, U, true, MAXT, true>), grid, block, 0, stream, start, stop, 0, args); \
             else     hipExtLaunchKernelGGL((scan_lookback_kernel<ST, VEC, U, false, MAXT, true>), grid, block, 0, stream, start, stop, 0, args);\
         } else {                                                                                     \
-            return hipErrorInvalidValue;                                                             \
+            if (rev) hipExtLaunchKernelGGL((scan_small_kernel<ST, VEC, U, true, MAXT, true>), grid, block, 0, stream, start, stop, 0, args);    \
+            else     hipExtLaunchKernelGGL((scan_small_kernel<ST, VEC, U, false, MAXT, true>), grid, block, 0, stream, start, stop, 0, args);   \
         }                                                                                            \
         return hipGetLastError();                                                                    \
     }

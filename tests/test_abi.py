@@ -83,10 +83,10 @@ def test_argument_errors_are_reported_before_any_launch():
                 hip.Plan(mode=hip.MODE_SMALL), hip.Plan(waves=17)):
         rc = L.scanscam_scan_fwd_plan(fake, fake, fake, 4, 4096, 0, None, 0, None, ctypes.byref(bad))
         assert rc == E_PLAN, bad
-    # Rows no longer than one chunk can use the 16-byte vector only if they start on 16-byte borders.
+    # Rows of fewer than four vectors can use the 16-byte vector only if they start on 16-byte borders.
     v4 = hip.Plan(vec=4)
     assert L.scanscam_scan_fwd_plan(fake, fake, fake, 4, 5, 0, None, 0, None, ctypes.byref(v4)) == E_PLAN
-    assert L.scanscam_scan_fwd_plan(fake + 4, fake, fake, 4, 64, 0, None, 0, None, ctypes.byref(v4)) == E_PLAN
+    assert L.scanscam_scan_fwd_plan(fake + 4, fake, fake, 4, 12, 0, None, 0, None, ctypes.byref(v4)) == E_PLAN
     # ... and element-aligned long rows only with 2 or 4 chunks per wave.
     v4u8 = hip.Plan(vec=4, unroll=8)
     assert L.scanscam_scan_fwd_plan(fake, fake, fake, 4, 1025, 0, None, 0, None, ctypes.byref(v4u8)) == E_PLAN
@@ -106,10 +106,10 @@ def test_strided_calls_check_their_arguments():
                                        None) == E_INVAL
     assert L.scanscam_scan_bwd_strided(fake, fake, fake, fake, None, None, None, None, None, None, 4, 64, 64, 0, None,
                                        0, None, None) == E_INVAL
-    # rows whose starts are not all 16-byte aligned cannot take a forced 16-byte vector when short
+    # rows whose starts are not all 16-byte aligned cannot take a forced 16-byte vector when shorter than 4 vectors
     v4 = hip.Plan(vec=4)
     odd = ctypes.byref(S(4096, 65))
-    assert L.scanscam_scan_fwd_strided(fake, fake, fake, odd, dense, dense, 4, 64, 64, 0, None, 0, None,
+    assert L.scanscam_scan_fwd_strided(fake, fake, fake, odd, dense, dense, 4, 64, 12, 0, None, 0, None,
                                        ctypes.byref(v4)) == E_PLAN
     # channels-last: the time stride is a 32-bit quantity
     big = ctypes.byref(S(0, 1 << 31))

@@ -281,6 +281,8 @@ def test_forced_plans_small(gpu, dtype):
         if vec == 1 and unroll not in (1, 4):
             continue
         lengths = [vec * k for k in (1, 2, 3, 4, 7, 8, 16, 31, 33, 64)] if vec > 1 else [1, 2, 3, 5, 8, 17, 32, 63, 64]
+        if vec > 1 and unroll in (2, 4):  # element-aligned rows of 4 vectors to one chunk: 16-byte lanes, last one partial
+            lengths += [4 * vec + 1, 7 * vec + vec - 1, 33 * vec + 1, 64 * vec - 1]
         for T in lengths:
             for rows in (1, 37, 515):
                 plan = hip.Plan(mode=hip.MODE_SMALL, vec=vec, unroll=unroll, waves=waves)
