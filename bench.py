@@ -28,6 +28,8 @@ Prints ONE JSON line. Besides the contract fields it carries
   host_library  the package's own loop for CPU tensors on the same tensors
                 (not the baseline: several rows side by side, several threads);
   long_rows     many rows of 16K to 96K elements (long-context shapes);
+  odd_lengths   row lengths that are no multiple of a 128-byte line or of the
+                16-byte vector;
   autograd_op   the same step through the op a model calls,
                 scanscam_amd.scan(a, b).backward(grad_h), outputs allocated per call;
   configs       forward and forward+backward GB/s of the other four synthetic
@@ -336,27 +338,43 @@ def long_rows(dev, args, hip, torch):
     mean microseconds per launch over back-to-back launches (each tensor is 268 MB / 134 MB, beyond the
     Infinity Cache).
     """
+    shapes = ((4096, 16384), (2048, 32768), (1365, 49152), (682, 98304))
+    return shape_table(dev, args, hip, torch, [(r, t, d) for d in (torch.float32, torch.bfloat16) for r, t in shapes])
+
+
+def odd_lengths(dev, args, hip, torch):
+    """Row lengths that are no multiple of a 128-byte line, or of the 16-byte vector; about 64 M elements each.
+
+    3000 and 9000: rows start inside a line (chunks are laid out from the line border before the row);
+    4097 and 70: rows start at any element (element-aligned vectors, partial first and last ones).
+    """
+    shapes = [(22369, 3000, torch.float32), (7456, 9000, torch.float32), (16380, 4097, torch.float32),
+              (958698, 70, torch.float32), (16380, 4097, torch.bfloat16)]
+    return shape_table(dev, args, hip, torch, shapes)
+
+
+def shape_table(dev, args, hip, torch, shapes):
+    """{shape: microseconds per launch, fraction of peak, plans} for (rows, T, dtype) triples, one buffer set each."""
     out = {}
-    for dtype in (torch.float32, torch.bfloat16):
-        for rows, T in ((4096, 16384), (2048, 32768), (1365, 49152), (682, 98304)):
-            g = torch.Generator(device=dev).manual_seed(0)
-            a = torch.rand((rows, T), generator=g, device=dev).to(dtype)
-            b = torch.randn((rows, T), generator=g, device=dev).to(dtype)
-            gh = torch.randn((rows, T), generator=g, device=dev).to(dtype)
-            s = object.__new__(DeviceSet)
-            s.a, s.b, s.gh = a, b, gh
-            s.h, s.ga, s.gb = (torch.empty_like(a) for _ in range(3))
-            f_ms, b_ms = time_batches([s], max(20, args.steps // 2), max(3, args.warmup // 2), hip, torch)
-            n, esize = a.numel(), a.element_size()
-            out[f"{rows}x{T}_{str(dtype).replace('torch.', '')}"] = {
-                "fwd_us": round(f_ms * 1e3, 1), "bwd_us": round(b_ms * 1e3, 1),
-                "fwd_frac": round(FWD_BYTES[esize] * n / (f_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-                "bwd_frac": round(BWD_BYTES[esize] * n / (b_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-                "plan_fwd": repr(hip.resolve_plan(rows, T, dtype, hip.FORWARD)),
-                "plan_bwd": repr(hip.resolve_plan(rows, T, dtype, hip.BACKWARD)),
-            }
-            del s, a, b, gh
-            torch.cuda.empty_cache()
+    for rows, T, dtype in shapes:
+        g = torch.Generator(device=dev).manual_seed(0)
+        a = torch.rand((rows, T), generator=g, device=dev).to(dtype)
+        b = torch.randn((rows, T), generator=g, device=dev).to(dtype)
+        gh = torch.randn((rows, T), generator=g, device=dev).to(dtype)
+        s = object.__new__(DeviceSet)
+        s.a, s.b, s.gh = a, b, gh
+        s.h, s.ga, s.gb = (torch.empty_like(a) for _ in range(3))
+        f_ms, b_ms = time_batches([s], max(20, args.steps // 2), max(3, args.warmup // 2), hip, torch)
+        n, esize = a.numel(), a.element_size()
+        out[f"{rows}x{T}_{str(dtype).replace('torch.', '')}"] = {
+            "fwd_us": round(f_ms * 1e3, 1), "bwd_us": round(b_ms * 1e3, 1),
+            "fwd_frac": round(FWD_BYTES[esize] * n / (f_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+            "bwd_frac": round(BWD_BYTES[esize] * n / (b_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+            "plan_fwd": repr(hip.resolve_plan(rows, T, dtype, hip.FORWARD)),
+            "plan_bwd": repr(hip.resolve_plan(rows, T, dtype, hip.BACKWARD)),
+        }
+        del s, a, b, gh
+        torch.cuda.empty_cache()
     return out
 
 
@@ -659,6 +677,7 @@ def main():
         out["reference_grid"] = reference_grid(dev, args, hip, torch)
         out["strided_views"] = strided_views(dev, args, hip, torch)
         out["long_rows"] = long_rows(dev, args, hip, torch)
+        out["odd_lengths"] = odd_lengths(dev, args, hip, torch)
 
     if not args.no_cpu:
         # 16-bit workloads: the reference has no 16-bit path, so its loop runs on the exact fp32 upcast.
