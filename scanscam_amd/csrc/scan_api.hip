@@ -568,6 +568,10 @@ int run_cl(bool rev, const void *a, const void *x, const void *h, void *y0, void
     args.C = (int32_t)C;
     args.segments = l.segments;
     args.group = l.group;
+    // Time steps that are not whole 128-byte lines: neighbouring channel groups on one XCD (see the kernel).
+    bool lines = true;
+    for (int k = 0; k < 5; k++) lines = lines && (sT[k] * esize) % 128 == 0 && aligned_to(ptrs[k], 128) && (sB[k] * esize) % 128 == 0;
+    args.xcd_order = (!lines && l.grid >= 64) ? 1 : 0;
     args.ws = nullptr;
     args.spin_limit = (plan && plan->spin_limit > 0) ? plan->spin_limit : scanscam::kSpinLimit;
 

@@ -43,6 +43,7 @@ struct ClArgs {
     int32_t C;
     int32_t segments;   // look-back kernel: tiles per (batch element, channel group)
     int32_t group;      // packed kernel: lanes per time step (power of two below 64)
+    int32_t xcd_order;  // scan_cl_kernel: consecutive (batch element, channel group) pairs share an XCD
     uint64_t *ws;       // look-back kernel: ticket counters + published pairs
     int32_t spin_limit; // look-back kernel: polls before a wait gives up
 };
@@ -223,7 +224,18 @@ __global__ __launch_bounds__(MAXT) void scan_cl_kernel(const ClArgs p)
     const int wave = threadIdx.x / kWave;
     const int W = blockDim.x / kWave;
     const int groups = (p.C + kWave * VEC - 1) / (kWave * VEC);  // channel groups per batch element
-    const ClLane<ST> ln = cl_lane<ST, VEC>(p, blockIdx.x / groups, blockIdx.x % groups, lane);
+    // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2. When a time step of C
+    // channels is not a whole number of 128-byte lines, neighbouring channel groups share a line at
+    // every time step; handled by different XCDs that line is fetched twice and written in two parts.
+    // xcd_order gives each XCD a contiguous run of (batch element, channel group) pairs instead, so that
+    // neighbours meet in one L2.
+    int bid = blockIdx.x;
+    if (p.xcd_order) {
+        const int n = gridDim.x, per = (n + 7) / 8, rem = n % 8 == 0 ? 8 : n % 8;
+        const int xcd = bid % 8, slot = bid / 8;
+        bid = xcd < rem ? xcd * per + slot : rem * per + (xcd - rem) * (per - 1) + slot;
+    }
+    const ClLane<ST> ln = cl_lane<ST, VEC>(p, bid / groups, bid % groups, lane);
 
     const int tile_steps = W * S;
     const int ntiles = (p.T + tile_steps - 1) / tile_steps;
