@@ -208,3 +208,55 @@ def test_few_channels_packed_kernel(gpu, dtype):
             assert rel_err(as_rows(got_h), h) <= bar, (plan, shape)
             assert rel_err(as_rows(got_gb), gb) <= bar, (plan, shape)
             assert rel_err(as_rows(got_ga), ga, prev_abs(as_rows(hs))) <= bar, (plan, shape)
+
+
+# (dtype, [batch, T, C], slice of C taken from a wider buffer or None). Automatic plans on grids of 64 and
+# more workgroups: time steps that are not whole 128-byte lines (every XCD then takes a contiguous run of
+# workgroups; numbers of workgroups that are and are not multiples of 8, dense tensors and views whose
+# rows are whole lines but start inside one), 320 workgroups of 16-byte lanes (4-wave workgroups), and
+# 16-bit single-channel lanes with 16 steps per wave.
+MANY_WORKGROUPS = [
+    (torch.float32, (37, 300, 1000), None),
+    (torch.float32, (67, 90, 1000), None),
+    (torch.bfloat16, (130, 60, 1096), None),
+    (torch.float32, (70, 129, 264), None),
+    (torch.float32, (65, 64, 1001), None),
+    (torch.float32, (67, 90, 520), None),
+    (torch.bfloat16, (33, 200, 1096), None),
+    (torch.float16, (64, 130, 1001), None),
+    (torch.float64, (40, 100, 500), None),
+    (torch.float32, (20, 150, 1000), (8, 1056)),
+    (torch.bfloat16, (24, 140, 1024), (16, 1088)),
+    (torch.float32, (80, 200, 1024), None),
+    (torch.bfloat16, (16, 1100, 1024), None),
+]
+
+
+@pytest.mark.parametrize("dtype,shape,window", MANY_WORKGROUPS)
+def test_automatic_plans_on_many_workgroups(gpu, dtype, shape, window):
+    bar = {torch.float32: 1e-5, torch.float64: 1e-13}.get(dtype, 1e-2)
+    B, T, C = shape
+    g = torch.Generator().manual_seed(T + C)
+
+    def place(t):
+        t = t.to(dtype).to(gpu)
+        if window is None:
+            return t
+        first, width = window
+        buf = torch.full((B, T, width), float("nan"), dtype=dtype, device=gpu)
+        buf[..., first:first + C] = t
+        return buf[..., first:first + C]
+
+    a = place(torch.rand(shape, generator=g, dtype=torch.float64))
+    b = place(torch.randn(shape, generator=g, dtype=torch.float64))
+    gh = place(torch.randn(shape, generator=g, dtype=torch.float64))
+    print(f"case cl many workgroups {dtype} shape={shape} window={window}", flush=True)
+    h = oracle.fwd(as_rows(a), as_rows(b))
+    got_h = hip.scan_forward(a.mT, b.mT)
+    assert got_h.shape == a.mT.shape and got_h.mT.is_contiguous()
+    assert rel_err(as_rows(got_h.mT), h) <= bar
+    hs = place(torch.from_numpy(h).mT)
+    ga, gb = oracle.bwd(as_rows(a), as_rows(hs), as_rows(gh))
+    got_ga, got_gb = hip.scan_backward(a.mT, hs.mT, gh.mT)
+    assert rel_err(as_rows(got_gb.mT), gb) <= bar
+    assert rel_err(as_rows(got_ga.mT), ga, prev_abs(as_rows(hs))) <= bar
