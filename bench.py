@@ -54,7 +54,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch at configs[1] from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by what the same
 # counters read for a copy kernel of known size (profiles/scan_row_f32_fwd_bwd_8x2048x4096_pmc_traffic.txt).
-MEASURED_TRAFFIC = {"fwd": 805.37e6, "bwd": 1347.53e6}
+MEASURED_TRAFFIC = {"fwd": 805.38e6, "bwd": 1347.36e6}
 METRIC = "scan HBM GB/s and % of MI355X peak, fwd and fwd+bwd, fp32 [B,C,T]"
 FWD_BYTES = {8: 24, 4: 12, 2: 6}
 BWD_BYTES = {8: 40, 4: 20, 2: 10}
