@@ -211,10 +211,11 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
         // Tiles of 32 chunks (8192 fp32 elements): fewer, larger tiles keep the wait for the
         // carry short relative to the time a tile spends on its data. With very few rows the
         // tiles in flight are neighbours in one row, which publish almost together and so wait
-        // longest for each other: 64 chunks there.
+        // longest for each other: 64 chunks there (up to 8 rows: forward +1 to +4 points of peak at
+        // 2^26 fp32 elements; from 12 rows on the 32-chunk tile is 4 to 6 points faster).
         l.unroll = u.unroll ? u.unroll : 4;
-        l.waves = u.waves ? u.waves : (rows <= 16 && l.unroll <= 4 ? 16 : 8);
-        if (!u.waves && !u.unroll && rows > 16) {
+        l.waves = u.waves ? u.waves : (rows <= 8 && l.unroll <= 4 ? 16 : 8);
+        if (!u.waves && !u.unroll && rows > 8) {
             // As many tiles as 8-wave tiles would take, but with only the waves they need: 75 chunks are 3
             // tiles of 7 waves (84 chunk slots), not of 8 (96).
             const int tiles = (nch + kTileChunks - 1) / kTileChunks;
