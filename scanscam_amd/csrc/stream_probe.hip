@@ -19,8 +19,14 @@
 //                             k / R of row k % R, so that tiles of all rows are in flight together. R = 1 is the
 //                             plain linear order. What the memory system gives that order with no scan, no tickets
 //                             and no carry chain.
+//   stream_probe cl              the channels-last kernels' access shape with no scan: tensors [B, T, C] fp32, a
+//                             workgroup owns 64 * VEC channels of one batch element and walks all of T in tiles of
+//                             W waves x S time steps; per step a wave reads one span of 64 * VEC channels. With and
+//                             without the kernels' one barrier per tile; and the same spans with one tile per
+//                             workgroup (the shape of the kernel that also splits time over workgroups).
 //
-//   hipcc -O3 --offload-arch=gfx950 stream_probe.hip -o stream_probe
+//   hipcc -O3 --offload-arch=gfx950 -Xclang -target-feature -Xclang -packed-fp32-ops stream_probe.hip -o stream_probe
+//   (or `make -C scanscam_amd/csrc`, which builds build/stream_probe)
 #include <hip/hip_runtime.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -363,13 +369,177 @@ static int run_order()
     return hipDeviceSynchronize() == hipSuccess ? 0 : 1;
 }
 
+// Channels-last access shape (scan_cl_kernel): see `stream_probe cl` above. T is a multiple of W * S.
+template <int VEC> struct ClVec { typedef f4 type; };
+template <> struct ClVec<1> { typedef float type; };
+
+template <int READS, int WRITES, int VEC, int S, bool SYNC>
+__global__ void cl_stream_kernel(const float *__restrict__ a, const float *__restrict__ b, const float *__restrict__ c,
+                                 float *__restrict__ o0, float *__restrict__ o1, int T, int C)
+{
+    typedef typename ClVec<VEC>::type V;
+    const int W = blockDim.x / 64, wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    const int groups = C / (64 * VEC);
+    const size_t col = (size_t)(blockIdx.x / groups) * T * C + (size_t)(blockIdx.x % groups) * 64 * VEC + lane * VEC;
+    for (int t0 = wave * S; t0 < T; t0 += W * S) {
+        V va[S], vb[S], vc[S];
+#pragma unroll
+        for (int k = 0; k < S; k++) {
+            const size_t at = col + (size_t)(t0 + k) * C;
+            va[k] = __builtin_nontemporal_load(reinterpret_cast<const V *>(a + at));
+            vb[k] = __builtin_nontemporal_load(reinterpret_cast<const V *>(b + at));
+            if (READS > 2) vc[k] = __builtin_nontemporal_load(reinterpret_cast<const V *>(c + at));
+        }
+        if (SYNC) __syncthreads();
+#pragma unroll
+        for (int k = 0; k < S; k++) {
+            const size_t at = col + (size_t)(t0 + k) * C;
+            V r = va[k] + vb[k];
+            if (READS > 2) r *= vc[k];
+            __builtin_nontemporal_store(r, reinterpret_cast<V *>(o0 + at));
+            if (WRITES > 1) __builtin_nontemporal_store(r + 1.0f, reinterpret_cast<V *>(o1 + at));
+        }
+    }
+}
+
+static float *g_cl[2][5];
+static const size_t kClElements = (size_t)1 << 28;  // per stream: the largest case below
+
+template <int READS, int WRITES, int VEC, int S, bool SYNC> static void cl_case(int B, int T, int C, int W)
+{
+    const size_t n = (size_t)B * T * C;
+    if (n > kClElements || T % (W * S) != 0 || C % (64 * VEC) != 0 || W < 1 || W > 16) {
+        fprintf(stderr, "cl_case: [%d, %d, %d] with %d waves x %d steps does not fit the buffers or the kernel\n", B, T, C, W, S);
+        exit(1);
+    }
+    int i = 0;
+    const float ms = mean_ms(
+        [&] {
+            float **s = g_cl[i++ % 2];
+            hipLaunchKernelGGL((cl_stream_kernel<READS, WRITES, VEC, S, SYNC>), dim3((unsigned)(B * (C / (64 * VEC)))),
+                               dim3(W * 64), 0, 0, s[0], s[1], s[2], s[3], s[4], T, C);
+        },
+        30);
+    const double bytes = (double)(READS + WRITES) * n * 4;
+    printf("  %dR%dW  [%4d, %5d, %5d]  %2d-byte lanes  %2d waves x %2d steps  %-10s %5d workgroups  %7.1f us  %4.1f %% of 8 TB/s\n",
+           READS, WRITES, B, T, C, VEC * 4, W, S, SYNC ? "barrier" : "no barrier", B * (C / (64 * VEC)), ms * 1e3,
+           bytes / (ms * 1e-3) / 8e12 * 100);
+}
+
+// The same spans taken one tile of W x S steps per workgroup (scan_cl_lookback_kernel's shape, with no tickets and
+// no carry chain): workgroup k takes tile k / RG of row-group k % RG (ROW_MAJOR = false: tiles of all row-groups in
+// flight together) or tile k % tiles of row-group k / tiles (ROW_MAJOR = true).
+template <int READS, int WRITES, int VEC, int S, bool ROW_MAJOR>
+__global__ void cl_tile_kernel(const float *__restrict__ a, const float *__restrict__ b, const float *__restrict__ c,
+                               float *__restrict__ o0, float *__restrict__ o1, int T, int C, int rowgroups, int tiles)
+{
+    typedef typename ClVec<VEC>::type V;
+    const int W = blockDim.x / 64, wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    const int groups = C / (64 * VEC);
+    const int rg = ROW_MAJOR ? blockIdx.x / tiles : blockIdx.x % rowgroups;
+    const int tile = ROW_MAJOR ? blockIdx.x % tiles : blockIdx.x / rowgroups;
+    const size_t col = (size_t)(rg / groups) * T * C + (size_t)(rg % groups) * 64 * VEC + lane * VEC;
+    const int t0 = (tile * W + wave) * S;
+    V va[S], vb[S], vc[S];
+#pragma unroll
+    for (int k = 0; k < S; k++) {
+        const size_t at = col + (size_t)(t0 + k) * C;
+        va[k] = __builtin_nontemporal_load(reinterpret_cast<const V *>(a + at));
+        vb[k] = __builtin_nontemporal_load(reinterpret_cast<const V *>(b + at));
+        if (READS > 2) vc[k] = __builtin_nontemporal_load(reinterpret_cast<const V *>(c + at));
+    }
+#pragma unroll
+    for (int k = 0; k < S; k++) {
+        const size_t at = col + (size_t)(t0 + k) * C;
+        V r = va[k] + vb[k];
+        if (READS > 2) r *= vc[k];
+        __builtin_nontemporal_store(r, reinterpret_cast<V *>(o0 + at));
+        if (WRITES > 1) __builtin_nontemporal_store(r + 1.0f, reinterpret_cast<V *>(o1 + at));
+    }
+}
+
+template <int READS, int WRITES, int VEC, int S, bool ROW_MAJOR> static void cl_tile_case(int B, int T, int C, int W)
+{
+    const size_t n = (size_t)B * T * C;
+    if (n > kClElements || T % (W * S) != 0 || C % (64 * VEC) != 0 || W < 1 || W > 16) {
+        fprintf(stderr, "cl_tile_case: [%d, %d, %d] with %d waves x %d steps does not fit the buffers or the kernel\n", B, T, C, W, S);
+        exit(1);
+    }
+    const int rowgroups = B * (C / (64 * VEC)), tiles = T / (W * S);
+    int i = 0;
+    const float ms = mean_ms(
+        [&] {
+            float **s = g_cl[i++ % 2];
+            hipLaunchKernelGGL((cl_tile_kernel<READS, WRITES, VEC, S, ROW_MAJOR>), dim3((unsigned)(rowgroups * tiles)),
+                               dim3(W * 64), 0, 0, s[0], s[1], s[2], s[3], s[4], T, C, rowgroups, tiles);
+        },
+        30);
+    const double bytes = (double)(READS + WRITES) * n * 4;
+    printf("  %dR%dW  [%4d, %5d, %5d]  %2d-byte lanes  one tile of %2d waves x %2d steps per workgroup, %-10s %6d workgroups  %7.1f us  %4.1f %% of 8 TB/s\n",
+           READS, WRITES, B, T, C, VEC * 4, W, S, ROW_MAJOR ? "row-major" : "tile-major", rowgroups * tiles, ms * 1e3,
+           bytes / (ms * 1e-3) / 8e12 * 100);
+}
+
+template <int READS, int WRITES> static void cl_tile_cases()
+{
+    cl_tile_case<READS, WRITES, 4, 4, false>(64, 2048, 1024, 4);
+    cl_tile_case<READS, WRITES, 4, 4, true>(64, 2048, 1024, 4);
+    cl_tile_case<READS, WRITES, 4, 4, false>(64, 2048, 1024, 8);
+    cl_tile_case<READS, WRITES, 4, 8, false>(64, 2048, 1024, 8);
+    cl_tile_case<READS, WRITES, 4, 8, false>(8, 4096, 2048, 8);
+    cl_tile_case<READS, WRITES, 4, 8, true>(8, 4096, 2048, 8);
+    cl_tile_case<READS, WRITES, 4, 8, false>(8, 4096, 2048, 4);
+    cl_tile_case<READS, WRITES, 4, 4, false>(8, 4096, 2048, 4);
+    cl_tile_case<READS, WRITES, 1, 16, false>(8, 4096, 2048, 8);
+    cl_tile_case<READS, WRITES, 1, 8, false>(8, 4096, 2048, 4);
+    cl_tile_case<READS, WRITES, 1, 16, false>(8, 4096, 512, 8);
+    cl_tile_case<READS, WRITES, 4, 8, false>(8, 4096, 512, 8);
+}
+
+template <int READS, int WRITES> static void cl_cases()
+{
+    cl_case<READS, WRITES, 4, 4, true>(64, 2048, 1024, 16);
+    cl_case<READS, WRITES, 4, 4, false>(64, 2048, 1024, 16);
+    cl_case<READS, WRITES, 4, 8, true>(64, 2048, 1024, 8);
+    cl_case<READS, WRITES, 4, 4, true>(64, 2048, 1024, 4);
+    cl_case<READS, WRITES, 4, 4, true>(256, 1024, 1024, 16);
+    cl_case<READS, WRITES, 4, 4, false>(256, 1024, 1024, 16);
+    cl_case<READS, WRITES, 4, 4, true>(256, 1024, 1024, 4);
+    cl_case<READS, WRITES, 4, 4, true>(512, 1024, 256, 16);
+    cl_case<READS, WRITES, 4, 4, false>(512, 1024, 256, 16);
+    cl_case<READS, WRITES, 1, 8, true>(8, 4096, 2048, 16);
+    cl_case<READS, WRITES, 1, 8, false>(8, 4096, 2048, 16);
+    cl_case<READS, WRITES, 1, 16, true>(8, 4096, 2048, 8);
+    cl_case<READS, WRITES, 1, 16, true>(8, 4096, 2048, 16);
+    cl_case<READS, WRITES, 1, 8, true>(64, 2048, 512, 16);
+    cl_case<READS, WRITES, 1, 8, true>(32, 2048, 1024, 16);
+}
+
+static int run_cl()
+{
+    const size_t bytes = kClElements * sizeof(float);
+    for (auto &set : g_cl)
+        for (auto &p : set) {
+            CHECK(hipMalloc(&p, bytes));
+            CHECK(hipMemset(p, 0, bytes));
+        }
+    printf("channels-last access shape, fp32, 2 rotated buffer sets of 1 GiB per stream:\n");
+    cl_cases<2, 1>();
+    cl_cases<3, 2>();
+    printf("one tile per workgroup:\n");
+    cl_tile_cases<2, 1>();
+    cl_tile_cases<3, 2>();
+    return hipDeviceSynchronize() == hipSuccess ? 0 : 1;
+}
+
 int main(int argc, char **argv)
 {
+    if (argc > 1 && strcmp(argv[1], "cl") == 0) return run_cl();
     if (argc > 1 && strcmp(argv[1], "order") == 0) return run_order();
     if (argc > 1 && strcmp(argv[1], "mix") == 0) return run_mix();
     if (argc > 1 && strcmp(argv[1], "ceiling") == 0) return run_ceiling(argc > 2 ? (size_t)atol(argv[2]) : 16384);
     if (argc > 1 && strcmp(argv[1], "copy") == 0) return run_copy(argc > 2 ? (size_t)atol(argv[2]) : 1024);
     if (argc > 1 && strcmp(argv[1], "policy") == 0) return run_policy(argc > 2 ? (size_t)atol(argv[2]) : 16384);
-    fprintf(stderr, "usage: %s copy [MiB] | ceiling [rows] | policy [rows] | mix | order\n", argv[0]);
+    fprintf(stderr, "usage: %s copy [MiB] | ceiling [rows] | policy [rows] | mix | order | cl\n", argv[0]);
     return 2;
 }
