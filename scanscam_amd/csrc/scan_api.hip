@@ -142,7 +142,13 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
     const int64_t lead = l.ragged ? 128 / esize - 1 : 128 / ((int64_t)l.vec * esize) - 1;
     const int64_t nvec = l.ragged ? (T + lead + l.vec - 1) / l.vec : (T + l.vec - 1) / l.vec + lead;
     const int64_t nch_plain = (T + chunk - 1) / chunk, nch_lines = (nvec + kWave - 1) / kWave;
-    out->line_shift = (!aligned128 && !small_rows && (T > chunk || l.ragged) && (nch_plain > 4 || nch_lines <= 4)) ? 1 : 0;
+    // Rows of up to 4 chunks take one wave with 1, 2 or 4 chunks (2 or 4 when element-aligned): no shift
+    // either where it would double that count and leave half the wave's slots empty (bf16 [33520, 1001], two
+    // chunks: 38 / 57 us without the shift, 51 / 87 us with it in a wave of 4).
+    auto chunks_of_one_wave = [&](int64_t n) { return pow2_ceil(l.ragged && n < 2 ? 2 : n); };
+    const bool same_wave_shape =
+        nch_plain > 4 || (nch_lines <= 4 && chunks_of_one_wave(nch_lines) == chunks_of_one_wave(nch_plain));
+    out->line_shift = (!aligned128 && !small_rows && (T > chunk || l.ragged) && same_wave_shape) ? 1 : 0;
     const int64_t nch64 = out->line_shift ? nch_lines : nch_plain;
     const int nch = (int)nch64;
     out->nch = nch;
@@ -186,8 +192,11 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
                 l.unroll = (l.vec == full && nch <= 6) ? 2 : 4;
                 l.wpr = (l.vec == full && (nch == 7 || nch == 8)) ? 2 : 4;
                 l.waves = 4;
-                // Element-aligned rows of 9-12 chunks: 3 waves (bf16 [16380, 4097]: 76 / 123 us, 96 / 149 with 4).
+                // Element-aligned rows of 9-12 chunks: 3 waves (bf16 [16380, 4097]: 76 / 123 us, 96 / 149 with 4);
+                // of 5-6 chunks: 3 waves x 2 chunks (bf16 [16376, 2049]: 45 / 66 us, 55 / 82 with 4 waves;
+                // fp32 [32736, 1025]: 69 / 110 against 76 / 110).
                 if (l.ragged && nch > 8 && nch <= 12) l.wpr = l.waves = 3;
+                if (l.ragged && nch >= 5 && nch <= 6) l.wpr = l.waves = 3;
             } else {
                 // Longer rows: a workgroup tile (waves x 4 chunks) that covers the row in one step, or
                 // in as few as 16 waves allow -- each further step waits for the carry of the last --

@@ -139,15 +139,46 @@ template <typename ST, int VEC> struct Vec {
     {
         __builtin_nontemporal_store(r, reinterpret_cast<raw_unaligned_t *>(p));
     }
-    // The components whose bit is set in `inside` only, the rest zero: the partial vector at the start
-    // or the end of a row (the others lie outside the row and are neither read nor written).
-    static __device__ __forceinline__ raw_t load_part(const ST *p, uint32_t inside)
+    // The partial vector at the start or the end of a row (bit k of `inside` set = component k lies
+    // inside the row; the others are neither read nor written) is loaded with one element-aligned
+    // 16-byte load like every other vector's: the window of VEC elements that ends with the row
+    // (partial vector at its end) or starts with it (at its start), whose components are then moved
+    // into place inside the registers (shift_components; those outside the row become zero). No
+    // branch and no instruction per element, so all loads of a wave are still issued before the first
+    // is waited for. Needs rows of at least VEC elements. window_shift: how many components the window
+    // starts after (> 0) or before (< 0) the vector; 0 for a whole vector and for a lane without one.
+    static __device__ __forceinline__ int window_shift(uint32_t inside)
     {
-        Elems<ST, VEC> e;
-#pragma unroll
-        for (int k = 0; k < VEC; k++) e.e[k] = ((inside >> k) & 1u) ? p[k] : (ST)0.0f;
-        return __builtin_bit_cast(raw_t, e);
+        const int lo = inside ? __builtin_ctz(inside) : 0, hi = inside ? 32 - __builtin_clz(inside) : VEC;
+        return hi < VEC ? hi - VEC : lo;  // < 0: the window starts before component 0; > 0: after it
     }
+    // Components moved up by s places (s > 0) or down by -s (s < 0) inside a 16-byte vector.
+    static __device__ __forceinline__ raw_t shift_components(raw_t r, int s)
+    {
+        if constexpr (sizeof(raw_t) != 16) {
+            return r;
+        } else {
+            const uint64_t lo = (uint64_t)r.x | ((uint64_t)r.y << 32), hi = (uint64_t)r.z | ((uint64_t)r.w << 32);
+            const int bits = (s < 0 ? -s : s) * (int)sizeof(ST) * 8;  // 0 ... 112
+            const int b = bits & 63;
+            const bool far = bits >= 64;
+            uint64_t out_lo, out_hi;
+            if (s < 0) {
+                out_lo = far ? (hi >> b) : ((lo >> b) | ((hi << 1) << (63 - b)));
+                out_hi = far ? 0 : (hi >> b);
+            } else {
+                out_hi = far ? (lo << b) : ((hi << b) | ((lo >> 1) >> (63 - b)));
+                out_lo = far ? 0 : (lo << b);
+            }
+            raw_t out;
+            out.x = (uint32_t)out_lo;
+            out.y = (uint32_t)(out_lo >> 32);
+            out.z = (uint32_t)out_hi;
+            out.w = (uint32_t)(out_hi >> 32);
+            return out;
+        }
+    }
+    // The components whose bit is set in `inside` only: one store per component under a lane mask.
     static __device__ __forceinline__ void store_part(ST *p, raw_t r, uint32_t inside)
     {
         const Elems<ST, VEC> e = __builtin_bit_cast(Elems<ST, VEC>, r);
@@ -323,11 +354,6 @@ struct WaveTile {
         return o;
     }
 
-    __device__ __forceinline__ raw_t fetch(const ST *p, int u) const
-    {
-        if (!RAGGED) return V::load(p);
-        return inside[u] == kAll ? V::load_unaligned(p) : V::load_part(p, inside[u]);
-    }
     __device__ __forceinline__ void put(ST *p, raw_t r, int u) const
     {
         if (!RAGGED) {
@@ -367,14 +393,13 @@ struct WaveTile {
                 rx[u] = V::load(x + at<1>(p, u));
                 if (REV) rh[u] = V::load(h + at<2>(p, u));
             } else {
-                ra[u] = V::zero_raw();
-                rx[u] = V::zero_raw();
-                if (REV) rh[u] = V::zero_raw();
-                if (valid[u]) {
-                    ra[u] = fetch(a + at<0>(p, u), u);
-                    rx[u] = fetch(x + at<1>(p, u), u);
-                    if (REV) rh[u] = fetch(h + at<2>(p, u), u);
-                }
+                // Just as unconditional: a partial vector is loaded as the window of VEC elements that
+                // starts or ends with the row (settle() moves its components into place once all loads
+                // are under way), lanes outside the row read the row's first vector.
+                const int s = V::window_shift(inside[u]);
+                ra[u] = V::load_unaligned(a + at<0>(p, u) + s);
+                rx[u] = V::load_unaligned(x + at<1>(p, u) + s);
+                if (REV) rh[u] = V::load_unaligned(h + at<2>(p, u) + s);
             }
             if (REV) {
                 edge_a[u] = CT(0);
@@ -386,6 +411,23 @@ struct WaveTile {
                 const bool need_h = !CHAIN || u == U - 1;
                 if (need_a && valid[u] && j == 0 && col[u] + VEC < p.T) edge_a[u] = (CT)a[at<0>(p, u) + VEC];
                 if (need_h && valid[u] && j == jlast && col[u] > 0) edge_h[u] = (CT)h[at<2>(p, u) - 1];
+            }
+        }
+    }
+
+    // RAGGED: the partial vectors, loaded as windows, get their components moved into place (those
+    // outside the row become zero). Only VALU work: no wait separates the loads issued by load().
+    __device__ __forceinline__ void settle()
+    {
+        if (RAGGED) {
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int s = V::window_shift(inside[u]);
+                if (s != 0) {
+                    ra[u] = V::shift_components(ra[u], s);
+                    rx[u] = V::shift_components(rx[u], s);
+                    if (REV) rh[u] = V::shift_components(rh[u], s);
+                }
             }
         }
     }
@@ -458,6 +500,7 @@ struct WaveTile {
     __device__ __forceinline__ void reduce(int j, int jlast, CT (&hp)[REV ? U : 1][VEC])
     {
         CT first_a[REV ? U : 1], last_h[REV ? U : 1];
+        settle();
         borders(first_a, last_h);
 #pragma unroll
         for (int u = 0; u < U; u++) {

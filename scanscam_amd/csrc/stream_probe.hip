@@ -24,6 +24,8 @@
 //                             W waves x S time steps; per step a wave reads one span of 64 * VEC channels. With and
 //                             without the kernels' one barrier per tile; and the same spans with one tile per
 //                             workgroup (the shape of the kernel that also splits time over workgroups).
+//   stream_probe misaligned      a copy with 16-byte accesses that start 2, 4, 6 or 8 bytes after a 16-byte border, in
+//                             every lane or in one lane per wave: what element-aligned vectors cost.
 //
 //   hipcc -O3 --offload-arch=gfx950 -Xclang -target-feature -Xclang -packed-fp32-ops stream_probe.hip -o stream_probe
 //   (or `make -C scanscam_amd/csrc`, which builds build/stream_probe)
@@ -532,14 +534,62 @@ static int run_cl()
     return hipDeviceSynchronize() == hipSuccess ? 0 : 1;
 }
 
+// 16-byte accesses that start OFFSET bytes after a 16-byte border (element-aligned vectors of rows that start
+// anywhere), in every lane (EVERY = true) or in lane 0 of each wave only. Copy of 2^26 floats.
+typedef f4 f4_unaligned __attribute__((aligned(2)));
+
+template <bool LOADS, bool STORES, bool EVERY>
+__global__ __launch_bounds__(256) void misaligned_kernel(const char *__restrict__ in, char *__restrict__ out, int offset)
+{
+    const size_t i = ((size_t)blockIdx.x * 1024 + (threadIdx.x / 64) * 256 + (threadIdx.x % 64)) * 16;
+    const bool mine = EVERY || (threadIdx.x % 64) == 0;
+    f4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+        v[u] = __builtin_nontemporal_load(reinterpret_cast<const f4_unaligned *>(in + i + u * 1024 + ((LOADS && mine) ? offset : 0)));
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+        __builtin_nontemporal_store(v[u], reinterpret_cast<f4_unaligned *>(out + i + u * 1024 + ((STORES && mine) ? offset : 0)));
+}
+
+template <bool LOADS, bool STORES, bool EVERY> static void misaligned_case(char *in, char *out, size_t bytes, int offset)
+{
+    const float ms = mean_ms(
+        [&] {
+            hipLaunchKernelGGL((misaligned_kernel<LOADS, STORES, EVERY>), dim3((unsigned)(bytes / 16384)), dim3(256), 0, 0, in, out, offset);
+        },
+        20);
+    printf("  offset %2d bytes in %-22s of %-6s  %7.1f us  %4.1f %% of 8 TB/s\n", offset, EVERY ? "every lane" : "lane 0 of each wave",
+           LOADS && STORES ? "both" : (LOADS ? "loads" : "stores"), ms * 1e3, 2.0 * bytes / (ms * 1e-3) / 8e12 * 100);
+}
+
+static int run_misaligned()
+{
+    const size_t bytes = (size_t)1 << 28;  // the kernels touch up to 16 bytes beyond: allocate one block more
+    char *in, *out;
+    CHECK(hipMalloc(&in, bytes + 16384));
+    CHECK(hipMalloc(&out, bytes + 16384));
+    CHECK(hipMemset(in, 0, bytes + 16384));
+    CHECK(hipMemset(out, 0, bytes + 16384));
+    printf("copy of 256 MiB with 16-byte accesses that start off a 16-byte border:\n");
+    for (int offset : {0, 2, 4, 8, 6}) {
+        misaligned_case<true, false, true>(in, out, bytes, offset);
+        misaligned_case<false, true, true>(in, out, bytes, offset);
+        misaligned_case<true, false, false>(in, out, bytes, offset);
+        misaligned_case<false, true, false>(in, out, bytes, offset);
+    }
+    return hipDeviceSynchronize() == hipSuccess ? 0 : 1;
+}
+
 int main(int argc, char **argv)
 {
+    if (argc > 1 && strcmp(argv[1], "misaligned") == 0) return run_misaligned();
     if (argc > 1 && strcmp(argv[1], "cl") == 0) return run_cl();
     if (argc > 1 && strcmp(argv[1], "order") == 0) return run_order();
     if (argc > 1 && strcmp(argv[1], "mix") == 0) return run_mix();
     if (argc > 1 && strcmp(argv[1], "ceiling") == 0) return run_ceiling(argc > 2 ? (size_t)atol(argv[2]) : 16384);
     if (argc > 1 && strcmp(argv[1], "copy") == 0) return run_copy(argc > 2 ? (size_t)atol(argv[2]) : 1024);
     if (argc > 1 && strcmp(argv[1], "policy") == 0) return run_policy(argc > 2 ? (size_t)atol(argv[2]) : 16384);
-    fprintf(stderr, "usage: %s copy [MiB] | ceiling [rows] | policy [rows] | mix | order | cl\n", argv[0]);
+    fprintf(stderr, "usage: %s copy [MiB] | ceiling [rows] | policy [rows] | mix | order | cl | misaligned\n", argv[0]);
     return 2;
 }
