@@ -346,10 +346,12 @@ def odd_lengths(dev, args, hip, torch):
     """Row lengths that are no multiple of a 128-byte line, or of the 16-byte vector; about 64 M elements each.
 
     3000 and 9000: rows start inside a line (chunks are laid out from the line border before the row);
-    4097 and 70: rows start at any element (element-aligned vectors, partial first and last ones).
+    4097 and 70, and the 16-bit lengths that are no multiple of 8: rows start at any element
+    (element-aligned vectors, partial first and last ones).
     """
     shapes = [(22369, 3000, torch.float32), (7456, 9000, torch.float32), (16380, 4097, torch.float32),
-              (958698, 70, torch.float32), (16380, 4097, torch.bfloat16)]
+              (958698, 70, torch.float32), (16380, 4097, torch.bfloat16), (67040, 1001, torch.bfloat16),
+              (134216, 500, torch.bfloat16), (32752, 2049, torch.bfloat16), (2013, 33333, torch.bfloat16)]
     return shape_table(dev, args, hip, torch, shapes)
 
 
