@@ -112,3 +112,43 @@ def test_random_cases(gpu, block):
         wga, wgb = oracle.bwd(ha, hh, hgh)
         assert rel_err(host(db.grad), wgb) <= bar, "grad of value"
         assert rel_err(host(da.grad), wga, hh) <= bar, "grad of gate"
+
+
+@pytest.mark.parametrize("block", range(4))
+def test_random_element_aligned_rows(gpu, block):
+    """
+    Rows that start at any element: lengths that are no multiple of the vector, bases offset by a few
+    elements, row strides padded by a few elements; the buffers around and between the rows hold NaN, so a
+    partial vector loaded from outside its row, or stored over it, shows.
+    """
+    rng = np.random.default_rng(3000 + block)
+    for i in range(40):
+        dtype = [torch.float32, torch.bfloat16, torch.float16, torch.float64][rng.integers(4)]
+        full = 16 // torch.empty(0, dtype=dtype).element_size()
+        kind = rng.integers(4)  # a group of lanes per row, a few chunks, many chunks, shorter than 4 vectors
+        lo, hi = [(4 * full, 64 * full + 1), (64 * full, 1280 * full), (1280 * full, 12800 * full), (1, 4 * full)][kind]
+        T = int(rng.integers(lo, hi))
+        rows = int(rng.integers(1, max(2, min(2000, (1 << 20) // T))))
+        offset = int(rng.integers(0, 2 * full))
+        stride = T + int(rng.integers(0, 3)) * int(rng.integers(0, 2 * full))
+        print(f"case ragged block={block} i={i} dtype={dtype} rows={rows} T={T} offset={offset} stride={stride}", flush=True)
+
+        def view_of(values):
+            buf = torch.full((rows * stride + offset + 64,), float("nan"), dtype=dtype, device=gpu)
+            v = buf[offset:offset + rows * stride].view(rows, stride)[:, :T]
+            v.copy_(torch.from_numpy(values).to(dtype))
+            return buf, v
+
+        _, a = view_of(rng.random((rows, T)))
+        _, b = view_of(rng.standard_normal((rows, T)))
+        _, gh = view_of(rng.standard_normal((rows, T)))
+        da, db = a.detach().requires_grad_(), b.detach().requires_grad_()
+        h = scanscam_amd.scan(da, db)
+        h.backward(gh)
+        bar = BARS[dtype]
+        ha, hb, hgh, hh = (np.ascontiguousarray(host(t)) for t in (a, b, gh, h))
+        assert not np.isnan(hh).any()
+        assert rel_err(hh, oracle.fwd(ha, hb)) <= bar, "forward"
+        wga, wgb = oracle.bwd(ha, hh, hgh)
+        assert rel_err(host(db.grad), wgb) <= bar, "grad of value"
+        assert rel_err(host(da.grad), wga, hh) <= bar, "grad of gate"
