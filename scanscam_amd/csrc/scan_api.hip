@@ -207,6 +207,15 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
                 l.unroll = 4;
                 const int steps = (nch + 63) / 64;
                 l.wpr = l.waves = (nch + steps * 4 - 1) / (steps * 4);
+                // 16-bit storage, 17-24 chunks (to 28 when element-aligned): two steps of half as many waves with
+                // 2 chunks each. These kernels are as much bound by their instructions as by memory (unpacking,
+                // 8 elements per lane and chunk), and with 2 chunks per wave they need half the registers, so
+                // twice the waves cover each other: bf16 [3883, 8640] 41.5 / 63.6 us -> 35.1 / 59.4 us, element-
+                // aligned [3297, 10175] 46.1 / 69.3 -> 35.9 / 60.8 us. From 32 chunks on the single step wins back.
+                if (esize == 2 && nch <= (l.ragged ? 28 : 24)) {
+                    l.unroll = 2;
+                    l.wpr = l.waves = (nch + 3) / 4;
+                }
             }
         } else {
             if (!l.unroll) l.unroll = 4;
