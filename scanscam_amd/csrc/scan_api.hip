@@ -93,10 +93,14 @@ bool row_major_order(int64_t rows, int tiles_per_row) { return rows >= 256 && ti
 // rounds do not come out.
 constexpr int kComputeUnits = 256;  // MI355X
 
-bool prefer_lookback_for_many_rows(int64_t rows, int nch, bool rev)
+bool prefer_lookback_for_many_rows(int64_t rows, int nch, bool rev, int esize)
 {
     const int tpr = (nch + kTileChunks - 1) / kTileChunks;
     if (rows < 256 || tpr < 2 || rows * tpr < 2048) return false;
+    // Two tiles of up to 24 chunks, 4- and 8-byte elements, forward: one workgroup of up to 12 waves per row is
+    // faster (fp32, 34-48 chunks: 72 against 63 % of peak at 16 M elements, 78-80 against 76 % at 64 M; from 52
+    // chunks on, and backward, the look-back kernel; 16-bit storage: the look-back kernel, 70 against 60-64 %).
+    if (!rev && esize >= 4 && tpr == 2 && nch <= 48) return false;
     const int64_t rounds = (rows + kComputeUnits - 1) / kComputeUnits;
     const bool ragged_rounds = rows * 100 < rounds * kComputeUnits * 93;  // the row kernel's CUs idle > 7 % of the time
     if (rev && tpr <= 16) return true;
@@ -165,7 +169,7 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
         // From 256 rows on, one 16-wave workgroup per row fills the chip as well as tiles over
         // workgroups do and needs no carry hand-off between workgroups.
         else if (nch >= 64 && rows < 256) l.mode = kModeLookback;
-        else if (prefer_lookback_for_many_rows(rows, nch, rev)) l.mode = kModeLookback;
+        else if (prefer_lookback_for_many_rows(rows, nch, rev, esize)) l.mode = kModeLookback;
         else l.mode = kModeRow;
     }
 

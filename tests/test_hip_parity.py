@@ -356,7 +356,7 @@ ROW, LOOKBACK = hip.MODE_ROW, hip.MODE_LOOKBACK
 AUTO_REGIMES = [
     (2048, 1280, (ROW, 4, 2), None),
     (2048, 4100, (ROW, 5, 4), None),          # 17 chunks: one step of a 5-wave workgroup
-    (2048, 10000, (LOOKBACK, 0, 4), None),    # 40 chunks = 2 tiles of 5 waves
+    (2048, 10000, (ROW, 10, 4), (LOOKBACK, 0, 4)),  # 40 chunks: forward one workgroup of 10 waves, backward 2 tiles of 5 waves
     (2048, 12501, (LOOKBACK, 0, 4), None),    # element-aligned rows, 50 chunks = 2 tiles of 7 waves, row-major order
     (700, 20000, (LOOKBACK, 0, 4), None),     # 3 tiles per row, 2100 tiles
     (256, 131072, (ROW, 16, 4), (LOOKBACK, 0, 4)),  # 16 tiles per row: only the backward pass gains
@@ -374,11 +374,12 @@ AUTO_REGIMES = [
 @pytest.mark.parametrize("rows,T,expect,expect_bwd", AUTO_REGIMES)
 def test_automatic_plan_regimes(gpu, rows, T, expect, expect_bwd):
     if (rows, T) == (2048, 10000):
-        # Tiles and row workgroups are fitted to the row: 40 chunks are 2 look-back tiles of 5 waves, or,
-        # with the row kernel forced, one workgroup of 10 waves.
-        assert hip.resolve_plan(rows, T, torch.float32, hip.FORWARD).waves == 5
-        forced = hip.resolve_plan(rows, T, torch.float32, hip.FORWARD, hip.Plan(mode=ROW))
-        assert (forced.waves, forced.waves_per_row, forced.unroll) == (10, 10, 4)
+        # Tiles and row workgroups are fitted to the row: 40 chunks are 2 look-back tiles of 5 waves
+        # (backward), or one workgroup of 10 waves (forward; 16-bit storage takes the tiles there too).
+        assert hip.resolve_plan(rows, T, torch.float32, hip.BACKWARD).waves == 5
+        fwd = hip.resolve_plan(rows, T, torch.float32, hip.FORWARD)
+        assert (fwd.waves, fwd.waves_per_row, fwd.unroll) == (10, 10, 4)
+        assert hip.resolve_plan(rows, 2 * T, torch.bfloat16, hip.FORWARD).mode == LOOKBACK
     plan = hip.resolve_plan(rows, T, torch.float32, hip.FORWARD)
     assert (plan.mode, plan.waves_per_row, plan.unroll) == expect, plan
     plan = hip.resolve_plan(rows, T, torch.float32, hip.BACKWARD)
