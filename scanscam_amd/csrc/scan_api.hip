@@ -216,7 +216,7 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
                 // 8 elements per lane and chunk), and with 2 chunks per wave they need half the registers, so
                 // twice the waves cover each other: bf16 [3883, 8640] 41.5 / 63.6 us -> 35.1 / 59.4 us, element-
                 // aligned [3297, 10175] 46.1 / 69.3 -> 35.9 / 60.8 us. From 32 chunks on the single step wins back.
-                if (esize == 2 && nch <= (l.ragged ? 28 : 24)) {
+                if (esize == 2 && l.vec == full && nch <= (l.ragged ? 28 : 24)) {
                     l.unroll = 2;
                     l.wpr = l.waves = (nch + 3) / 4;
                 }

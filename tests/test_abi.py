@@ -154,3 +154,30 @@ def test_lookback_workspace_size_formula():
     # tile = 2 waves * 2 chunks * 256 elements = 1024 elements; 5 tiles per row of 4100;
     # one ticket counter (a 16-word line) per row, 2 words per tile, 4 per super-tile of 64 tiles.
     assert hip.workspace_bytes(3, 4100, torch.float32, hip.FORWARD, plan) == (3 * 16 + 3 * 5 * 2 + 3 * 1 * 4) * 8
+
+
+def test_every_automatic_plan_is_a_valid_plan():
+    # The rules that pick the launch shape (rows per workgroup, waves fitted to the row, chunks per wave by
+    # storage type, kernel family by direction) must never produce a shape the library then refuses:
+    # sizes on both sides of every rule's borders, all storage types, both directions, with and without
+    # one element per lane forced.
+    L = hip.lib()
+    lengths = list(range(1, 70)) + [100, 127, 128, 129, 255, 256, 257, 500, 511, 512, 513, 1000, 1001, 1023, 1024,
+                                    1025, 1280, 1500, 2047, 2048, 2049, 3000, 4096, 4097, 4100, 5000, 8191, 8192,
+                                    8640, 8704, 10000, 10001, 12223, 12288, 12289, 14271, 14336, 16320, 16384,
+                                    16640, 20000, 33333, 65536, 65537, 100000, 131072, 1000001, 1 << 22]
+    checked = 0
+    for dtype in (torch.float32, torch.bfloat16, torch.float16, torch.float64):
+        code = hip._dtype_code(dtype)
+        for rows in (1, 3, 16, 255, 256, 700, 5000, 100000):
+            for T in lengths:
+                for direction in (hip.FORWARD, hip.BACKWARD):
+                    for vec in (0, 1):
+                        plan, out = hip.Plan(vec=vec), hip.Plan()
+                        rc = L.scanscam_resolve_plan(rows, T, code, direction, ctypes.byref(plan), ctypes.byref(out))
+                        assert rc == 0, (dtype, rows, T, direction, vec, hip.strerror(rc))
+                        assert 1 <= out.waves <= 16 and out.unroll in (1, 2, 4, 8) and out.mode in (1, 2, 3)
+                        if out.mode == 2:
+                            assert out.waves_per_row >= 1 and out.waves % out.waves_per_row == 0
+                        checked += 1
+    assert checked > 10000
