@@ -43,7 +43,7 @@ struct ClArgs {
     int32_t C;
     int32_t segments;   // look-back kernel: tiles per (batch element, channel group)
     int32_t group;      // packed kernel: lanes per time step (power of two below 64)
-    int32_t xcd_order;  // scan_cl_kernel: consecutive (batch element, channel group) pairs share an XCD
+    int32_t xcd_order;  // scan_cl_kernel, scan_cl_lookback_kernel: consecutive (batch element, channel group) pairs share an XCD
     uint64_t *ws;       // look-back kernel: ticket counters + published pairs
     int32_t spin_limit; // look-back kernel: polls before a wait gives up
 };
@@ -192,6 +192,15 @@ __device__ __forceinline__ void cl_tile(const ClLane<ST> &ln, int T, int tile0, 
     if (APPLY) steps.apply(ln, T, mine);
 }
 
+// Index r of n, dealt round-robin to the 8 XCDs (r % 8), mapped so that every XCD holds one contiguous run
+// of the n indices: a permutation of 0 ... n-1.
+__device__ __forceinline__ int xcd_contiguous(int r, int n)
+{
+    const int per = (n + 7) / 8, rem = n % 8 == 0 ? 8 : n % 8;
+    const int xcd = r % 8, slot = r / 8;
+    return xcd < rem ? xcd * per + slot : rem * per + (xcd - rem) * (per - 1) + slot;
+}
+
 template <typename ST, int VEC>
 __device__ __forceinline__ ClLane<ST> cl_lane(const ClArgs &p, int64_t batch_index, int group, int lane)
 {
@@ -229,12 +238,7 @@ __global__ __launch_bounds__(MAXT) void scan_cl_kernel(const ClArgs p)
     // every time step; handled by different XCDs that line is fetched twice and written in two parts.
     // xcd_order gives each XCD a contiguous run of (batch element, channel group) pairs instead, so that
     // neighbours meet in one L2.
-    int bid = blockIdx.x;
-    if (p.xcd_order) {
-        const int n = gridDim.x, per = (n + 7) / 8, rem = n % 8 == 0 ? 8 : n % 8;
-        const int xcd = bid % 8, slot = bid / 8;
-        bid = xcd < rem ? xcd * per + slot : rem * per + (xcd - rem) * (per - 1) + slot;
-    }
+    const int bid = p.xcd_order ? xcd_contiguous((int)blockIdx.x, (int)gridDim.x) : (int)blockIdx.x;
     const ClLane<ST> ln = cl_lane<ST, VEC>(p, bid / groups, bid % groups, lane);
 
     const int tile_steps = W * S;
@@ -480,7 +484,11 @@ __global__ __launch_bounds__(MAXT) void scan_cl_lookback_kernel(const ClArgs p)
     const int W = blockDim.x / kWave;
     const int groups = (p.C + kWave * VEC - 1) / (kWave * VEC);
     const int64_t rowgroups = p.batch * groups;
-    const int64_t rg = blockIdx.x % rowgroups;
+    // Row-groups of a workgroup's XCD: with p.xcd_order (time steps that are not whole 128-byte lines) a
+    // contiguous run of them, so that channel groups that share a line meet in one L2 (as in scan_cl_kernel;
+    // exact when the number of row-groups is a multiple of 8, where a row-group keeps its XCD over all tiles).
+    const int64_t rg0 = blockIdx.x % rowgroups;
+    const int64_t rg = (p.xcd_order && rowgroups % 8 == 0) ? xcd_contiguous((int)rg0, (int)rowgroups) : rg0;
 
     if (threadIdx.x == 0)
         lds_ticket = __hip_atomic_fetch_add(reinterpret_cast<unsigned *>(p.ws + rg * kCounterStride), 1u,

@@ -213,8 +213,8 @@ def test_few_channels_packed_kernel(gpu, dtype):
 # (dtype, [batch, T, C], slice of C taken from a wider buffer or None). Automatic plans on grids of 64 and
 # more workgroups: time steps that are not whole 128-byte lines (every XCD then takes a contiguous run of
 # workgroups; numbers of workgroups that are and are not multiples of 8, dense tensors and views whose
-# rows are whole lines but start inside one), 320 workgroups of 16-byte lanes (4-wave workgroups), and
-# 16-bit single-channel lanes with 16 steps per wave.
+# rows are whole lines but start inside one; also with time split over workgroups), 320 workgroups of
+# 16-byte lanes (4-wave workgroups), and 16-bit single-channel lanes with 16 steps per wave.
 MANY_WORKGROUPS = [
     (torch.float32, (37, 300, 1000), None),
     (torch.float32, (67, 90, 1000), None),
@@ -227,6 +227,8 @@ MANY_WORKGROUPS = [
     (torch.float64, (40, 100, 500), None),
     (torch.float32, (20, 150, 1000), (8, 1056)),
     (torch.bfloat16, (24, 140, 1024), (16, 1088)),
+    (torch.float32, (8, 2100, 500), None),      # time split over workgroups, 64 row-groups: XCD runs there too
+    (torch.bfloat16, (8, 1500, 1000), None),
     (torch.float32, (80, 200, 1024), None),
     (torch.bfloat16, (16, 1100, 1024), None),
 ]
