@@ -470,10 +470,11 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         if (C <= 32 && (esize == 2 || pow2_ceil(C) <= 16 || is_pow2((int)C))) l->vec = narrow;
         // 16-bit storage, 33 to 511 channels: with 8 channels per lane a time step fills only part of a wave, and
         // the kernel that then packs several steps into a wave needs more registers than it has (bf16
-        // [256, 512, 256]: 28 / 29 % of peak; [256, 4096, 64]: 25 / 28 %). One channel per lane up to 64 channels
-        // (a full wave: 61 / 62 %), two above (66 / 68 % at 256 channels; 47 / 48 % at 96, where single channels
-        // would split a step into a full and a half-empty wave: 33 / 31 %).
-        if (esize == 2 && C > 32 && C < (int64_t)kWave * full) l->vec = (C <= kWave || !pair_possible) ? 1 : 2;
+        // [256, 512, 256]: 28 / 29 % of peak; [256, 4096, 64]: 25 / 28 %). One channel per lane at exactly 64
+        // channels (a full wave: 61 / 62 %), two otherwise (66 / 68 % at 256 channels; 47 / 48 % at 96, where single
+        // channels would split a step into a full and a half-empty wave: 33 / 31 %; 46 / 46 % at 56, two steps per
+        // instruction, against 33 / 29 %).
+        if (esize == 2 && C > 32 && C < (int64_t)kWave * full) l->vec = (C == kWave || !pair_possible) ? 1 : 2;
     }
     if (l->vec != 1 && l->vec != full && !(l->vec == 2 && esize == 2)) return SCANSCAM_EPLAN;
     if (l->vec == full && !vec_possible) return SCANSCAM_EPLAN;
