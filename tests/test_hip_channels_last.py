@@ -230,6 +230,11 @@ MANY_WORKGROUPS = [
     (torch.float32, (8, 2100, 500), None),      # time split over workgroups, 64 row-groups: XCD runs there too
     (torch.bfloat16, (8, 1500, 1000), None),
     (torch.float32, (80, 200, 1024), None),
+    (torch.bfloat16, (260, 130, 64), None),     # 16-bit, 33-511 channels: one channel per lane at 64 ...
+    (torch.bfloat16, (260, 130, 96), None),     # ... pairs otherwise (48 lanes of a wave)
+    (torch.float16, (300, 100, 40), None),      # (two time steps per instruction)
+    (torch.bfloat16, (257, 64, 256), None),
+    (torch.bfloat16, (9, 3000, 64), None),      # the same with time split over workgroups
     (torch.bfloat16, (16, 1100, 1024), None),
 ]
 
