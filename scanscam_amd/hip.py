@@ -535,8 +535,12 @@ def _check_same(*tensors: torch.Tensor) -> None:
             raise RuntimeError(f"scanscam_amd.hip: expected GPU tensors on one device, got {t.device}")
         if t.dtype != first.dtype:
             raise TypeError(f"scanscam_amd.hip: tensors differ in dtype ({first.dtype} and {t.dtype})")
-        if t.shape != first.shape or t.dim() < 1:
-            raise AssertionError("scanscam_amd.hip: expected tensors of one shape with at least 1 dimension")
+        # The reference's contract for every scan (scanscam/decorator.py:19-20, 37-39).
+        if t.shape != first.shape:
+            raise AssertionError(
+                f"scan arguments must have one shape, got {tuple(first.shape)} and {tuple(t.shape)}")
+        if t.dim() < 2:
+            raise AssertionError(f"scan arguments need at least 2 dimensions, got shape {tuple(t.shape)}")
 
 
 def _plan_ref(plan: Optional[Plan]):

@@ -27,6 +27,13 @@ def pytest_configure(config):
         __graft_entry__.build()
 
 
+def pytest_report_header(config):
+    # Which build of the HIP library this session loads (SCANSCAM_HIP_LIB may point at another one).
+    from scanscam_amd import hip
+
+    return f"scanscam_amd HIP library: {hip.LIB_PATH} ({'loaded' if hip.has_hip_ops else 'NOT loaded'})"
+
+
 @pytest.fixture(scope="session")
 def gpu():
     """The GPU device; GPU tests fail loudly (not skip) if the HIP library is missing."""

@@ -91,6 +91,48 @@ def test_gpu_entry_points_reject_cpu_tensors_and_unknown_dtypes():
         hip.resolve_plan(4, 8, torch.int32)
 
 
+def test_reference_import_names_resolve_to_this_package():
+    """Code written against the reference imports `scanscam...` (scanscam/cuda_test.py:7-16,
+    scanscam/cpu_test.py:7-8, scanscam/op.py:5-6); every such name must lead here."""
+    import scanscam
+    import scanscam.cuda
+    from scanscam import cpu, cuda  # noqa: F401
+    from scanscam.baseline import naive_linear_scan_backward, naive_linear_scan_forward
+    from scanscam.cpu import simple_linear_scan_backward, simple_linear_scan_forward
+    from scanscam.cuda import (
+        blocked_linear_scan_backward,
+        blocked_linear_scan_forward,
+        coalesced_linear_scan_forward,
+        simple_linear_scan_backward as gpu_simple_backward,
+        simple_linear_scan_forward as gpu_simple_forward,
+        transposed_linear_scan_backward,
+        transposed_linear_scan_forward,
+    )
+    from scanscam.decorator import preprocess_backward_scan_args, preprocess_scan_args
+    from scanscam.op import Scan, is_transpose_contig, scan
+
+    assert scanscam.scan is scanscam_amd.scan and scan is scanscam_amd.scan and Scan is op.Scan
+    assert scanscam.__all__ == ["scan"]  # scanscam/__init__.py:3
+    assert is_transpose_contig is op.is_transpose_contig
+    assert scanscam.cuda is scanscam_amd.cuda and scanscam.cpu is scanscam_amd.cpu
+    assert blocked_linear_scan_forward is hip.blocked_linear_scan_forward
+    assert blocked_linear_scan_backward is hip.blocked_linear_scan_backward
+    assert transposed_linear_scan_forward is hip.transposed_linear_scan_forward
+    assert transposed_linear_scan_backward is hip.transposed_linear_scan_backward
+    assert coalesced_linear_scan_forward is gpu_simple_forward is hip.blocked_linear_scan_forward
+    assert gpu_simple_backward is hip.blocked_linear_scan_backward
+    assert naive_linear_scan_forward is baseline.naive_linear_scan_forward
+    assert naive_linear_scan_backward is baseline.naive_linear_scan_backward
+    assert simple_linear_scan_forward is scanscam_amd.cpu.simple_linear_scan_forward
+    assert simple_linear_scan_backward is scanscam_amd.cpu.simple_linear_scan_backward
+    assert preprocess_scan_args is decorator.preprocess_scan_args
+    assert preprocess_backward_scan_args is decorator.preprocess_backward_scan_args
+    # The op itself, called through the reference's name on CPU tensors.
+    g = torch.Generator().manual_seed(5)
+    a, b = torch.rand((3, 4, 9), generator=g), torch.randn((3, 4, 9), generator=g)
+    assert np.allclose(scanscam.scan(a, b).numpy(), oracle.fwd(a.numpy(), b.numpy()), rtol=1e-5, atol=1e-4)
+
+
 def _levels(*tensors):
     return hip._two_levels(tensors[0].shape[:-1], [t.stride()[:-1] for t in tensors])
 

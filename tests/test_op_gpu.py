@@ -93,6 +93,24 @@ def test_wrapper_names_of_the_reference(gpu):
         hip.blocked_linear_scan_forward(a.long(), b.long())
 
 
+def test_fewer_than_two_dimensions_are_refused_as_in_the_reference(gpu):
+    # scanscam/decorator.py:19-20, 37-39: every scan asserts len(shape) >= 2. The op's GPU path, which does
+    # not go through the decorators, must raise the same error as the CPU paths do.
+    a = torch.rand(64, device=gpu, requires_grad=True)
+    b = torch.randn(64, device=gpu)
+    with pytest.raises(AssertionError):
+        scanscam_amd.scan(a, b)
+    with pytest.raises(AssertionError):
+        hip.scan_forward(a.detach(), b)
+    with pytest.raises(AssertionError):
+        hip.scan_backward(a.detach(), b, b)
+    with pytest.raises(AssertionError):
+        scanscam_amd.scan(a.detach().cpu(), b.cpu())  # same input, CPU branch
+    with pytest.raises(AssertionError):
+        hip.scan_forward(a.detach().reshape(1, 64), b.reshape(2, 32))
+    assert scanscam_amd.scan(a.reshape(1, 64), b.reshape(1, 64)).shape == (1, 64)
+
+
 def test_reference_module_and_function_names(gpu):
     # A test written for the reference (scanscam/cuda_test.py:19-126: each wrapper of scanscam.cuda
     # against the tensor-level loop, N(0,1) inputs, atol 1e-4) runs against scanscam_amd.cuda unchanged.
