@@ -48,7 +48,8 @@ enum {
     SCANSCAM_EALIGN = 3,    /* pointer not aligned to its element size, or workspace not to 8 bytes */
     SCANSCAM_EPLAN = 4,     /* explicit plan not valid for this shape / alignment */
     SCANSCAM_EWORKSPACE = 5,/* workspace missing or smaller than scanscam_workspace_bytes() */
-    SCANSCAM_ELAUNCH = 6    /* the HIP runtime refused the launch */
+    SCANSCAM_ELAUNCH = 6,   /* the HIP runtime refused the launch */
+    SCANSCAM_ESCRATCH = 7   /* scanscam_scan_fwd_noalloc: the shape needs more than SCANSCAM_NOALLOC_SCRATCH_BYTES */
 };
 
 /* Kernel families. */
@@ -96,6 +97,24 @@ int scanscam_scan_fwd(const void *a, const void *b, void *h, int64_t rows, int64
  */
 int scanscam_scan_bwd(const void *a, const void *h, const void *gh, void *ga, void *gb, int64_t rows,
                       int64_t T, int dtype, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * scanscam_scan_fwd for callers that cannot allocate device memory: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc. It has no counterpart in the reference (whose
+ * kernels need no workspace, src/scanscam_cuda.cu:260-307). Same arguments, results (bit for bit) and
+ * errors as scanscam_scan_fwd, without the workspace: where rows are split over workgroups, the
+ * look-back descriptors live in a fixed array of SCANSCAM_NOALLOC_SCRATCH_BYTES in the GPU's memory
+ * that belongs to the library (one per GPU it runs on, held until the process ends), found once per
+ * device on the first call there. The call itself allocates and frees nothing, on the device or
+ * through any library. A shape whose descriptors do not fit (more than about 65 000 look-back tiles,
+ * i.e. 0.5 G fp32 elements in long rows) is refused with SCANSCAM_ESCRATCH and nothing is launched.
+ * Every call clears the part of the array it uses, with a kernel on `stream`. All calls on one GPU
+ * share that GPU's array: calls that may overlap in time on one GPU (two streams, two threads) race
+ * and must use scanscam_scan_fwd with separate workspaces instead.
+ */
+#define SCANSCAM_NOALLOC_SCRATCH_BYTES (1 << 20)
+int scanscam_scan_fwd_noalloc(const void *a, const void *b, void *h, int64_t rows, int64_t T, int dtype,
+                              void *stream);
 
 /*
  * Bytes of device workspace the call above of that direction needs for this

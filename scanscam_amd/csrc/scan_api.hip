@@ -4,6 +4,14 @@
 
 #include "scan_launch.hpp"
 
+#include <mutex>
+
+// Look-back scratch of scanscam_scan_fwd_noalloc: a fixed array in every GPU's memory that the library
+// runs on, held until the process ends. Host code never uses this name as an address -- it is a
+// host-side stand-in for the symbol; noalloc_scratch() asks the runtime where the current device keeps
+// its copy and hands that pointer to the kernels.
+static __device__ __align__(256) unsigned char scratch[SCANSCAM_NOALLOC_SCRATCH_BYTES];
+
 namespace {
 
 using scanscam::kCounterStride;
@@ -277,6 +285,25 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
 
 bool aligned_to(const void *p, size_t n) { return (reinterpret_cast<uintptr_t>(p) % n) == 0; }
 
+// Address of `scratch` on the current device: looked up once per device, with that device current
+// (every GPU holds its own copy of the array at its own address), and kept.
+constexpr int kMaxDevices = 64;
+int noalloc_scratch(void **out)
+{
+    static std::mutex lock;
+    static void *ptr[kMaxDevices];  // zero-initialised: not looked up yet
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return SCANSCAM_ELAUNCH;
+    std::lock_guard<std::mutex> hold(lock);
+    if (!ptr[dev]) {
+        void *p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return SCANSCAM_ELAUNCH;
+        ptr[dev] = p;
+    }
+    *out = ptr[dev];
+    return SCANSCAM_OK;
+}
+
 const scanscam_strides *const kDense[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
 
 // Tensor order everywhere below: a, x, h, y0, y1 (x = b forwards, gh backwards; y0 = h forwards,
@@ -284,7 +311,7 @@ const scanscam_strides *const kDense[5] = {nullptr, nullptr, nullptr, nullptr, n
 int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y1,
         const scanscam_strides *const st[5], int64_t n0, int64_t n1, int64_t T, int dtype, void *workspace,
         size_t workspace_bytes, void *stream, const scanscam_plan *plan, void *start_event = nullptr,
-        void *stop_event = nullptr)
+        void *stop_event = nullptr, bool use_scratch = false)
 {
     const int esize = elem_size(dtype);
     if (esize == 0) return SCANSCAM_EDTYPE;
@@ -387,6 +414,14 @@ int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y
     };
 
     if (r.l.mode == kModeLookback) {
+        if (use_scratch) {
+            // The library's own fixed array instead of a caller's workspace; every call clears the part
+            // it uses (below), whatever the call before left there.
+            if (r.ws_bytes > (size_t)SCANSCAM_NOALLOC_SCRATCH_BYTES) return SCANSCAM_ESCRATCH;
+            const int src = noalloc_scratch(&workspace);
+            if (src != SCANSCAM_OK) return src;
+            workspace_bytes = SCANSCAM_NOALLOC_SCRATCH_BYTES;
+        }
         if (!workspace || workspace_bytes < r.ws_bytes) return SCANSCAM_EWORKSPACE;
         if (!aligned_to(workspace, 8)) return SCANSCAM_EALIGN;
         args.ws = static_cast<uint64_t *>(workspace);
@@ -663,6 +698,12 @@ int scanscam_scan_bwd(const void *a, const void *h, const void *gh, void *ga, vo
     return run(true, a, gh, h, gb, ga, kDense, 1, rows, T, dtype, workspace, workspace_bytes, stream, nullptr);
 }
 
+int scanscam_scan_fwd_noalloc(const void *a, const void *b, void *h, int64_t rows, int64_t T, int dtype, void *stream)
+{
+    return run(false, a, b, nullptr, h, nullptr, kDense, 1, rows, T, dtype, nullptr, 0, stream, nullptr, nullptr, nullptr,
+               /*use_scratch=*/true);
+}
+
 size_t scanscam_workspace_bytes(int64_t rows, int64_t T, int dtype, int direction)
 {
     return workspace_for(rows, T, dtype, direction, nullptr);
@@ -797,6 +838,9 @@ const char *scanscam_strerror(int code)
     case SCANSCAM_EPLAN: return "launch plan not valid for this shape or alignment";
     case SCANSCAM_EWORKSPACE: return "workspace missing or smaller than scanscam_workspace_bytes()";
     case SCANSCAM_ELAUNCH: return "HIP runtime refused the kernel launch";
+    case SCANSCAM_ESCRATCH:
+        return "shape needs more look-back scratch than the library's fixed array (scanscam_scan_fwd_noalloc): "
+               "use scanscam_scan_fwd with a workspace";
     default: return "unknown scanscam error code";
     }
 }

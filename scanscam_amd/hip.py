@@ -81,6 +81,8 @@ def _bind(path: str) -> ctypes.CDLL:
     lib.scanscam_scan_fwd.restype = i32
     lib.scanscam_scan_bwd.argtypes = [p, p, p, p, p, i64, i64, i32, p, sz, p]
     lib.scanscam_scan_bwd.restype = i32
+    lib.scanscam_scan_fwd_noalloc.argtypes = [p, p, p, i64, i64, i32, p]
+    lib.scanscam_scan_fwd_noalloc.restype = i32
     lib.scanscam_workspace_bytes.argtypes = [i64, i64, i32, i32]
     lib.scanscam_workspace_bytes.restype = sz
     lib.scanscam_scan_fwd_plan.argtypes = [p, p, p, i64, i64, i32, p, sz, p, plan_p]

@@ -147,6 +147,12 @@ static int check_case(const char *name, long rows, long T, long C, int channels_
         HIP_OK(hipEventElapsedTime(&ms, ev0, ev1));
         HIP_OK(hipMemcpy(got, o0, n * 4, hipMemcpyDeviceToHost));
         if (memcmp(got, again, n * 4) != 0 || worst(got, h, n) > 1e-5 || !(ms > 0.0f && ms < 100.0f)) failures++;
+        /* And without a workspace: the entry point for callers that cannot allocate gives the same bits. */
+        HIP_OK(hipMemset(o0, 0, n * 4));
+        if (scanscam_scan_fwd_noalloc(da, db, o0, rows, T, SCANSCAM_F32, stream) != SCANSCAM_OK) failures++;
+        HIP_OK(hipStreamSynchronize(stream));
+        HIP_OK(hipMemcpy(got, o0, n * 4, hipMemcpyDeviceToHost));
+        if (memcmp(got, again, n * 4) != 0) failures++;
         if (scanscam_scan_bwd_plan(da, dh, dgh, o1, o0, rows, T, SCANSCAM_F32, ws, ws_bytes, stream, NULL) != SCANSCAM_OK)
             failures++;
         HIP_OK(hipStreamSynchronize(stream));

@@ -32,7 +32,7 @@ def test_library_is_built_and_loads():
 
 def test_every_declared_symbol_is_exported():
     names = declared_functions()
-    assert "scanscam_scan_fwd" in names and "scanscam_scan_bwd" in names and len(names) == 18
+    assert "scanscam_scan_fwd" in names and "scanscam_scan_bwd" in names and len(names) == 19
     raw = ctypes.CDLL(hip.LIB_PATH)
     for name in names:
         assert hasattr(raw, name), f"{name} declared in scanscam_hip.h but not exported"
@@ -51,7 +51,7 @@ def test_header_is_plain_c():
 
 def test_strerror_covers_every_code():
     seen = set()
-    for code in range(7):
+    for code in range(8):
         msg = hip.strerror(code)
         assert msg and msg not in seen
         seen.add(msg)
