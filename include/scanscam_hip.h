@@ -219,6 +219,15 @@ int scanscam_scan_bwd_cl_strided(const void *a, const void *h, const void *gh, v
                                  void *workspace, size_t workspace_bytes, void *stream, const scanscam_plan *plan);
 
 /*
+ * Whether a wait for another workgroup's carry expired in a call that used this workspace (see
+ * spin_limit in scanscam_plan): waits for the work on `stream` to finish, reads the workspace's flag
+ * word and writes 1 or 0 to *timed_out. A correct launch never sets it; where it is set, the
+ * affected outputs hold NaN. Meant for debugging and tests: it blocks the host. No counterpart in
+ * the reference.
+ */
+int scanscam_workspace_timed_out(const void *workspace, void *stream, int *timed_out);
+
+/*
  * Writes the plan the automatic choice resolves to for this shape (assuming
  * 16-byte aligned pointers) into *out. Returns 0 or an error code.
  */

@@ -809,6 +809,19 @@ int scanscam_scan_bwd_cl_strided(const void *a, const void *h, const void *gh, v
     return run_cl(true, a, gh, h, gb, ga, st, batch, T, C, dtype, workspace, workspace_bytes, stream, plan);
 }
 
+int scanscam_workspace_timed_out(const void *workspace, void *stream, int *timed_out)
+{
+    if (!workspace || !timed_out) return SCANSCAM_EINVAL;
+    if (!aligned_to(workspace, 8)) return SCANSCAM_EALIGN;
+    uint64_t word = 0;
+    if (hipStreamSynchronize(static_cast<hipStream_t>(stream)) != hipSuccess) return SCANSCAM_ELAUNCH;
+    if (hipMemcpy(&word, static_cast<const uint64_t *>(workspace) + scanscam::kTimeoutWord, sizeof(word),
+                  hipMemcpyDeviceToHost) != hipSuccess)
+        return SCANSCAM_ELAUNCH;
+    *timed_out = word != 0 ? 1 : 0;
+    return SCANSCAM_OK;
+}
+
 int scanscam_resolve_plan(int64_t rows, int64_t T, int dtype, int direction, const scanscam_plan *plan,
                           scanscam_plan *out)
 {
@@ -845,6 +858,6 @@ const char *scanscam_strerror(int code)
     }
 }
 
-int scanscam_abi_version(void) { return 1; }
+int scanscam_abi_version(void) { return 2; }
 
 }  // extern "C"

@@ -29,7 +29,7 @@ LIB_PATH = os.environ.get("SCANSCAM_HIP_LIB") or os.path.join(_HERE, "libscansca
 
 MODE_AUTO, MODE_SMALL, MODE_ROW, MODE_LOOKBACK = 0, 1, 2, 3
 FORWARD, BACKWARD = 0, 1
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _DTYPES = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2, torch.float64: 3}
 
@@ -101,6 +101,8 @@ def _bind(path: str) -> ctypes.CDLL:
     lib.scanscam_scan_bwd_cl.restype = i32
     lib.scanscam_workspace_bytes_cl.argtypes = [i64, i64, i64, i32, i32, plan_p]
     lib.scanscam_workspace_bytes_cl.restype = sz
+    lib.scanscam_workspace_timed_out.argtypes = [p, p, ctypes.POINTER(ctypes.c_int)]
+    lib.scanscam_workspace_timed_out.restype = i32
     lib.scanscam_resolve_plan.argtypes = [i64, i64, i32, i32, plan_p, plan_p]
     lib.scanscam_resolve_plan.restype = i32
     lib.scanscam_strerror.argtypes = [i32]
@@ -116,7 +118,7 @@ _lib: Optional[ctypes.CDLL] = None
 _load_error: Optional[str] = None
 try:
     _lib = _bind(LIB_PATH)
-except OSError as exc:  # not built, or built for another ABI
+except (OSError, AttributeError) as exc:  # not built, or built for another ABI
     _load_error = str(exc)
 
 has_hip_ops = _lib is not None
@@ -413,9 +415,21 @@ simple_linear_scan_backward = blocked_linear_scan_backward
 has_cuda_ops = has_hip_ops
 
 
-def _workspace_cl(L, batch: int, T: int, C: int, dtype: torch.dtype, direction: int, plan_ref,
+@functools.lru_cache(maxsize=4096)
+def _workspace_bytes_cl_auto(batch: int, T: int, C: int, code: int, direction: int) -> int:
+    return int(lib().scanscam_workspace_bytes_cl(batch, T, C, code, direction, None))
+
+
+def workspace_bytes_cl(batch: int, T: int, C: int, dtype: torch.dtype, direction: int = FORWARD,
+                       plan: Optional[Plan] = None) -> int:
+    if plan is None:
+        return _workspace_bytes_cl_auto(batch, T, C, _dtype_code(dtype), direction)
+    return int(lib().scanscam_workspace_bytes_cl(batch, T, C, _dtype_code(dtype), direction, ctypes.byref(plan)))
+
+
+def _workspace_cl(L, batch: int, T: int, C: int, dtype: torch.dtype, direction: int, plan: Optional[Plan],
                   device: torch.device) -> Tuple[Optional[torch.Tensor], int, int]:
-    n = int(L.scanscam_workspace_bytes_cl(batch, T, C, _dtype_code(dtype), direction, plan_ref))
+    n = workspace_bytes_cl(batch, T, C, dtype, direction, plan)
     if n == 0:
         return None, 0, 0
     ws = torch.empty(n, dtype=torch.uint8, device=device)
@@ -451,7 +465,7 @@ def transposed_linear_scan_forward(x: torch.Tensor, y: torch.Tensor, channels_pe
         return out
     plan_ref = ctypes.byref(plan) if plan is not None else None
     with _on(x.device):
-        ws, ws_ptr, ws_n = _workspace_cl(L, batch, T, C, x.dtype, FORWARD, plan_ref, x.device)
+        ws, ws_ptr, ws_n = _workspace_cl(L, batch, T, C, x.dtype, FORWARD, plan, x.device)
         rc = L.scanscam_scan_fwd_cl(x.data_ptr(), y.data_ptr(), out.data_ptr(), batch, T, C, _dtype_code(x.dtype),
                                     ws_ptr, ws_n, torch.cuda.current_stream().cuda_stream, plan_ref)
     if rc != 0:
@@ -473,13 +487,53 @@ def transposed_linear_scan_backward(x: torch.Tensor, y: torch.Tensor, z: torch.T
         return out_a, out_b
     plan_ref = ctypes.byref(plan) if plan is not None else None
     with _on(x.device):
-        ws, ws_ptr, ws_n = _workspace_cl(L, batch, T, C, x.dtype, BACKWARD, plan_ref, x.device)
+        ws, ws_ptr, ws_n = _workspace_cl(L, batch, T, C, x.dtype, BACKWARD, plan, x.device)
         rc = L.scanscam_scan_bwd_cl(x.data_ptr(), y.data_ptr(), z.data_ptr(), out_a.data_ptr(), out_b.data_ptr(),
                                     batch, T, C, _dtype_code(x.dtype), ws_ptr, ws_n,
                                     torch.cuda.current_stream().cuda_stream, plan_ref)
     if rc != 0:
         raise RuntimeError(f"scanscam_scan_bwd_cl: {strerror(rc)}")
     return out_a, out_b
+
+
+def prepare_forward_cl(x: torch.Tensor, y: torch.Tensor, out: torch.Tensor, plan: Optional[Plan] = None):
+    """``prepare_forward`` for contiguous ``[batch, T, C]`` tensors: a callable that launches this scan again."""
+    L = lib()
+    _check_channels_last(x, y, out)
+    batch, T, C = x.shape
+    ws, ws_ptr, ws_n = _workspace_cl(L, batch, T, C, x.dtype, FORWARD, plan, x.device)
+    args = (x.data_ptr(), y.data_ptr(), out.data_ptr(), batch, T, C, _dtype_code(x.dtype), ws_ptr, ws_n)
+    plan_ref = _plan_ref(plan)
+    keep = (x, y, out, ws, plan)
+    current_stream = torch.cuda.current_stream
+
+    def launch(_keep=keep) -> None:
+        rc = L.scanscam_scan_fwd_cl(*args, current_stream().cuda_stream, plan_ref)
+        if rc != 0:
+            raise RuntimeError(f"scanscam_scan_fwd_cl: {strerror(rc)}")
+
+    return launch
+
+
+def prepare_backward_cl(x: torch.Tensor, y: torch.Tensor, z: torch.Tensor, out_a: torch.Tensor, out_b: torch.Tensor,
+                        plan: Optional[Plan] = None):
+    """The backward counterpart of ``prepare_forward_cl`` (gate ``x``, output ``y``, output grad ``z``)."""
+    L = lib()
+    _check_channels_last(x, y, z, out_a, out_b)
+    batch, T, C = x.shape
+    ws, ws_ptr, ws_n = _workspace_cl(L, batch, T, C, x.dtype, BACKWARD, plan, x.device)
+    args = (x.data_ptr(), y.data_ptr(), z.data_ptr(), out_a.data_ptr(), out_b.data_ptr(), batch, T, C,
+            _dtype_code(x.dtype), ws_ptr, ws_n)
+    plan_ref = _plan_ref(plan)
+    keep = (x, y, z, out_a, out_b, ws, plan)
+    current_stream = torch.cuda.current_stream
+
+    def launch(_keep=keep) -> None:
+        rc = L.scanscam_scan_bwd_cl(*args, current_stream().cuda_stream, plan_ref)
+        if rc != 0:
+            raise RuntimeError(f"scanscam_scan_bwd_cl: {strerror(rc)}")
+
+    return launch
 
 
 # ---------------------------------------------------------------------------
@@ -623,7 +677,7 @@ def _run_cl(inputs, n_out: int, direction: int, plan: Optional[Plan]):
     st = [Strides(int(b), int(t.stride(-1))) for b, t in zip(sb, tensors)]
     plan_ref = _plan_ref(plan)
     with _on(first.device):
-        ws, ws_ptr, ws_n = _workspace_cl(L, batch, T, C, first.dtype, direction, plan_ref, first.device)
+        ws, ws_ptr, ws_n = _workspace_cl(L, batch, T, C, first.dtype, direction, plan, first.device)
         stream = torch.cuda.current_stream().cuda_stream
         ptrs = [t.data_ptr() for t in tensors]
         refs = [ctypes.byref(x) for x in st]

@@ -258,7 +258,7 @@ static int check_strided(const char *name, long B, long C, long T, int channels_
 
 int main(void)
 {
-    if (scanscam_abi_version() != 1) {
+    if (scanscam_abi_version() != 2) {
         fprintf(stderr, "abi_check: unexpected ABI version %d\n", scanscam_abi_version());
         return 1;
     }

@@ -32,7 +32,7 @@ def test_library_is_built_and_loads():
 
 def test_every_declared_symbol_is_exported():
     names = declared_functions()
-    assert "scanscam_scan_fwd" in names and "scanscam_scan_bwd" in names and len(names) == 19
+    assert "scanscam_scan_fwd" in names and "scanscam_scan_bwd" in names and len(names) == 20
     raw = ctypes.CDLL(hip.LIB_PATH)
     for name in names:
         assert hasattr(raw, name), f"{name} declared in scanscam_hip.h but not exported"
