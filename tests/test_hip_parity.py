@@ -619,6 +619,11 @@ def test_expired_wait_is_reported_and_every_wave_exits(gpu):
     assert rc == 0
     torch.cuda.synchronize()  # returns: no wave is left spinning
     expired = int(ws.view(torch.int64)[1].item()) != 0
+    # The library's own query of that flag says the same.
+    flag = ctypes.c_int(-1)
+    assert hip.lib().scanscam_workspace_timed_out(ws.data_ptr(), torch.cuda.current_stream().cuda_stream,
+                                                  ctypes.byref(flag)) == 0
+    assert flag.value == int(expired)
     if expired:
         assert bool(torch.isnan(out).any())
         ok = ~torch.isnan(out)
