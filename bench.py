@@ -10,6 +10,7 @@ algorithmic bytes (32 B per element: forward reads a, b and writes h = 12 B;
 backward reads a, h, grad_h and writes grad_a, grad_b = 20 B).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-configs] [--workload N]
+                    [--channels-last BxTxC[:dtype]]
 
 --workload runs another of the synthetic configurations (1, 3, 4, 4f16, 5; or `long`, `long16`) through the same timed
 region instead of configuration 2 (used for the rocprofv3 summaries under profiles/).
@@ -24,7 +25,10 @@ Prints ONE JSON line. Besides the contract fields it carries
   roofline_fwd  the same for the forward kernel;
   cpu_baseline  the reference's single-threaded CPU loop on the same tensors,
                 timed on this host (oracle/_ref if it was built, else the C
-                restatement in oracle/);
+                restatement in oracle/); every entry of `configs` carries the
+                same for its own tensors;
+  kernel_time   median over the launches after the region of forward + backward
+                kernel time per step, as GB/s (steadier than the wall-clock value);
   host_library  the package's own loop for CPU tensors on the same tensors
                 (not the baseline: several rows side by side, several threads);
   long_rows     many rows of 16K to 96K elements (long-context shapes);
@@ -52,14 +56,54 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per launch at configs[1] from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by what the same
-# counters read for a copy kernel of known size (profiles/scan_row_f32_fwd_bwd_8x2048x4096_pmc_traffic.txt).
-MEASURED_TRAFFIC = {"fwd": 805.38e6, "bwd": 1347.36e6}
+# HBM bytes per launch at configs[1] come from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by what the same
+# counters read for a copy kernel of known size. They are read from this summary, which names the
+# kernel sources it was taken with (a digest); with other sources the figure is reported as null.
+TRAFFIC_PROFILE = os.path.join("profiles", "scan_row_f32_fwd_bwd_8x2048x4096_pmc_traffic.txt")
+KERNEL_SOURCES = ("scan_kernels.hpp", "scan_launch.hpp", "scan_api.hip", "scan_f32.hip")
 METRIC = "scan HBM GB/s and % of MI355X peak, fwd and fwd+bwd, fp32 [B,C,T]"
 FWD_BYTES = {8: 24, 4: 12, 2: 6}
 BWD_BYTES = {8: 40, 4: 20, 2: 10}
 # Launches shorter than this are paced by the host's call; they are also timed replaying from a HIP graph.
 GRAPH_BELOW_MS = 0.025
+
+
+def kernel_sources_digest():
+    """sha256 over the sources the row kernels are built from (what a traffic profile is valid for)."""
+    import hashlib
+
+    d = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "scanscam_amd", "csrc", name), "rb") as f:
+            d.update(f.read())
+    return d.hexdigest()
+
+
+def measured_traffic():
+    """({"fwd": bytes, "bwd": bytes}, source) from the committed counter summary, or nulls if it is stale.
+
+    The summary carries two machine-readable lines:
+        traffic_bytes_per_launch fwd=<int> bwd=<int>
+        kernel_sources_sha256 <hex>
+    """
+    none = {"fwd": None, "bwd": None}
+    try:
+        with open(os.path.join(ROOT, TRAFFIC_PROFILE)) as f:
+            lines = f.read().splitlines()
+    except OSError:
+        return none, {"file": TRAFFIC_PROFILE, "state": "missing"}
+    vals, digest = None, None
+    for line in lines:
+        w = line.split()
+        if len(w) == 3 and w[0] == "traffic_bytes_per_launch":
+            vals = {k: int(v) for k, v in (x.split("=") for x in w[1:])}
+        if len(w) == 2 and w[0] == "kernel_sources_sha256":
+            digest = w[1]
+    if vals is None or digest is None:
+        return none, {"file": TRAFFIC_PROFILE, "state": "no machine-readable figures"}
+    if digest != kernel_sources_digest():
+        return none, {"file": TRAFFIC_PROFILE, "state": "stale: taken with other kernel sources"}
+    return vals, {"file": TRAFFIC_PROFILE, "state": "taken with these kernel sources", "kernel_sources_sha256": digest}
 
 
 # --workload: name -> (configuration number for make_config, description)
@@ -172,7 +216,8 @@ def time_kernels(sets, steps, warmup, hip, torch):
 def kernel_statistics(sets, launches, hip, torch):
     """After the timed region: `launches` more steps, every launch with its own bound events.
 
-    Returns {"fwd": (median ms, min ms, mean ms), "bwd": ...} over all of them.
+    Returns {"fwd": (median ms, min ms, mean ms), "bwd": ..., "step": ...} over all of them
+    ("step" = forward kernel + backward kernel of the same step).
     """
     runs = []
     for i in range(launches):
@@ -188,6 +233,8 @@ def kernel_statistics(sets, launches, hip, torch):
     for name, k in (("fwd", 2), ("bwd", 3)):
         ms = [r[k].elapsed_ms() for r in runs]
         out[name] = (statistics.median(ms), min(ms), statistics.fmean(ms))
+    both = [r[2].elapsed_ms() + r[3].elapsed_ms() for r in runs]  # kernel time of a whole step
+    out["step"] = (statistics.median(both), min(both), statistics.fmean(both))
     return out
 
 
@@ -428,6 +475,51 @@ def strided_views(dev, args, hip, torch):
     return out
 
 
+def channels_last_workload(spec, args, hip, torch):
+    """--channels-last BxTxC[:dtype]: forward and backward over contiguous [B, T, C] tensors (scanned along T).
+
+    Buffer sets rotate over >= 1 GiB; mean microseconds per launch over back-to-back launches. Used for the
+    rocprofv3 summaries of the channels-last kernels under profiles/; prints its own JSON line.
+    """
+    shape_s, _, dtype_s = spec.partition(":")
+    B, T, C = (int(v) for v in shape_s.lower().split("x"))
+    dtype = {"": torch.float32, "f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16,
+             "f64": torch.float64}[dtype_s]
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(0)
+    n = B * T * C
+    esize = torch.empty(0, dtype=dtype).element_size()
+    nsets = max(1, min(16, -(-(1 << 30) // (6 * n * esize))))
+    fwd, bwd = [], []
+    for _ in range(nsets):
+        a = torch.rand((B, T, C), generator=g, device=dev).to(dtype)
+        b = torch.randn((B, T, C), generator=g, device=dev).to(dtype)
+        gh = torch.randn((B, T, C), generator=g, device=dev).to(dtype)
+        h, ga, gb = (torch.empty_like(a) for _ in range(3))
+        fwd.append(hip.prepare_forward_cl(a, b, h))
+        bwd.append(hip.prepare_backward_cl(a, h, gh, ga, gb))
+    ms = []
+    for calls in (fwd, bwd):
+        for i in range(max(args.warmup, nsets)):
+            calls[i % nsets]()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for i in range(args.steps):
+            calls[i % nsets]()
+        e1.record()
+        torch.cuda.synchronize()
+        ms.append(e0.elapsed_time(e1) / args.steps)
+    print(json.dumps({
+        "workload": f"channels-last [B={B}, T={T}, C={C}] {str(dtype).replace('torch.', '')}, a ~ U(0,1), b, grad_h ~ N(0,1)",
+        "buffer_sets": nsets, "steps": args.steps,
+        "fwd_us": round(ms[0] * 1e3, 2), "bwd_us": round(ms[1] * 1e3, 2),
+        "fwd_frac": round(FWD_BYTES[esize] * n / (ms[0] * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+        "bwd_frac": round(BWD_BYTES[esize] * n / (ms[1] * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+        "fwd_bytes": FWD_BYTES[esize] * n, "bwd_bytes": BWD_BYTES[esize] * n,
+    }))
+
+
 def cpu_baseline(a, b, gh, reps):
     """The reference's CPU loop on the same tensors, one thread."""
     import numpy as np
@@ -529,6 +621,8 @@ def main():
     ap.add_argument("--no-configs", action="store_true", help="skip the other four configurations")
     ap.add_argument("--workload", default="2", choices=sorted(WORKLOADS),
                     help="synthetic configuration the timed region runs (default 2, the one the metric is quoted on)")
+    ap.add_argument("--channels-last", metavar="BxTxC[:dtype]", default=None,
+                    help="time the channels-last kernels on this shape instead (dtype f32, bf16, f16 or f64) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (rows are independent, so more GPUs would "
@@ -547,6 +641,9 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     dev = torch.device("cuda:0")
+    if args.channels_last:
+        channels_last_workload(args.channels_last, args, hip, torch)
+        return
 
     cfg, label = WORKLOADS[args.workload]
     a, b, gh = make_config(cfg, torch)
@@ -568,7 +665,7 @@ def main():
               hip.MODE_LOOKBACK: "scan_lookback_kernel"}[plan_f.mode]
     storage = {"float32": "float", "bfloat16": "__bf16", "float16": "_Float16"}[str(a.dtype).replace("torch.", "")]
     kernel = f"{family}<{storage}, {plan_f.vec}, {plan_f.unroll}, REV=%s>"
-    traffic = MEASURED_TRAFFIC if args.workload == "2" else {"fwd": None, "bwd": None}
+    traffic, traffic_source = measured_traffic() if args.workload == "2" else ({"fwd": None, "bwd": None}, None)
 
     out = {
         "metric": METRIC,
@@ -590,6 +687,11 @@ def main():
             "plan": repr(plan_f),
         },
         "frac_of_peak": round(step_gbps / HBM_PEAK_GBPS, 4),
+        # The steadier figure: median over the launches after the region of (forward + backward kernel
+        # time) per step, from events bound to the kernels (no gaps between launches in it).
+        "kernel_time": {"launches": max(50, args.steps), "fwd_bwd_median_ms": round(stats["step"][0], 4),
+                        "GBps": round(step_bytes * n / (stats["step"][0] * 1e-3) / 1e9, 1),
+                        "frac": round(step_bytes * n / (stats["step"][0] * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)},
         "elements_per_s": round(n / wall),
         "fwd": {"ms": round(fwd_ms, 4), "min_ms": round(fwd_min, 4), "GBps": round(fwd_gbps, 1),
                 "frac": round(fwd_gbps / HBM_PEAK_GBPS, 4)},
@@ -604,6 +706,7 @@ def main():
             "unit": "GB/s",
             "frac": round(bwd_gbps / HBM_PEAK_GBPS, 4),
             "traffic": traffic["bwd"],
+            "traffic_source": traffic_source,
             "bytes_per_launch": BWD_BYTES[esize] * n,
             "avg_ms": round(bwd_ms, 4),
             "min_ms": round(bwd_min, 4),
@@ -618,6 +721,7 @@ def main():
             "unit": "GB/s",
             "frac": round(fwd_gbps / HBM_PEAK_GBPS, 4),
             "traffic": traffic["fwd"],
+            "traffic_source": traffic_source,
             "bytes_per_launch": FWD_BYTES[esize] * n,
             "avg_ms": round(fwd_ms, 4),
             "min_ms": round(fwd_min, 4),
@@ -671,6 +775,11 @@ def main():
                     fwd_bwd_graph_ms=round(gf_ms + gb_ms, 4),
                     fwd_bwd_graph_frac=round((FWD_BYTES[esize] + BWD_BYTES[esize]) * cn / ((gf_ms + gb_ms) * 1e-3)
                                              / 1e9 / HBM_PEAK_GBPS, 4))
+            if not args.no_cpu and ca.dtype != torch.float64:
+                # The reference's loop on this configuration's own tensors (16-bit storage: on the fp32 upcast).
+                c = cpu_baseline(ca.float(), cb.float(), cgh.float(), reps=2)
+                others[key]["cpu_baseline"] = {k: c[k] for k in ("value", "unit", "cores", "kind", "fwd_GBps",
+                                                                 "bwd_GBps", "sample")}
             del csets, first
             torch.cuda.empty_cache()
         out["configs"] = others

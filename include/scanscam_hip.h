@@ -167,7 +167,9 @@ int scanscam_scan_bwd_timed(const void *a, const void *h, const void *gh, void *
  * GPU, time is also cut into tiles over workgroups, carried by a look-back
  * chain, which needs a workspace (scanscam_workspace_bytes_cl, same rules as
  * above); mode = SCANSCAM_MODE_ROW forbids that split, SCANSCAM_MODE_LOOKBACK
- * forces it.
+ * forces it. A time step (C channels, or the time stride of a strided call)
+ * must stay below 4 GiB / 18 = 227 MiB (the kernels address a wave's steps with
+ * 32-bit offsets from its first one): larger ones return SCANSCAM_EINVAL.
  */
 int scanscam_scan_fwd_cl(const void *a, const void *b, void *h, int64_t batch, int64_t T, int64_t C, int dtype,
                          void *workspace, size_t workspace_bytes, void *stream, const scanscam_plan *plan);

@@ -625,6 +625,10 @@ int run_cl(bool rev, const void *a, const void *x, const void *h, void *y0, void
     scanscam::ClLaunch l;
     const int rc = resolve_cl(plan, batch, T, C, dtype, aligned16, aligned4, &l);
     if (rc != SCANSCAM_OK) return rc;
+    // A wave addresses its steps (at most 16, and one neighbour on either side backwards) with 32-bit byte
+    // offsets from its first one, the lane's channel included.
+    for (int k = 0; k < 5; k++)
+        if ((uint64_t)sT[k] * (uint64_t)esize * 18u + (uint64_t)C * (uint64_t)esize >= (uint64_t(1) << 32)) return SCANSCAM_EINVAL;
 
     scanscam::ClArgs args;
     args.a = a;

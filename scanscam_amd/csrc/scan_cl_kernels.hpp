@@ -48,13 +48,98 @@ struct ClArgs {
     int32_t spin_limit; // look-back kernel: polls before a wait gives up
 };
 
-// One workgroup's view of its channels: pointers already offset to (batch
-// element, first channel of the lane).
+// One workgroup's view of its channels: pointers offset to the batch element
+// (the same in every lane, so they live in scalar registers, and so does every
+// time-step offset added to them) and the lane's first channel `c`, the only
+// per-lane part of an address: loads and stores then take the scalar-base form
+// with one shared 32-bit lane offset instead of a 64-bit address pair in vector
+// registers per access.
 template <typename ST> struct ClLane {
     const ST *a, *x, *h;
     ST *y0, *y1;
     int pa, px, ph, py0, py1;  // elements from one time step to the next, per tensor
+    unsigned c;                // byte offset of the lane's first channel (0 for a lane without channels)
     bool c_ok;
+
+    // base + elems elements + the lane's channel offset. The lane part enters as a zero-extended 32-bit
+    // byte count, the form the scalar-base addressing mode takes.
+    static __device__ __forceinline__ const ST *at(const ST *base, int64_t elems, unsigned c)
+    {
+        return reinterpret_cast<const ST *>(reinterpret_cast<const char *>(base + elems) + c);
+    }
+    static __device__ __forceinline__ ST *at(ST *base, int64_t elems, unsigned c)
+    {
+        return reinterpret_cast<ST *>(reinterpret_cast<char *>(base + elems) + c);
+    }
+};
+
+// Addressing for the kernels in which a wave's lanes are the channels of one time step: an access is
+// (base, lane offset, step offset), where the base is a 64-bit address that is the same for the whole wave
+// (batch element and first time step of the wave's span: scalar registers), the lane offset is the lane's
+// channel in bytes (one vector register, shared by every access of the kernel) and the step offset is the
+// time step's distance from the base in bytes (a scalar). Offsets are 32-bit: the host keeps
+// (S + 2) * time stride * element size below 4 GiB for these kernels.
+// Two forms. BUF: buffer instructions, which take exactly these three operands, so no 64-bit address is
+// formed per lane and access. Otherwise global instructions on base + offsets. Measured on the same
+// kernels in one run (cl_buffered() below holds the outcome): the forward passes run the same either way
+// (within 2 %; bf16 [64, 2048, 1001], lanes of one 16-bit channel, 265 us against 310); the backward
+// passes (five tensors, i.e. five resources of four scalar registers) are 2-10 % faster on global
+// instructions when a workgroup walks all of T (bf16 [256, 4096, 64] 142 us against 157, [16, 4096, 1024]
+// 147 against 160, fp32 [64, 2048, 1024] 453 against 463) except with one 16-bit channel per lane and 8
+// steps per wave ([64, 2048, 1001] bf16: 463 us against 541); with time split over workgroups fp32 is 3-6 %
+// faster on global instructions ([4, 16384, 1024] 261 us against 277) and 16-bit storage 30 % faster on
+// buffer instructions ([8, 4096, 512] bf16 48 us against 69).
+template <typename ST, int VEC, bool BUF> struct ClAccess;
+
+template <typename ST, int VEC, int S, bool REV, bool SPLIT /* time split over workgroups */>
+constexpr bool cl_buffered()
+{
+    if (!REV) return true;
+    if (SPLIT) return sizeof(ST) == 2;
+    return sizeof(ST) * VEC == 2 && S <= 8;
+}
+
+template <typename ST, int VEC> struct ClAccess<ST, VEC, true> {
+    using raw_t = typename Vec<ST, VEC>::raw_t;
+    static constexpr int kBytes = (int)sizeof(raw_t);
+    using Base = __amdgpu_buffer_rsrc_t;
+    static __device__ __forceinline__ Base base(const ST *p)
+    {
+        // No bounds: the offsets handed in are always inside the tensor.
+        return __builtin_amdgcn_make_buffer_rsrc(const_cast<ST *>(p), 0, -1, 0x00020000);
+    }
+    // aux 2 = non-temporal (streamed data), 0 = the caches' normal policy.
+    template <int AUX> static __device__ __forceinline__ raw_t load(Base r, unsigned lane_off, unsigned step_off)
+    {
+        if constexpr (kBytes == 16) return __builtin_amdgcn_raw_buffer_load_b128(r, lane_off, step_off, AUX);
+        else if constexpr (kBytes == 8) return __builtin_amdgcn_raw_buffer_load_b64(r, lane_off, step_off, AUX);
+        else if constexpr (kBytes == 4) return __builtin_amdgcn_raw_buffer_load_b32(r, lane_off, step_off, AUX);
+        else return __builtin_amdgcn_raw_buffer_load_b16(r, lane_off, step_off, AUX);
+    }
+    static __device__ __forceinline__ void store(raw_t v, Base r, unsigned lane_off, unsigned step_off)
+    {
+        if constexpr (kBytes == 16) __builtin_amdgcn_raw_buffer_store_b128(v, r, lane_off, step_off, 2);
+        else if constexpr (kBytes == 8) __builtin_amdgcn_raw_buffer_store_b64(v, r, lane_off, step_off, 2);
+        else if constexpr (kBytes == 4) __builtin_amdgcn_raw_buffer_store_b32(v, r, lane_off, step_off, 2);
+        else __builtin_amdgcn_raw_buffer_store_b16(v, r, lane_off, step_off, 2);
+    }
+};
+
+template <typename ST, int VEC> struct ClAccess<ST, VEC, false> {
+    using raw_t = typename Vec<ST, VEC>::raw_t;
+    typedef raw_t raw_elem_aligned_t __attribute__((aligned(sizeof(ST))));
+    using Base = char *;
+    static __device__ __forceinline__ Base base(const ST *p) { return reinterpret_cast<char *>(const_cast<ST *>(p)); }
+    template <int AUX> static __device__ __forceinline__ raw_t load(Base r, unsigned lane_off, unsigned step_off)
+    {
+        const raw_elem_aligned_t *q = reinterpret_cast<const raw_elem_aligned_t *>(r + step_off + lane_off);
+        if (AUX == 2) return __builtin_nontemporal_load(q);
+        return *q;
+    }
+    static __device__ __forceinline__ void store(raw_t v, Base r, unsigned lane_off, unsigned step_off)
+    {
+        __builtin_nontemporal_store(v, reinterpret_cast<raw_elem_aligned_t *>(r + step_off + lane_off));
+    }
 };
 
 // One wave's S consecutive time steps of a tile, for the 64*VEC channels of the workgroup.
@@ -62,44 +147,68 @@ template <typename ST> struct ClLane {
 //   apply       replays the steps from the scan value entering them and stores the results
 // With APPLY = false only load_fold is used, and its loads are left cacheable (the data is
 // read again later).
-template <typename ST, int VEC, int S, bool REV, bool APPLY, typename CT>
+template <typename ST, int VEC, int S, bool REV, bool APPLY, typename CT, bool SPLIT = false>
 struct ClSteps {
     using V = Vec<ST, VEC>;
     using raw_t = typename V::raw_t;
+    using BV = ClAccess<ST, VEC, cl_buffered<ST, VEC, S, REV, SPLIT>()>;
+    using Base = typename BV::Base;
 
     CT g[S][VEC], v[S][VEC];
     raw_t rh[(REV && APPLY) ? S : 1];
-    bool ok[S], h_ok[S];
-    int tau0;  // scan position of the first step
+    int tau0;   // scan position of the first step
+    int limit;  // scan positions from here on do not exist
+    int tb;     // time step the resources' bases point at: no access of this wave lies before it
 
-    __device__ __forceinline__ void load_fold(const ClLane<ST> &ln, int T, int first_step, int limit,
-                                              CT (&A)[VEC], CT (&B)[VEC])
+    // Byte distance of time step t from the base, for a tensor with `stride` elements per step.
+    __device__ __forceinline__ unsigned step_off(int t, int stride) const
+    {
+        return (unsigned)(t - tb) * (unsigned)stride * (unsigned)sizeof(ST);
+    }
+
+    // Whether a step exists, and whether its shifted operands do, is the same for every lane of the
+    // wave (tau0 and limit are wave-uniform): scalar conditions, scalar offsets. A lane without
+    // channels (C no multiple of the workgroup's channels) computes on channel 0's data like any
+    // other lane and only its stores are masked, so no per-lane mask is kept per step.
+    raw_t ra[S], rx[S];  // what issue() brought; dead once fold() has run
+
+    // Issues every load of the wave's S steps; nothing waits for them here.
+    __device__ __forceinline__ void issue(const ClLane<ST> &ln, int T, int first_step, int limit_)
     {
         tau0 = first_step;
-        // Every load is issued unconditionally, masked lanes from offset 0 of their own column (always
-        // valid), and masked by a select afterwards: no branch separates the loads, so all of a wave's
-        // S x streams loads are in flight before the first one is waited for.
-        raw_t ra[S], rx[S];
-        bool a_ok[S];
+        limit = limit_;
+        // Forwards the wave touches times tau0 ... tau0+S-1; backwards T-1-tau for the same tau, plus
+        // a[t+1] and h[t-1]: nothing before T-1-(tau0+S-1)-1. Clamped into the tensor.
+        const int lowest = REV ? T - 1 - (tau0 + S - 1) - 1 : tau0;
+        tb = lowest < 0 ? 0 : (lowest > T - 1 ? T - 1 : lowest);
+        const Base res_a = BV::base(ln.a + (int64_t)tb * ln.pa), res_x = BV::base(ln.x + (int64_t)tb * ln.px);
+        const Base res_h = BV::base(ln.h + (int64_t)tb * ln.ph);
+        // Every load is issued unconditionally (a step that does not exist reads the base): no
+        // branch separates the loads, so all of a wave's S x streams loads are in flight before the
+        // first one is waited for.
 #pragma unroll
         for (int s = 0; s < S; s++) {
             const int tau = tau0 + s;
             const int t = REV ? T - 1 - tau : tau;
-            ok[s] = ln.c_ok && tau < limit;
+            const bool in = tau < limit;
             // The gate of step t is a[t] forwards and a[t+1] backwards (0 past the end); h[-1] = 0.
-            a_ok[s] = ok[s] && (!REV || t + 1 < T);
-            h_ok[s] = ok[s] && t > 0;
-            const int64_t off_x = ok[s] ? (int64_t)t * ln.px : 0;
-            const int64_t off_a = a_ok[s] ? (int64_t)(REV ? t + 1 : t) * ln.pa : 0;
+            const bool a_in = in && (!REV || t + 1 < T), h_in = in && t > 0;
+            const unsigned off_x = in ? step_off(t, ln.px) : 0u;
+            const unsigned off_a = a_in ? step_off(REV ? t + 1 : t, ln.pa) : 0u;
             if (APPLY) {
-                ra[s] = V::load(ln.a + off_a);
-                rx[s] = V::load(ln.x + off_x);
-                if (REV) rh[s] = V::load(ln.h + (h_ok[s] ? (int64_t)(t - 1) * ln.ph : 0));
+                ra[s] = BV::template load<2>(res_a, ln.c, off_a);
+                rx[s] = BV::template load<2>(res_x, ln.c, off_x);
+                if (REV) rh[s] = BV::template load<2>(res_h, ln.c, h_in ? step_off(t - 1, ln.ph) : 0u);
             } else {
-                ra[s] = V::load_cached(ln.a + off_a);
-                rx[s] = V::load_cached(ln.x + off_x);
+                ra[s] = BV::template load<0>(res_a, ln.c, off_a);
+                rx[s] = BV::template load<0>(res_x, ln.c, off_x);
             }
         }
+    }
+
+    // Folds the issued steps to one affine pair per channel (and keeps gate and value per step for apply()).
+    __device__ __forceinline__ void fold(int T, CT (&A)[VEC], CT (&B)[VEC])
+    {
 #pragma unroll
         for (int k = 0; k < VEC; k++) {
             A[k] = CT(1);
@@ -107,25 +216,37 @@ struct ClSteps {
         }
 #pragma unroll
         for (int s = 0; s < S; s++) {
+            const int tau = tau0 + s;
+            const int t = REV ? T - 1 - tau : tau;
+            const bool in = tau < limit, a_in = in && (!REV || t + 1 < T);
             CT fa[VEC], fx[VEC];
             V::unpack(ra[s], fa);
             V::unpack(rx[s], fx);
 #pragma unroll
             for (int k = 0; k < VEC; k++) {
-                g[s][k] = ok[s] ? (a_ok[s] ? fa[k] : CT(0)) : CT(1);
-                v[s][k] = ok[s] ? fx[k] : CT(0);
+                g[s][k] = in ? (a_in ? fa[k] : CT(0)) : CT(1);
+                v[s][k] = in ? fx[k] : CT(0);
                 B[k] = fma_(g[s][k], B[k], v[s][k]);
                 A[k] = A[k] * g[s][k];
             }
         }
     }
 
+    __device__ __forceinline__ void load_fold(const ClLane<ST> &ln, int T, int first_step, int limit_,
+                                              CT (&A)[VEC], CT (&B)[VEC])
+    {
+        issue(ln, T, first_step, limit_);
+        fold(T, A, B);
+    }
+
     __device__ __forceinline__ void apply(const ClLane<ST> &ln, int T, CT (&mine)[VEC])
     {
+        const Base res_y0 = BV::base(ln.y0 + (int64_t)tb * ln.py0), res_y1 = BV::base(ln.y1 + (int64_t)tb * ln.py1);
 #pragma unroll
         for (int s = 0; s < S; s++) {
             const int tau = tau0 + s;
             const int t = REV ? T - 1 - tau : tau;
+            const bool in = tau < limit, h_in = in && t > 0;
             CT out[VEC];
 #pragma unroll
             for (int k = 0; k < VEC; k++) {
@@ -133,15 +254,15 @@ struct ClSteps {
                 out[k] = mine[k];
             }
             if (!REV) {
-                if (ok[s]) V::store(ln.y0 + (int64_t)t * ln.py0, V::pack(out));
+                if (in && ln.c_ok) BV::store(V::pack(out), res_y0, ln.c, step_off(t, ln.py0));
             } else {
                 CT fh[VEC], ga[VEC];
                 V::unpack(rh[s], fh);
 #pragma unroll
-                for (int k = 0; k < VEC; k++) ga[k] = out[k] * (h_ok[s] ? fh[k] : CT(0));
-                if (ok[s]) {
-                    V::store(ln.y0 + (int64_t)t * ln.py0, V::pack(out));
-                    V::store(ln.y1 + (int64_t)t * ln.py1, V::pack(ga));
+                for (int k = 0; k < VEC; k++) ga[k] = out[k] * (h_in ? fh[k] : CT(0));
+                if (in && ln.c_ok) {
+                    BV::store(V::pack(out), res_y0, ln.c, step_off(t, ln.py0));
+                    BV::store(V::pack(ga), res_y1, ln.c, step_off(t, ln.py1));
                 }
             }
         }
@@ -207,12 +328,12 @@ __device__ __forceinline__ ClLane<ST> cl_lane(const ClArgs &p, int64_t batch_ind
     const int64_t c0 = ((int64_t)group * kWave + lane) * VEC;  // first channel of this lane
     ClLane<ST> ln;
     ln.c_ok = c0 < p.C;
-    const int64_t c = ln.c_ok ? c0 : 0;
-    ln.a = static_cast<const ST *>(p.a) + batch_index * p.sB[0] + c;
-    ln.x = static_cast<const ST *>(p.x) + batch_index * p.sB[1] + c;
-    ln.h = static_cast<const ST *>(p.h) + batch_index * p.sB[2] + c;
-    ln.y0 = static_cast<ST *>(p.y0) + batch_index * p.sB[3] + c;
-    ln.y1 = static_cast<ST *>(p.y1) + batch_index * p.sB[4] + c;
+    ln.c = ln.c_ok ? (unsigned)(c0 * sizeof(ST)) : 0u;
+    ln.a = static_cast<const ST *>(p.a) + batch_index * p.sB[0];
+    ln.x = static_cast<const ST *>(p.x) + batch_index * p.sB[1];
+    ln.h = static_cast<const ST *>(p.h) + batch_index * p.sB[2];
+    ln.y0 = static_cast<ST *>(p.y0) + batch_index * p.sB[3];
+    ln.y1 = static_cast<ST *>(p.y1) + batch_index * p.sB[4];
     ln.pa = p.sT[0];
     ln.px = p.sT[1];
     ln.ph = p.sT[2];
@@ -230,7 +351,7 @@ __global__ __launch_bounds__(MAXT) void scan_cl_kernel(const ClArgs p)
     CT *lds = reinterpret_cast<CT *>(lds_raw);
 
     const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x / kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // wave-uniform: kept in a scalar register
     const int W = blockDim.x / kWave;
     const int groups = (p.C + kWave * VEC - 1) / (kWave * VEC);  // channel groups per batch element
     // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2. When a time step of C
@@ -311,9 +432,9 @@ __global__ __launch_bounds__(MAXT) void scan_cl_packed_kernel(const ClArgs p)
             ok[s] = ln.c_ok && tau < p.T;
             a_ok[s] = ok[s] && (!REV || t + 1 < p.T);  // backward gate a[t+1], 0 past the end
             h_ok[s] = ok[s] && t > 0;                   // h[-1] = 0
-            ra[s] = V::load(ln.a + (a_ok[s] ? (int64_t)(REV ? t + 1 : t) * ln.pa : 0));
-            rx[s] = V::load(ln.x + (ok[s] ? (int64_t)t * ln.px : 0));
-            if (REV) rh[s] = V::load(ln.h + (h_ok[s] ? (int64_t)(t - 1) * ln.ph : 0));
+            ra[s] = V::load(ln.at(ln.a, a_ok[s] ? (int64_t)(REV ? t + 1 : t) * ln.pa : 0, ln.c));
+            rx[s] = V::load(ln.at(ln.x, ok[s] ? (int64_t)t * ln.px : 0, ln.c));
+            if (REV) rh[s] = V::load(ln.at(ln.h, h_ok[s] ? (int64_t)(t - 1) * ln.ph : 0, ln.c));
         }
         // PA/PB: the pair of everything in this wave's span up to and including the lane's step of
         // instruction s; (RA, RB): instructions 0..s-1 composed (the same in every lane of a channel).
@@ -414,15 +535,15 @@ __global__ __launch_bounds__(MAXT) void scan_cl_packed_kernel(const ClArgs p)
 #pragma unroll
             for (int k = 0; k < VEC; k++) out[k] = fma_(PA[s][k], mine[k], PB[s][k]);
             if (!REV) {
-                if (ok[s]) V::store(ln.y0 + (int64_t)tt[s] * ln.py0, V::pack(out));
+                if (ok[s]) V::store(ln.at(ln.y0, (int64_t)tt[s] * ln.py0, ln.c), V::pack(out));
             } else {
                 CT fh[VEC], ga[VEC];
                 V::unpack(rh[s], fh);
 #pragma unroll
                 for (int k = 0; k < VEC; k++) ga[k] = out[k] * (h_ok[s] ? fh[k] : CT(0));
                 if (ok[s]) {
-                    V::store(ln.y0 + (int64_t)tt[s] * ln.py0, V::pack(out));
-                    V::store(ln.y1 + (int64_t)tt[s] * ln.py1, V::pack(ga));
+                    V::store(ln.at(ln.y0, (int64_t)tt[s] * ln.py0, ln.c), V::pack(out));
+                    V::store(ln.at(ln.y1, (int64_t)tt[s] * ln.py1, ln.c), V::pack(ga));
                 }
             }
         }
@@ -448,7 +569,7 @@ __global__ __launch_bounds__(MAXT) void scan_cl_packed_kernel(const ClArgs p)
 // r * kCounterStride, word 1 raised on a timed-out wait; then per (row-group,
 // tile) its pair, A then B, each [VEC][64] published values; then per
 // (row-group, super-tile) SA, SB, SI likewise (4 slots, one unused).
-// LDS: 7 arrays of [W][VEC][64] values (wave pairs A, B; tile aggregates A, B;
+// LDS: [W][7][VEC][64] values (per wave slot: wave pairs A, B; tile aggregates A, B;
 // super-tile SI, SA, SB).
 // ---------------------------------------------------------------------------
 template <typename CT, int VEC>
@@ -480,39 +601,40 @@ __global__ __launch_bounds__(MAXT) void scan_cl_lookback_kernel(const ClArgs p)
     __shared__ int lds_flags[2][kMaxWaves];
 
     const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x / kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // wave-uniform: kept in a scalar register
     const int W = blockDim.x / kWave;
     const int groups = (p.C + kWave * VEC - 1) / (kWave * VEC);
     const int64_t rowgroups = p.batch * groups;
+    const int tpr = p.segments;              // tiles per row-group
+    const int spr = (tpr + W - 1) / W;       // super-tiles per row-group
+    // LDS: per wave slot w, seven [VEC][64] arrays one after the other, so that an access is the slot's
+    // base plus the lane (one register) and a constant.
+    enum { exA, exB,   // pairs of this tile's waves
+           tA, tB,     // aggregates of tiles 0..j-1 of the super-tile
+           sI, sA, sB  // super-tiles m-1, m-2, ...
+    };
+    constexpr int kVals = VEC * kWave * D::W;  // words of one [VEC][64] array of published values
+#define AT(arr, w, k) lds[((w) * 7 + (arr)) * (VEC * kWave) + (k) * kWave + lane]
+
     // Row-groups of a workgroup's XCD: with p.xcd_order (time steps that are not whole 128-byte lines) a
     // contiguous run of them, so that channel groups that share a line meet in one L2 (as in scan_cl_kernel;
     // exact when the number of row-groups is a multiple of 8, where a row-group keeps its XCD over all tiles).
     const int64_t rg0 = blockIdx.x % rowgroups;
     const int64_t rg = (p.xcd_order && rowgroups % 8 == 0) ? xcd_contiguous((int)rg0, (int)rowgroups) : rg0;
-
     if (threadIdx.x == 0)
         lds_ticket = __hip_atomic_fetch_add(reinterpret_cast<unsigned *>(p.ws + rg * kCounterStride), 1u,
                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
-    const int tile = (int)__builtin_amdgcn_readfirstlane(lds_ticket);
+    const int tile = (int)__builtin_amdgcn_readfirstlane((int)lds_ticket);
     const ClLane<ST> ln = cl_lane<ST, VEC>(p, rg / groups, (int)(rg % groups), lane);
-
-    const int tpr = p.segments;              // tiles per row-group
-    const int spr = (tpr + W - 1) / W;       // super-tiles per row-group
-    const int j = tile % W, m = tile / W;
-    const int plane = W * VEC * kWave;
-    CT *exA = lds, *exB = lds + plane;                         // pairs of this tile's waves
-    CT *tA = lds + 2 * plane, *tB = lds + 3 * plane;           // aggregates of tiles 0..j-1 of the super-tile
-    CT *sI = lds + 4 * plane, *sA = lds + 5 * plane, *sB = lds + 6 * plane;  // super-tiles m-1, m-2, ...
-    constexpr int kVals = VEC * kWave * D::W;  // words of one [VEC][64] array of published values
     uint64_t *tiles = p.ws + rowgroups * kCounterStride + rg * (int64_t)tpr * 2 * kVals;
     uint64_t *supers = p.ws + rowgroups * kCounterStride + rowgroups * (int64_t)tpr * 2 * kVals +
                        rg * (int64_t)spr * 4 * kVals;
-#define AT(arr, w, k) arr[((w) * VEC + (k)) * kWave + lane]
+    const int j = tile % W, m = tile / W;
 
-    ClSteps<ST, VEC, S, REV, true, CT> steps;
+    ClSteps<ST, VEC, S, REV, true, CT, true> cur;
     CT A[VEC], B[VEC];
-    steps.load_fold(ln, p.T, tile * W * S + wave * S, p.T, A, B);
+    cur.load_fold(ln, p.T, tile * W * S + wave * S, p.T, A, B);
 #pragma unroll
     for (int k = 0; k < VEC; k++) {
         AT(exA, wave, k) = A[k];
@@ -688,7 +810,7 @@ __global__ __launch_bounds__(MAXT) void scan_cl_lookback_kernel(const ClArgs p)
 #pragma unroll
         for (int k = 0; k < VEC; k++) carry[k] = fma_(AT(exA, q, k), carry[k], AT(exB, q, k));
     }
-    steps.apply(ln, p.T, carry);
+    cur.apply(ln, p.T, carry);
 #undef AT
 }
 

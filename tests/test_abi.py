@@ -116,6 +116,10 @@ def test_strided_calls_check_their_arguments():
     assert L.scanscam_scan_fwd_cl_strided(fake, fake, fake, big, None, None, 2, 8, 64, 0, None, 0, None, None) == E_INVAL
     assert L.scanscam_scan_bwd_cl_strided(fake, fake, fake, fake, fake, neg, None, None, None, None, 2, 8, 64, 0, None,
                                           0, None, None) == E_INVAL
+    # ... and a time step stays below 4 GiB / 18 (a wave addresses its steps with 32-bit offsets)
+    wide = ctypes.byref(S(0, 60_000_000))
+    assert L.scanscam_scan_fwd_cl_strided(fake, fake, fake, wide, None, None, 1, 8, 64, 0, None, 0, None, None) == E_INVAL
+    assert L.scanscam_scan_fwd_cl(fake, fake, fake, 1, 8, 60_000_000, 0, None, 0, None, None) == E_INVAL
     # empty problems succeed without touching anything
     assert L.scanscam_scan_fwd_strided(None, None, None, None, None, None, 0, 5, 64, 0, None, 0, None, None) == E_OK
     assert L.scanscam_scan_fwd_cl_strided(None, None, None, None, None, None, 3, 0, 64, 0, None, 0, None, None) == E_OK
