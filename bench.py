@@ -662,7 +662,7 @@ def main():
     rows, T = first.a.shape
     plan_f = hip.resolve_plan(rows, T, a.dtype, hip.FORWARD)
     family = {hip.MODE_SMALL: "scan_small_kernel", hip.MODE_ROW: "scan_row_kernel",
-              hip.MODE_LOOKBACK: "scan_lookback_kernel"}[plan_f.mode]
+              hip.MODE_LOOKBACK: "scan_lookback_kernel", hip.MODE_FLAT: "scan_flat_kernel"}[plan_f.mode]
     storage = {"float32": "float", "bfloat16": "__bf16", "float16": "_Float16"}[str(a.dtype).replace("torch.", "")]
     kernel = f"{family}<{storage}, {plan_f.vec}, {plan_f.unroll}, REV=%s>"
     traffic, traffic_source = measured_traffic() if args.workload == "2" else ({"fwd": None, "bwd": None}, None)

@@ -57,7 +57,9 @@ enum {
     SCANSCAM_MODE_AUTO = 0,
     SCANSCAM_MODE_SMALL = 1,   /* T <= 64*vec: several rows per wave, no carries */
     SCANSCAM_MODE_ROW = 2,     /* a workgroup (or part of one) walks a whole row */
-    SCANSCAM_MODE_LOOKBACK = 3 /* rows cut into tiles over workgroups, decoupled look-back carries */
+    SCANSCAM_MODE_LOOKBACK = 3, /* rows cut into tiles over workgroups, decoupled look-back carries */
+    SCANSCAM_MODE_FLAT = 4      /* dense tensors, 16/sizeof(storage) <= T <= 64 * that: all rows scanned as one
+                                   stream of aligned vectors with a reset at every row start (unroll 2 or 4) */
 };
 
 /*

@@ -17,6 +17,7 @@ namespace {
 using scanscam::kCounterStride;
 using scanscam::kMaxCounters;
 using scanscam::kSuper;
+using scanscam::kModeFlat;
 using scanscam::kModeLookback;
 using scanscam::kModeRow;
 using scanscam::kModeSmall;
@@ -119,8 +120,30 @@ bool prefer_lookback_for_many_rows(int64_t rows, int nch, bool rev, int esize)
 // Turns (shape, alignment, direction, optional user plan) into a launch. `aligned128` says whether every
 // row of every tensor starts on a 128-byte line border; `aligned16` says
 // whether every tensor base is 16-byte aligned.
+int gcd_int(int a, int b) { return b == 0 ? a : gcd_int(b, a % b); }
+
+// Rows the flat kernel can take of `rows` rows of length T: the largest count whose elements are a whole
+// number of 16-byte vectors (the few rows left over go to the other kernels).
+int64_t flat_rows(int64_t rows, int64_t T, int full) { return rows - rows % (full / gcd_int((int)(T % full), full)); }
+
+// Short rows that start at any element, or whose vectors do not fill the SMALL kernel's power-of-two group of
+// lanes: the flat kernel, where the tensors allow it (dense, 16-byte aligned bases). Measured at 32 M and 64 M
+// elements, forward / backward, % of peak: fp32 flat 80-83 / 76-79 at every T from 4 to 256, SMALL the same
+// where T / 4 is a power of two and 64-77 / 63-77 elsewhere (T = 70: 64 / 64, 132: 70 / 67, 36: 74 / 72); float64
+// alike. 16-bit storage: flat 72-73 / 66-68 at every T (the three-component scan costs its instruction-bound
+// backward pass 8-10 points), SMALL 70-77 / 68-78 on vector-aligned rows that fill at least 0.6 of their group,
+// 57-68 / 55-67 otherwise (T = 100, 136, 264, 500).
+bool prefer_flat(int64_t T, int full, int esize)
+{
+    if (T % full != 0) return true;
+    const int nv = (int)(T / full), group = pow2_ceil(nv);
+    if (esize == 2) return nv * 10 < group * 6;
+    return nv != group;
+}
+
+// `flat_ok`: the tensors are dense [rows, T] arrays on 16-byte aligned bases (what the flat kernel needs).
 int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool aligned16, bool aligned128, bool rev,
-            Resolved *out)
+            Resolved *out, bool flat_ok = false)
 {
     const int esize = elem_size(dtype);
     if (esize == 0) return SCANSCAM_EDTYPE;
@@ -131,6 +154,25 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
 
     Launch &l = out->l;
     l = Launch{0, 0, 0, 0, 1, 64, 0, false, 1};
+    const bool flat_possible = flat_ok && T >= full && T <= (int64_t)kWave * full && flat_rows(rows, T, full) > 0;
+    if (u.mode == kModeFlat || (u.mode == SCANSCAM_MODE_AUTO && flat_possible && !u.vec && prefer_flat(T, full, esize))) {
+        if (!flat_possible) return SCANSCAM_EPLAN;
+        if (u.vec && u.vec != full) return SCANSCAM_EPLAN;
+        l.mode = kModeFlat;
+        l.vec = full;
+        // 4 waves x 4 chunks; 16-bit storage (twice the registers per chunk) 8 waves x 2 chunks.
+        l.unroll = u.unroll ? u.unroll : (esize == 2 ? 2 : 4);
+        l.waves = u.waves ? u.waves : (esize == 2 ? 8 : 4);
+        if ((l.unroll != 2 && l.unroll != 4) || l.waves < 1 || l.waves > scanscam::kMaxWaves) return SCANSCAM_EPLAN;
+        out->nch = 1;
+        out->tiles_per_row = 0;
+        out->counters = 1;
+        out->row_major = 0;
+        out->line_shift = 0;
+        out->super_base = 0;
+        out->ws_bytes = 0;
+        return SCANSCAM_OK;
+    }
     // The full 16-byte vector needs rows that start on 16-byte borders -- or the element-aligned ("ragged")
     // variants of the kernels: ROW and LOOKBACK for rows of at least nine tenths of a chunk (on shorter rows
     // most of their lanes would idle), SMALL for rows of 4 vectors to one chunk (shorter ones lose nothing
@@ -311,7 +353,7 @@ const scanscam_strides *const kDense[5] = {nullptr, nullptr, nullptr, nullptr, n
 int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y1,
         const scanscam_strides *const st[5], int64_t n0, int64_t n1, int64_t T, int dtype, void *workspace,
         size_t workspace_bytes, void *stream, const scanscam_plan *plan, void *start_event = nullptr,
-        void *stop_event = nullptr, bool use_scratch = false)
+        void *stop_event = nullptr, bool use_scratch = false, bool allow_flat = true)
 {
     const int esize = elem_size(dtype);
     if (esize == 0) return SCANSCAM_EDTYPE;
@@ -370,9 +412,44 @@ int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y
         aligned128 = aligned128 && aligned_to(ptrs[k], 128) && s0[k] % line == 0 && s1[k] % line == 0;
     }
 
+    // The flat kernel takes dense [rows, T] tensors on 16-byte aligned bases (rows of any length).
+    bool flat_ok = allow_flat && n0 == 1;
+    for (int k = 0; k < 5; k++) flat_ok = flat_ok && (!used[k] || (aligned_to(ptrs[k], 16) && (n1 == 1 || s1[k] == T)));
+    // One pair of events cannot bracket the flat launch and the launch for the rows it leaves over.
+    if ((start_event || stop_event) && flat_rows(rows, T, full) != rows) flat_ok = false;
+
     Resolved r;
-    const int rc = resolve(plan, rows, T, dtype, aligned16, aligned128, rev, &r);
+    const int rc = resolve(plan, rows, T, dtype, aligned16, aligned128, rev, &r, flat_ok);
     if (rc != SCANSCAM_OK) return rc;
+
+    if (r.l.mode == kModeFlat) {
+        const int64_t taken = flat_rows(rows, T, full);
+        scanscam::FlatArgs fa;
+        fa.a = a;
+        fa.x = x;
+        fa.h = h;
+        fa.y0 = y0;
+        fa.y1 = y1;
+        fa.N = taken * T;
+        fa.T = (int32_t)T;
+        hipStream_t fs = static_cast<hipStream_t>(stream);
+        hipEvent_t e0 = static_cast<hipEvent_t>(start_event), e1 = static_cast<hipEvent_t>(stop_event);
+        hipError_t e = hipErrorInvalidValue;
+        switch (dtype) {
+        case SCANSCAM_F32: e = scanscam::launch_scan_flat<float>(fa, r.l.unroll, r.l.waves, rev, fs, e0, e1); break;
+        case SCANSCAM_BF16: e = scanscam::launch_scan_flat<__bf16>(fa, r.l.unroll, r.l.waves, rev, fs, e0, e1); break;
+        case SCANSCAM_F16: e = scanscam::launch_scan_flat<_Float16>(fa, r.l.unroll, r.l.waves, rev, fs, e0, e1); break;
+        case SCANSCAM_F64: e = scanscam::launch_scan_flat<double>(fa, r.l.unroll, r.l.waves, rev, fs, e0, e1); break;
+        }
+        if (e != hipSuccess) return SCANSCAM_ELAUNCH;
+        if (taken == rows) return SCANSCAM_OK;
+        // The few rows left over (fewer than a vector has elements): the other kernels, on the tail of every tensor.
+        const int64_t off = taken * T * esize;
+        auto tail = [&](const void *q) { return q ? static_cast<const void *>(static_cast<const char *>(q) + off) : nullptr; };
+        return run(rev, tail(a), tail(x), tail(h), const_cast<void *>(tail(y0)), const_cast<void *>(tail(y1)), kDense, 1,
+                   rows - taken, T, dtype, workspace, workspace_bytes, stream, nullptr, nullptr, nullptr, use_scratch,
+                   /*allow_flat=*/false);
+    }
 
     ScanArgs args;
     args.a = a;
@@ -834,7 +911,7 @@ int scanscam_resolve_plan(int64_t rows, int64_t T, int dtype, int direction, con
     // Dense tensors on allocation borders: rows start on line borders exactly when a row is whole lines.
     const int esize = elem_size(dtype);
     const bool lines = esize != 0 && (T * esize) % 128 == 0;
-    const int rc = resolve(plan, rows, T, dtype, true, lines, direction == SCANSCAM_BACKWARD, &r);
+    const int rc = resolve(plan, rows, T, dtype, true, lines, direction == SCANSCAM_BACKWARD, &r, /*flat_ok=*/true);
     if (rc != SCANSCAM_OK) return rc;
     out->mode = r.l.mode;
     out->vec = r.l.vec;

@@ -4,4 +4,5 @@
 namespace scanscam {
 SCANSCAM_DEFINE_LAUNCH(__bf16)
 SCANSCAM_DEFINE_CL_LAUNCH(__bf16)
+SCANSCAM_DEFINE_FLAT_LAUNCH(__bf16)
 }  // namespace scanscam

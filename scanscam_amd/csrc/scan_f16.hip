@@ -4,4 +4,5 @@
 namespace scanscam {
 SCANSCAM_DEFINE_LAUNCH(_Float16)
 SCANSCAM_DEFINE_CL_LAUNCH(_Float16)
+SCANSCAM_DEFINE_FLAT_LAUNCH(_Float16)
 }  // namespace scanscam

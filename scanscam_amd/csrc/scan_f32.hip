@@ -4,4 +4,5 @@
 namespace scanscam {
 SCANSCAM_DEFINE_LAUNCH(float)
 SCANSCAM_DEFINE_CL_LAUNCH(float)
+SCANSCAM_DEFINE_FLAT_LAUNCH(float)
 }  // namespace scanscam

@@ -4,4 +4,5 @@
 namespace scanscam {
 SCANSCAM_DEFINE_LAUNCH(double)
 SCANSCAM_DEFINE_CL_LAUNCH(double)
+SCANSCAM_DEFINE_FLAT_LAUNCH(double)
 }  // namespace scanscam

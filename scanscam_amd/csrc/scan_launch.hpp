@@ -4,11 +4,12 @@
 #include <hip/hip_ext.h>
 
 #include "scan_cl_kernels.hpp"
+#include "scan_flat_kernels.hpp"
 #include "scan_kernels.hpp"
 
 namespace scanscam {
 
-enum Mode { kModeSmall = 1, kModeRow = 2, kModeLookback = 3 };
+enum Mode { kModeSmall = 1, kModeRow = 2, kModeLookback = 3, kModeFlat = 4 };
 
 // A fully resolved launch: which kernel, with which shape.
 struct Launch {
@@ -83,6 +84,34 @@ hipError_t launch_scan(const ScanArgs &args, const Launch &l, bool rev, hipStrea
         SCANSCAM_LAUNCH_CASE(ST, 1, 1)                                                               \
         SCANSCAM_LAUNCH_CASE(ST, 1, 4)                                                               \
         return hipErrorInvalidValue;                                                                 \
+    }
+
+// The flat kernel (dense short rows scanned as one stream): `unroll` chunks per wave (2 or 4), `waves` waves
+// per workgroup, full vector only. Returns hipErrorInvalidValue for an unroll that is not instantiated.
+template <typename ST>
+hipError_t launch_scan_flat(const FlatArgs &args, int unroll, int waves, bool rev, hipStream_t stream, hipEvent_t start,
+                            hipEvent_t stop);
+
+#define SCANSCAM_FLAT_CASE(ST, U)                                                                     \
+    if (unroll == (U)) {                                                                              \
+        if (rev) hipExtLaunchKernelGGL((scan_flat_kernel<ST, FULL, U, true, 1024>), grid, block, 0, stream, start, stop, 0, args);  \
+        else     hipExtLaunchKernelGGL((scan_flat_kernel<ST, FULL, U, false, 1024>), grid, block, 0, stream, start, stop, 0, args); \
+        return hipGetLastError();                                                                     \
+    }
+
+#define SCANSCAM_DEFINE_FLAT_LAUNCH(ST)                                                               \
+    template <>                                                                                       \
+    hipError_t launch_scan_flat<ST>(const FlatArgs &args, int unroll, int waves, bool rev, hipStream_t stream, \
+                                    hipEvent_t start, hipEvent_t stop)                                \
+    {                                                                                                 \
+        constexpr int FULL = 16 / (int)sizeof(ST);                                                    \
+        const int64_t per_wg = (int64_t)waves * unroll * kWave * FULL;                                \
+        /* backwards the kernel shifts its positions by up to one chunk, to sit on line borders */   \
+        const int64_t positions = args.N + (rev ? kWave * FULL - 1 : 0);                              \
+        const dim3 grid((unsigned)((positions + per_wg - 1) / per_wg)), block((unsigned)(waves * kWave)); \
+        SCANSCAM_FLAT_CASE(ST, 2)                                                                     \
+        SCANSCAM_FLAT_CASE(ST, 4)                                                                     \
+        return hipErrorInvalidValue;                                                                  \
     }
 
 // Channels-last launches. `steps` = time steps per wave per tile (S).

@@ -27,7 +27,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # SCANSCAM_HIP_LIB points at another build of the same ABI (tuning builds).
 LIB_PATH = os.environ.get("SCANSCAM_HIP_LIB") or os.path.join(_HERE, "libscanscam_hip.so")
 
-MODE_AUTO, MODE_SMALL, MODE_ROW, MODE_LOOKBACK = 0, 1, 2, 3
+MODE_AUTO, MODE_SMALL, MODE_ROW, MODE_LOOKBACK, MODE_FLAT = 0, 1, 2, 3, 4
 FORWARD, BACKWARD = 0, 1
 ABI_VERSION = 2
 

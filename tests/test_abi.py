@@ -142,7 +142,13 @@ def test_empty_inputs_are_a_successful_noop():
         (16384, 2048, torch.float16, hip.MODE_ROW, 8),
         (131072, 64, torch.float32, hip.MODE_SMALL, 4),     # many short rows
         (32, 1025, torch.float32, hip.MODE_ROW, 4),         # odd length: element-aligned 16-byte vectors
-        (32, 5, torch.float32, hip.MODE_SMALL, 1),
+        (32, 5, torch.float32, hip.MODE_FLAT, 4),           # short rows of any length, dense: one flat stream
+        (32, 70, torch.float32, hip.MODE_FLAT, 4),
+        (32, 48, torch.float32, hip.MODE_FLAT, 4),          # 12 vectors: no power-of-two group of lanes
+        (32, 3, torch.float32, hip.MODE_SMALL, 1),          # shorter than a vector
+        (32, 100, torch.bfloat16, hip.MODE_FLAT, 8),
+        (32, 104, torch.bfloat16, hip.MODE_SMALL, 8),       # 16-bit storage keeps groups that are at least 0.6 full
+        (3, 5, torch.float32, hip.MODE_SMALL, 1),           # too few rows for a whole number of vectors
     ],
 )
 def test_automatic_plan_per_regime(rows, T, dtype, mode, vec):
@@ -180,7 +186,7 @@ def test_every_automatic_plan_is_a_valid_plan():
                         plan, out = hip.Plan(vec=vec), hip.Plan()
                         rc = L.scanscam_resolve_plan(rows, T, code, direction, ctypes.byref(plan), ctypes.byref(out))
                         assert rc == 0, (dtype, rows, T, direction, vec, hip.strerror(rc))
-                        assert 1 <= out.waves <= 16 and out.unroll in (1, 2, 4, 8) and out.mode in (1, 2, 3)
+                        assert 1 <= out.waves <= 16 and out.unroll in (1, 2, 4, 8) and out.mode in (1, 2, 3, 4)
                         if out.mode == 2:
                             assert out.waves_per_row >= 1 and out.waves % out.waves_per_row == 0
                         checked += 1
