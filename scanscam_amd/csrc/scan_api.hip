@@ -63,7 +63,7 @@ int pow2_ceil(int64_t v)
 
 bool unroll_ok(int vec, int full, int unroll)
 {
-    if (vec == full) return unroll == 1 || unroll == 2 || unroll == 4 || unroll == 8;
+    if (vec == full) return unroll == 1 || unroll == 2 || unroll == 3 || unroll == 4 || unroll == 8;
     return unroll == 1 || unroll == 4;
 }
 
@@ -199,7 +199,8 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
     // Rows of up to 4 chunks take one wave with 1, 2 or 4 chunks (2 or 4 when element-aligned): no shift
     // either where it would double that count and leave half the wave's slots empty (bf16 [33520, 1001], two
     // chunks: 38 / 57 us without the shift, 51 / 87 us with it in a wave of 4).
-    auto chunks_of_one_wave = [&](int64_t n) { return pow2_ceil(l.ragged && n < 2 ? 2 : n); };
+    // (Element-aligned 16-bit rows of three chunks take a wave of exactly three, below.)
+    auto chunks_of_one_wave = [&](int64_t n) { return (l.ragged && esize == 2 && n == 3) ? 3 : pow2_ceil(l.ragged && n < 2 ? 2 : n); };
     const bool same_wave_shape =
         nch_plain > 4 || (nch_lines <= 4 && chunks_of_one_wave(nch_lines) == chunks_of_one_wave(nch_plain));
     out->line_shift = (!aligned128 && !small_rows && (T > chunk || l.ragged) && same_wave_shape) ? 1 : 0;
@@ -235,7 +236,20 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
         l.waves = u.waves;
         l.wpr = u.waves_per_row;
         if (!l.unroll && !l.waves && !l.wpr) {
-            if (nch <= 4) {
+            // Element-aligned rows of 16-bit storage that take 3 or 9 chunks: waves of exactly 3 chunks instead of 4
+            // with a quarter of their slots empty. These kernels issue the most instructions per byte, and the
+            // empty slots cost them their share: bf16 [65000, 1025] 58 / 67 -> 72 / 74 % of peak, [16380, 4097]
+            // (9 chunks, 3 waves) 59-65 / 62-68 -> 73 / 73 %. fp32 and rows of whole vectors gain nothing from it
+            // (fp32 [87000, 769] 79 / 75 -> 76 / 72 %, bf16 [43000, 1536] 79 / 78 either way).
+            const bool threes = l.ragged && esize == 2 && l.vec == full;
+            if (threes && nch == 3) {
+                l.unroll = 3;
+                l.wpr = 1;
+                l.waves = 4;
+            } else if (threes && nch == 9) {
+                l.unroll = 3;
+                l.wpr = l.waves = 3;
+            } else if (nch <= 4) {
                 l.unroll = (l.vec == full) ? pow2_ceil(nch) : (nch == 1 ? 1 : 4);
                 l.wpr = 1;
                 l.waves = 4;
@@ -290,7 +304,13 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
         if (!u.waves && !u.unroll && rows > 8) {
             // As many tiles as 8-wave tiles would take, but with only the waves they need: 75 chunks are 3
             // tiles of 7 waves (84 chunk slots), not of 8 (96).
-            const int tiles = (nch + kTileChunks - 1) / kTileChunks;
+            int tiles = (nch + kTileChunks - 1) / kTileChunks;
+            // Element-aligned rows of 16-bit storage up to 96 chunks: tiles of up to 16 chunks (3-4 waves). Their
+            // waves do more arithmetic per byte (components of partial vectors moved into place, masks per
+            // element), and the smaller workgroups cover each other better: bf16 [2013, 33333] 55 / 58 -> 62 / 66 %
+            // of peak, [3947, 17001] 59 / 63 -> 65 / 68 %, [1973, 34001] 61 / 62 -> 63 / 67 %; from 190 chunks on
+            // the larger tile is 3-4 points faster, and rows of whole vectors keep it throughout.
+            if (l.ragged && esize == 2 && nch <= 96) tiles = (nch + kTileChunks / 2 - 1) / (kTileChunks / 2);
             l.waves = (nch + tiles * l.unroll - 1) / (tiles * l.unroll);
         }
         const int tile_chunks = l.waves * l.unroll;
@@ -314,8 +334,8 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
     }
 
     if (l.ragged) {
-        if (!u.unroll && l.unroll < 2) l.unroll = 2;  // instantiated for 2 and 4 chunks per wave
-        if (l.unroll != 2 && l.unroll != 4) return SCANSCAM_EPLAN;
+        if (!u.unroll && l.unroll < 2) l.unroll = 2;  // instantiated for 2, 3 and 4 chunks per wave
+        if (l.unroll != 2 && l.unroll != 3 && l.unroll != 4) return SCANSCAM_EPLAN;
     }
     if (!unroll_ok(l.vec, full, l.unroll)) return SCANSCAM_EPLAN;
     if (l.waves < 1 || l.waves > scanscam::kMaxWaves ||

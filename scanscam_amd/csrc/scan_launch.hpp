@@ -75,10 +75,12 @@ hipError_t launch_scan(const ScanArgs &args, const Launch &l, bool rev, hipStrea
         constexpr int FULL = 16 / (int)sizeof(ST);                                                   \
         const dim3 grid((unsigned)l.grid, (unsigned)l.grid_y), block((unsigned)(l.waves * kWave));   \
         SCANSCAM_RAGGED_CASE(ST, FULL, 2)                                                            \
+        SCANSCAM_RAGGED_CASE(ST, FULL, 3)                                                            \
         SCANSCAM_RAGGED_CASE(ST, FULL, 4)                                                            \
         if (l.ragged) return hipErrorInvalidValue;                                                   \
         SCANSCAM_LAUNCH_CASE(ST, FULL, 1)                                                            \
         SCANSCAM_LAUNCH_CASE(ST, FULL, 2)                                                            \
+        SCANSCAM_LAUNCH_CASE(ST, FULL, 3)                                                            \
         SCANSCAM_LAUNCH_CASE(ST, FULL, 4)                                                            \
         SCANSCAM_LAUNCH_CASE(ST, FULL, 8)                                                            \
         SCANSCAM_LAUNCH_CASE(ST, 1, 1)                                                               \

@@ -78,7 +78,7 @@ def test_argument_errors_are_reported_before_any_launch():
     assert L.scanscam_scan_fwd(fake, fake, fake, 4, 1 << 20, 0, None, 0, None) == E_WORKSPACE
     assert L.scanscam_scan_fwd(fake, fake, fake, 4, 1 << 20, 0, fake, 64, None) == E_WORKSPACE
     # Bad explicit plans.
-    for bad in (hip.Plan(mode=9), hip.Plan(vec=3), hip.Plan(mode=hip.MODE_ROW, unroll=3),
+    for bad in (hip.Plan(mode=9), hip.Plan(vec=3), hip.Plan(mode=hip.MODE_ROW, unroll=5),
                 hip.Plan(mode=hip.MODE_ROW, unroll=8, waves=8), hip.Plan(mode=hip.MODE_ROW, waves=4, waves_per_row=3),
                 hip.Plan(mode=hip.MODE_SMALL), hip.Plan(waves=17)):
         rc = L.scanscam_scan_fwd_plan(fake, fake, fake, 4, 4096, 0, None, 0, None, ctypes.byref(bad))
@@ -186,7 +186,7 @@ def test_every_automatic_plan_is_a_valid_plan():
                         plan, out = hip.Plan(vec=vec), hip.Plan()
                         rc = L.scanscam_resolve_plan(rows, T, code, direction, ctypes.byref(plan), ctypes.byref(out))
                         assert rc == 0, (dtype, rows, T, direction, vec, hip.strerror(rc))
-                        assert 1 <= out.waves <= 16 and out.unroll in (1, 2, 4, 8) and out.mode in (1, 2, 3, 4)
+                        assert 1 <= out.waves <= 16 and out.unroll in (1, 2, 3, 4, 8) and out.mode in (1, 2, 3, 4)
                         if out.mode == 2:
                             assert out.waves_per_row >= 1 and out.waves % out.waves_per_row == 0
                         checked += 1
