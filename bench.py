@@ -10,7 +10,7 @@ algorithmic bytes (32 B per element: forward reads a, b and writes h = 12 B;
 backward reads a, h, grad_h and writes grad_a, grad_b = 20 B).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-configs] [--workload N]
-                    [--channels-last BxTxC[:dtype]]
+                    [--channels-last BxTxC[:dtype]] [--launch-shapes]
 
 --workload runs another of the synthetic configurations (1, 3, 4, 4f16, 5; or `long`, `long16`) through the same timed
 region instead of configuration 2 (used for the rocprofv3 summaries under profiles/).
@@ -238,14 +238,15 @@ def kernel_statistics(sets, launches, hip, torch):
     return out
 
 
-def time_batches(sets, launches, warmup, hip, torch):
+def time_batches(sets, launches, warmup, hip, torch, plan=None):
     """Mean ms per launch of each direction over `launches` back-to-back launches.
 
     For kernels of a few microseconds, where an event pair around every launch
     would cost as much as the launch: two events bracket the whole batch, so the
     figure includes the gaps between launches.
     """
-    calls = [(hip.prepare_forward(s.a, s.b, s.h), hip.prepare_backward(s.a, s.h, s.gh, s.ga, s.gb)) for s in sets]
+    calls = [(hip.prepare_forward(s.a, s.b, s.h, plan=plan), hip.prepare_backward(s.a, s.h, s.gh, s.ga, s.gb, plan=plan))
+             for s in sets]
     out = []
     for d in (0, 1):
         for i in range(warmup):
@@ -261,7 +262,7 @@ def time_batches(sets, launches, warmup, hip, torch):
     return out[0], out[1]
 
 
-def time_graph(sets, replays, hip, torch):
+def time_graph(sets, replays, hip, torch, plan=None):
     """Mean ms per launch of each direction when the launches replay from a HIP graph.
 
     One launch per buffer set is captured (a kernel of a few microseconds is otherwise
@@ -272,8 +273,8 @@ def time_graph(sets, replays, hip, torch):
         side = torch.cuda.Stream()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.stream(side):
-            calls = [(hip.prepare_forward(s.a, s.b, s.h), hip.prepare_backward(s.a, s.h, s.gh, s.ga, s.gb))[d]
-                     for s in sets]
+            calls = [(hip.prepare_forward(s.a, s.b, s.h, plan=plan),
+                      hip.prepare_backward(s.a, s.h, s.gh, s.ga, s.gb, plan=plan))[d] for s in sets]
             calls[0]()
             side.synchronize()
             with torch.cuda.graph(graph, stream=side):
@@ -475,6 +476,40 @@ def strided_views(dev, args, hip, torch):
     return out
 
 
+def launch_shapes(args, hip, torch):
+    """--launch-shapes: configuration 1 ([1024, 1024] fp32) under every launch shape of the row kernel.
+
+    Microseconds per launch, launched one by one and replayed from a HIP graph (64 buffer sets in rotation),
+    and the same for a scan of [4, 64] elements, which is the cost of a launch with nothing to stream.
+    Prints one JSON line; its summary is kept under profiles/.
+    """
+    dev = torch.device("cuda:0")
+    a, b, gh = make_config(1, torch)
+    first = DeviceSet(a, b, gh, dev, torch)
+    sets = [first] + [first.clone(torch) for _ in range(63)]
+    out = {"workload": WORKLOADS["1"][1], "shapes": []}
+    shapes = [None] + [hip.Plan(mode=hip.MODE_ROW, vec=4, unroll=u, waves=w, waves_per_row=r) for u, w, r in
+                       ((4, 4, 1), (4, 2, 1), (4, 1, 1), (4, 8, 1), (2, 4, 2), (2, 2, 2), (2, 8, 2), (1, 4, 4), (1, 8, 4),
+                        (1, 16, 4), (2, 16, 2), (1, 2, 2), (3, 4, 1))]
+    for plan in shapes:
+        f_ms, b_ms = time_batches(sets, 256, 64, hip, torch, plan=plan)
+        gf_ms, gb_ms = time_graph(sets, 20, hip, torch, plan=plan)
+        out["shapes"].append({"plan": repr(plan) if plan is not None else "automatic: " + repr(hip.resolve_plan(1024, 1024, a.dtype, hip.FORWARD)),
+                              "fwd_us": round(f_ms * 1e3, 2), "fwd_graph_us": round(gf_ms * 1e3, 2),
+                              "bwd_us": round(b_ms * 1e3, 2), "bwd_graph_us": round(gb_ms * 1e3, 2)})
+    tiny = []
+    for _ in range(64):
+        s = object.__new__(DeviceSet)
+        s.a, s.b, s.gh = (torch.rand((4, 64), device=dev) for _ in range(3))
+        s.h, s.ga, s.gb = (torch.empty_like(s.a) for _ in range(3))
+        tiny.append(s)
+    f_ms, b_ms = time_batches(tiny, 256, 64, hip, torch)
+    gf_ms, gb_ms = time_graph(tiny, 20, hip, torch)
+    out["launch_floor_4x64"] = {"fwd_us": round(f_ms * 1e3, 2), "fwd_graph_us": round(gf_ms * 1e3, 2),
+                                "bwd_us": round(b_ms * 1e3, 2), "bwd_graph_us": round(gb_ms * 1e3, 2)}
+    print(json.dumps(out))
+
+
 def channels_last_workload(spec, args, hip, torch):
     """--channels-last BxTxC[:dtype]: forward and backward over contiguous [B, T, C] tensors (scanned along T).
 
@@ -623,6 +658,8 @@ def main():
                     help="synthetic configuration the timed region runs (default 2, the one the metric is quoted on)")
     ap.add_argument("--channels-last", metavar="BxTxC[:dtype]", default=None,
                     help="time the channels-last kernels on this shape instead (dtype f32, bf16, f16 or f64) and exit")
+    ap.add_argument("--launch-shapes", action="store_true",
+                    help="time configuration 1 under every launch shape, one by one and from a HIP graph, and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (rows are independent, so more GPUs would "
@@ -643,6 +680,9 @@ def main():
     dev = torch.device("cuda:0")
     if args.channels_last:
         channels_last_workload(args.channels_last, args, hip, torch)
+        return
+    if args.launch_shapes:
+        launch_shapes(args, hip, torch)
         return
 
     cfg, label = WORKLOADS[args.workload]
