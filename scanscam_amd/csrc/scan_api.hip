@@ -583,10 +583,26 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     auto groups = [&](int vec) { return (C + (int64_t)kWave * vec - 1) / ((int64_t)kWave * vec); };
     // Pairs halve the number of workgroups: not where single channels just reach 256 of them and pairs do not.
     const int narrow = pair_possible && (batch * groups(2) >= 256 || batch * groups(1) < 256) ? 2 : 1;
+    // Element-aligned lanes: where C is no multiple of the lane's channels, or the tensors are only element-aligned,
+    // wider lanes are still possible in the kernel in which a workgroup walks all of T -- vectors loaded and
+    // stored at element alignment, the last lane of a time step on the window of channels that ends with it.
+    // Worth it when the wider lanes still give at least 256 workgroups and a time step fills a wave (not the
+    // packed kernel's regime).
+    auto ragged_fits = [&](int vec) { return vec > 1 && C >= (int64_t)kWave * vec && batch * groups(vec) >= 256; };
+    l->ragged = false;
     if (u.vec) {
         l->vec = u.vec;
     } else if (!vec_possible) {
         l->vec = narrow;
+        if (u.mode != kModeLookback) {
+            if (ragged_fits(full)) {
+                l->vec = full;
+                l->ragged = true;
+            } else if (esize == 2 && !pair_possible && ragged_fits(2)) {
+                l->vec = 2;
+                l->ragged = true;
+            }
+        }
     } else {
         // A workgroup owns 64*vec channels of one batch element. Enough of them: 16-byte loads.
         // Not enough: narrow lanes, which give full/narrow times as many workgroups; if even those
@@ -609,8 +625,11 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         if (esize == 2 && C > 32 && C < (int64_t)kWave * full) l->vec = (C == kWave || !pair_possible) ? 1 : 2;
     }
     if (l->vec != 1 && l->vec != full && !(l->vec == 2 && esize == 2)) return SCANSCAM_EPLAN;
-    if (l->vec == full && !vec_possible) return SCANSCAM_EPLAN;
-    if (l->vec == 2 && esize == 2 && !pair_possible) return SCANSCAM_EPLAN;
+    // A forced wide lane that the alignment or C does not allow as it stands: element-aligned, where that kernel applies.
+    if (u.vec && ((l->vec == full && full > 1 && !vec_possible) || (l->vec == 2 && esize == 2 && full != 2 && !pair_possible))) {
+        if (C < (int64_t)kWave * l->vec || u.mode == kModeLookback) return SCANSCAM_EPLAN;
+        l->ragged = true;
+    }
     // Too few (batch element, channel group) pairs to fill the GPU: cut time into tiles over
     // workgroups as well. kind 0: one workgroup walks all of T. kind 2: tiles by ticket with a
     // look-back chain of per-channel pairs (mode = SCANSCAM_MODE_LOOKBACK forces it,
@@ -619,6 +638,7 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     l->kind = 0;
     if (u.mode == kModeLookback || (u.mode == SCANSCAM_MODE_AUTO && rowgroups < 256)) l->kind = 2;
     if (u.mode == kModeSmall) return SCANSCAM_EPLAN;
+    if (l->ragged && l->kind != 0) return SCANSCAM_EPLAN;  // (the automatic choice never gets here: it asked for 256 workgroups)
 
     // Steps per wave per tile: with one channel per lane and tiles over workgroups, 16 (8 measured 1.2-1.4
     // times slower: twice as many tiles pay the carry wait).
@@ -636,7 +656,8 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // 48 -> 59 %, [128, 2048, 256] 56 -> 67 %), backward -2 to +4. With more workgroups, or rows too short to
     // fill such tiles, it costs 2 to 10 points; fp32 gains nothing from it.
     const bool narrow_lane = l->vec < full;
-    const bool long_steps = l->kind != 0 || (esize == 2 && rowgroups < 512 && T >= 1024);
+    // (element-aligned pairs of 16-bit channels likewise: bf16 [64, 2048, 1001] 36 / 34 -> 39 / 38 % of peak)
+    const bool long_steps = l->kind != 0 || (esize == 2 && T >= 1024 && (rowgroups < 512 || (l->ragged && l->vec == 2)));
     l->steps = u.unroll ? u.unroll : (narrow_lane ? (long_steps ? 16 : 8) : ((l->kind != 0 && full <= 4) ? 8 : 4));
     if (!u.unroll && l->group <= 16 && narrow_lane) l->steps = 4;  // packed, 4 or more steps per instruction
     const bool steps_ok = (l->vec == full) ? (l->steps == 2 || l->steps == 4 || l->steps == 8)

@@ -60,6 +60,10 @@ template <typename ST> struct ClLane {
     int pa, px, ph, py0, py1;  // elements from one time step to the next, per tensor
     unsigned c;                // byte offset of the lane's first channel (0 for a lane without channels)
     bool c_ok;
+    // Element-aligned lanes (RAGGED): C need not be a multiple of the lane's VEC channels, so the last lane of
+    // a time step may own fewer. It loads the window of VEC channels that ends with the time step instead
+    // (`c` points there) and moves its components down by `shift` places; its stores go out per channel.
+    int shift;
 
     // base + elems elements + the lane's channel offset. The lane part enters as a zero-extended 32-bit
     // byte count, the form the scalar-base addressing mode takes.
@@ -147,11 +151,25 @@ template <typename ST, int VEC> struct ClAccess<ST, VEC, false> {
 //   apply       replays the steps from the scan value entering them and stores the results
 // With APPLY = false only load_fold is used, and its loads are left cacheable (the data is
 // read again later).
-template <typename ST, int VEC, int S, bool REV, bool APPLY, typename CT, bool SPLIT = false>
+// Components of a vector moved down by s places (those moved in from above are zero).
+template <typename ST, int VEC>
+__device__ __forceinline__ typename Vec<ST, VEC>::raw_t cl_shift_down(typename Vec<ST, VEC>::raw_t r, int s)
+{
+    if constexpr (sizeof(r) == 16) {
+        return Vec<ST, VEC>::shift_components(r, -s);
+    } else if constexpr (sizeof(r) == 4) {
+        return r >> (s * (int)sizeof(ST) * 8);
+    } else {
+        return r;  // lanes of one element have nothing to move
+    }
+}
+
+template <typename ST, int VEC, int S, bool REV, bool APPLY, typename CT, bool SPLIT = false, bool RAGGED = false>
 struct ClSteps {
     using V = Vec<ST, VEC>;
     using raw_t = typename V::raw_t;
-    using BV = ClAccess<ST, VEC, cl_buffered<ST, VEC, S, REV, SPLIT>()>;
+    // Element-aligned lanes take global instructions (buffer instructions want 4-byte alignment).
+    using BV = ClAccess<ST, VEC, !RAGGED && cl_buffered<ST, VEC, S, REV, SPLIT>()>;
     using Base = typename BV::Base;
 
     CT g[S][VEC], v[S][VEC];
@@ -207,8 +225,16 @@ struct ClSteps {
     }
 
     // Folds the issued steps to one affine pair per channel (and keeps gate and value per step for apply()).
-    __device__ __forceinline__ void fold(int T, CT (&A)[VEC], CT (&B)[VEC])
+    __device__ __forceinline__ void fold(int T, CT (&A)[VEC], CT (&B)[VEC], int shift = 0)
     {
+        if (RAGGED && shift != 0) {  // the last lane of a time step: its window's components into place
+#pragma unroll
+            for (int s = 0; s < S; s++) {
+                ra[s] = cl_shift_down<ST, VEC>(ra[s], shift);
+                rx[s] = cl_shift_down<ST, VEC>(rx[s], shift);
+                if (REV && APPLY) rh[s] = cl_shift_down<ST, VEC>(rh[s], shift);
+            }
+        }
 #pragma unroll
         for (int k = 0; k < VEC; k++) {
             A[k] = CT(1);
@@ -236,7 +262,23 @@ struct ClSteps {
                                               CT (&A)[VEC], CT (&B)[VEC])
     {
         issue(ln, T, first_step, limit_);
-        fold(T, A, B);
+        fold(T, A, B, ln.shift);
+    }
+
+    // A lane's vector to its channels of one time step; the last lane of an element-aligned time step stores
+    // the channels it owns one by one (its window started `shift` channels early).
+    static __device__ __forceinline__ void put(raw_t r, Base res, const ClLane<ST> &ln, unsigned off)
+    {
+        if (!RAGGED || ln.shift == 0) {
+            BV::store(r, res, ln.c, off);
+        } else if constexpr (RAGGED) {
+            using One = ClAccess<ST, 1, false>;
+            const Elems<ST, VEC> e = __builtin_bit_cast(Elems<ST, VEC>, r);
+#pragma unroll
+            for (int k = 0; k < VEC; k++)
+                if (k < VEC - ln.shift)
+                    One::store(__builtin_bit_cast(typename One::raw_t, e.e[k]), res, ln.c + (unsigned)((ln.shift + k) * sizeof(ST)), off);
+        }
     }
 
     __device__ __forceinline__ void apply(const ClLane<ST> &ln, int T, CT (&mine)[VEC])
@@ -254,15 +296,15 @@ struct ClSteps {
                 out[k] = mine[k];
             }
             if (!REV) {
-                if (in && ln.c_ok) BV::store(V::pack(out), res_y0, ln.c, step_off(t, ln.py0));
+                if (in && ln.c_ok) put(V::pack(out), res_y0, ln, step_off(t, ln.py0));
             } else {
                 CT fh[VEC], ga[VEC];
                 V::unpack(rh[s], fh);
 #pragma unroll
                 for (int k = 0; k < VEC; k++) ga[k] = out[k] * (h_in ? fh[k] : CT(0));
                 if (in && ln.c_ok) {
-                    BV::store(V::pack(out), res_y0, ln.c, step_off(t, ln.py0));
-                    BV::store(V::pack(ga), res_y1, ln.c, step_off(t, ln.py1));
+                    put(V::pack(out), res_y0, ln, step_off(t, ln.py0));
+                    put(V::pack(ga), res_y1, ln, step_off(t, ln.py1));
                 }
             }
         }
@@ -276,11 +318,11 @@ struct ClSteps {
 //                  far; the tile's pair is composed onto it; nothing is stored
 //                  (kept for callers that only need a pair; unused by the kernels here).
 // lds_A / lds_B: [W][VEC][64] values each; the caller alternates two buffers.
-template <typename ST, int VEC, int S, bool REV, bool APPLY, typename CT>
+template <typename ST, int VEC, int S, bool REV, bool APPLY, typename CT, bool RAGGED = false>
 __device__ __forceinline__ void cl_tile(const ClLane<ST> &ln, int T, int tile0, int limit, int wave, int W,
                                         int lane, CT *lds_A, CT *lds_B, CT (&runA)[VEC], CT (&run)[VEC])
 {
-    ClSteps<ST, VEC, S, REV, APPLY, CT> steps;
+    ClSteps<ST, VEC, S, REV, APPLY, CT, false, RAGGED> steps;
     CT A[VEC], B[VEC];
     steps.load_fold(ln, T, tile0 + wave * S, limit, A, B);
 
@@ -322,13 +364,14 @@ __device__ __forceinline__ int xcd_contiguous(int r, int n)
     return xcd < rem ? xcd * per + slot : rem * per + (xcd - rem) * (per - 1) + slot;
 }
 
-template <typename ST, int VEC>
+template <typename ST, int VEC, bool RAGGED = false>
 __device__ __forceinline__ ClLane<ST> cl_lane(const ClArgs &p, int64_t batch_index, int group, int lane)
 {
     const int64_t c0 = ((int64_t)group * kWave + lane) * VEC;  // first channel of this lane
     ClLane<ST> ln;
     ln.c_ok = c0 < p.C;
-    ln.c = ln.c_ok ? (unsigned)(c0 * sizeof(ST)) : 0u;
+    ln.shift = (RAGGED && ln.c_ok && c0 + VEC > p.C) ? (int)(c0 + VEC - p.C) : 0;  // C >= VEC: the host checks it
+    ln.c = ln.c_ok ? (unsigned)((c0 - ln.shift) * sizeof(ST)) : 0u;
     ln.a = static_cast<const ST *>(p.a) + batch_index * p.sB[0];
     ln.x = static_cast<const ST *>(p.x) + batch_index * p.sB[1];
     ln.h = static_cast<const ST *>(p.h) + batch_index * p.sB[2];
@@ -343,7 +386,7 @@ __device__ __forceinline__ ClLane<ST> cl_lane(const ClArgs &p, int64_t batch_ind
 }
 
 // Dynamic LDS: two buffers (tiles alternate) of A and B, each [W][VEC][64] values.
-template <typename ST, int VEC, int S, bool REV, int MAXT>
+template <typename ST, int VEC, int S, bool REV, int MAXT, bool RAGGED = false>
 __global__ __launch_bounds__(MAXT) void scan_cl_kernel(const ClArgs p)
 {
     using CT = typename ComputeOf<ST>::type;
@@ -360,7 +403,7 @@ __global__ __launch_bounds__(MAXT) void scan_cl_kernel(const ClArgs p)
     // xcd_order gives each XCD a contiguous run of (batch element, channel group) pairs instead, so that
     // neighbours meet in one L2.
     const int bid = p.xcd_order ? xcd_contiguous((int)blockIdx.x, (int)gridDim.x) : (int)blockIdx.x;
-    const ClLane<ST> ln = cl_lane<ST, VEC>(p, bid / groups, bid % groups, lane);
+    const ClLane<ST> ln = cl_lane<ST, VEC, RAGGED>(p, bid / groups, bid % groups, lane);
 
     const int tile_steps = W * S;
     const int ntiles = (p.T + tile_steps - 1) / tile_steps;
@@ -371,8 +414,8 @@ __global__ __launch_bounds__(MAXT) void scan_cl_kernel(const ClArgs p)
 
     for (int it = 0; it < ntiles; it++) {
         CT *lds_A = lds + (it & 1) * 2 * plane;
-        cl_tile<ST, VEC, S, REV, true, CT>(ln, p.T, it * tile_steps, p.T, wave, W, lane, lds_A, lds_A + plane,
-                                           unused, carry);
+        cl_tile<ST, VEC, S, REV, true, CT, RAGGED>(ln, p.T, it * tile_steps, p.T, wave, W, lane, lds_A, lds_A + plane,
+                                                   unused, carry);
     }
 }
 

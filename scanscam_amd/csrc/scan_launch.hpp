@@ -124,6 +124,8 @@ struct ClLaunch {
     int kind;       // 0: a workgroup walks all of T; 2: tiles over workgroups with a look-back chain
     int group;      // kind 0: lanes per time step; below 64: the packed kernel for few channels
     int segments;   // kind 2: tiles per row-group
+    bool ragged;    // kind 0, full lanes of a wave: lanes of vec channels on time steps that are only element-aligned,
+                    // or whose C is no multiple of vec
     int64_t grid;
     size_t lds_bytes;
     size_t ws_bytes;
@@ -143,6 +145,13 @@ hipError_t launch_scan_cl(const ClArgs &args, const ClLaunch &l, bool rev, hipSt
         } else if (l.group < kWave) {                                                                  \
             if (rev) hipLaunchKernelGGL((scan_cl_packed_kernel<ST, VEC, S, true, MAXT>), grid, block, l.lds_bytes, stream, args);  \
             else     hipLaunchKernelGGL((scan_cl_packed_kernel<ST, VEC, S, false, MAXT>), grid, block, l.lds_bytes, stream, args); \
+        } else if (l.ragged) {                                                                         \
+            if constexpr ((VEC) > 1) {                                                                 \
+                if (rev) hipLaunchKernelGGL((scan_cl_kernel<ST, VEC, S, true, MAXT, true>), grid, block, l.lds_bytes, stream, args);  \
+                else     hipLaunchKernelGGL((scan_cl_kernel<ST, VEC, S, false, MAXT, true>), grid, block, l.lds_bytes, stream, args); \
+            } else {                                                                                   \
+                return hipErrorInvalidValue;                                                           \
+            }                                                                                          \
         } else {                                                                                       \
             if (rev) hipLaunchKernelGGL((scan_cl_kernel<ST, VEC, S, true, MAXT>), grid, block, l.lds_bytes, stream, args);  \
             else     hipLaunchKernelGGL((scan_cl_kernel<ST, VEC, S, false, MAXT>), grid, block, l.lds_bytes, stream, args); \

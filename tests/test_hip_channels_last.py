@@ -104,6 +104,54 @@ def test_forced_plans(gpu, dtype):
     assert n > 60
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16, torch.float16])
+def test_element_aligned_lanes(gpu, dtype):
+    """Wide lanes where C is no multiple of the lane's channels, or the tensors start at any element."""
+    full = 16 // torch.empty(0, dtype=dtype).element_size()
+    bar = {torch.float32: 1e-5, torch.float64: 1e-13}.get(dtype, 1e-2)
+    g = torch.Generator().manual_seed(23)
+    n = 0
+    for shape in [(3, 107, 64 * full + 1), (2, 70, 64 * full + full - 1), (5, 33, 130 * full + 3), (2, 50, 401)]:
+        a = torch.rand(shape, generator=g, dtype=torch.float64).to(dtype)
+        b = torch.randn(shape, generator=g, dtype=torch.float64).to(dtype)
+        gh = torch.randn(shape, generator=g, dtype=torch.float64).to(dtype)
+        h = oracle.fwd(as_rows(a), as_rows(b))
+        hs = torch.from_numpy(h).mT.contiguous().to(dtype)
+        ga, gb = oracle.bwd(as_rows(a), as_rows(hs), as_rows(gh))
+        hp = prev_abs(as_rows(hs))
+        numel = a.numel()
+        for offset in (0, 1):  # views that start one element into their allocation
+            def view_of(t):
+                buf = torch.full((numel + 8,), float("nan"), dtype=dtype, device=gpu)
+                v = buf[offset:offset + numel].view(shape)
+                v.copy_(t)
+                return v
+            da, db, dgh, dhs = view_of(a), view_of(b), view_of(gh), view_of(hs)
+            for vec in ((full, 2) if full == 8 else (full,)):
+                if shape[-1] < 64 * vec:
+                    continue
+                for steps in ((2, 4, 8) if vec == full else (4, 8, 16)):
+                    plan = hip.Plan(vec=vec, unroll=steps, waves=3, mode=hip.MODE_ROW)
+                    print(f"case cl element-aligned {dtype} shape={shape} offset={offset} {plan}", flush=True)
+                    got_h = hip.transposed_linear_scan_forward(da, db, plan=plan)
+                    got_ga, got_gb = hip.transposed_linear_scan_backward(da, dhs, dgh, plan=plan)
+                    assert rel_err(as_rows(got_h), h) <= bar, (plan, shape)
+                    assert rel_err(as_rows(got_gb), gb) <= bar, (plan, shape)
+                    assert rel_err(as_rows(got_ga), ga, hp) <= bar, (plan, shape)
+                    n += 1
+    assert n >= 20
+    # The automatic choice takes such lanes where they still give 256 workgroups ...
+    shape = (260, 40, 64 * full + 5)
+    a = torch.rand(shape, generator=g, dtype=torch.float64).to(dtype)
+    b = torch.randn(shape, generator=g, dtype=torch.float64).to(dtype)
+    want = oracle.fwd(as_rows(a), as_rows(b))
+    assert rel_err(as_rows(hip.transposed_linear_scan_forward(a.to(gpu), b.to(gpu))), want) <= bar
+    # ... and a forced wide lane is refused where a time step does not fill a wave of them.
+    small = torch.rand(2, 8, 64 * full - 3, device=gpu).to(dtype)
+    with pytest.raises(RuntimeError, match="plan"):
+        hip.transposed_linear_scan_forward(small, small, plan=hip.Plan(vec=full, mode=hip.MODE_ROW))
+
+
 def test_matches_row_layout_kernels(gpu):
     # Same data through both layouts: the two kernel families must agree closely
     # (each is within 1e-5 of the oracle; they differ only in association order).
