@@ -12,7 +12,7 @@ backward reads a, h, grad_h and writes grad_a, grad_b = 20 B).
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-configs] [--workload N]
                     [--channels-last BxTxC[:dtype]] [--launch-shapes]
 
---workload runs another of the synthetic configurations (1, 3, 4, 4f16, 5; or `long`, `long16`) through the same timed
+--workload runs another of the synthetic configurations (1, 3, 4, 4f16, 5; or `long`, `long16`, `short70`) through the same timed
 region instead of configuration 2 (used for the rocprofv3 summaries under profiles/).
 
 Prints ONE JSON line. Besides the contract fields it carries
@@ -119,6 +119,8 @@ WORKLOADS = {
     "5": (5, "configs[4]: forward + backward fp32 scan, many short rows [B=256, C=512, T=64], a ~ U(0,1), b ~ N(0,1)"),
     "long16": (60, "long-context shape in bf16 storage / fp32 arithmetic (not one of the five configurations): "
                    "forward + backward scan, [B=1, C=2048, T=32768], a=sigmoid(N(0,1)), b ~ N(0,1)"),
+    "short70": (7, "short rows of odd length (not one of the five configurations): forward + backward fp32 scan, "
+                   "[958698, 70], a ~ U(0,1), b ~ N(0,1)"),
     "long": (6, "long-context shape (not one of the five configurations): forward + backward fp32 scan, "
                 "[B=1, C=2048, T=32768], a=sigmoid(N(0,1)), b ~ N(0,1)"),
 }
@@ -148,6 +150,9 @@ def make_config(n, torch):
         shape = (1, 2048, 32768)
         a, b = torch.sigmoid(torch.randn(shape)), torch.randn(shape)
         dtype = torch.float32 if n == 6 else torch.bfloat16
+    elif n == 7:
+        shape = (958698, 70)
+        a, b = torch.rand(shape), torch.randn(shape)
     elif n == 20:  # configuration 2's bytes in float64 (the reference's other storage type): half its T
         shape = (8, 2048, 2048)
         a, b = torch.sigmoid(torch.randn(shape)), torch.randn(shape)
