@@ -730,6 +730,7 @@ def main():
             "elements": n,
             "buffer_sets": nsets,
             "plan": repr(plan_f),
+            "library": os.path.relpath(hip.LIB_PATH, ROOT),  # the build that ran (SCANSCAM_HIP_LIB may name another)
         },
         "frac_of_peak": round(step_gbps / HBM_PEAK_GBPS, 4),
         # The steadier figure: median over the launches after the region of (forward + backward kernel

@@ -33,6 +33,13 @@ __global__ __launch_bounds__(256) void scan_ws_clear_kernel(uint64_t *ws, int64_
     if (i < words) ws[i] = 0;
 }
 
+hipError_t clear_workspace(uint64_t *ws, int64_t words, hipStream_t stream)
+{
+    void *params[] = {&ws, &words};
+    return hipLaunchKernel(reinterpret_cast<const void *>(scan_ws_clear_kernel), dim3((unsigned)((words + 255) / 256)),
+                           dim3(256), params, 0, stream);
+}
+
 constexpr int64_t kMaxT = (int64_t(1) << 31) - (int64_t(1) << 20);
 
 int elem_size(int dtype)
@@ -523,9 +530,7 @@ int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y
         if (!aligned_to(workspace, 8)) return SCANSCAM_EALIGN;
         args.ws = static_cast<uint64_t *>(workspace);
         const int64_t words = (int64_t)(r.ws_bytes / sizeof(uint64_t));
-        hipLaunchKernelGGL(scan_ws_clear_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0,
-                           s, args.ws, words);
-        if (hipGetLastError() != hipSuccess) return SCANSCAM_ELAUNCH;
+        if (clear_workspace(args.ws, words, s) != hipSuccess) return SCANSCAM_ELAUNCH;
         // One launch over all rows; the kernel splits a row index into (group, row). Its grid is far
         // below every launch limit by construction.
         return launch(args, r.l) == hipSuccess ? SCANSCAM_OK : SCANSCAM_ELAUNCH;
@@ -776,9 +781,7 @@ int run_cl(bool rev, const void *a, const void *x, const void *h, void *y0, void
         if (!aligned_to(workspace, 8)) return SCANSCAM_EALIGN;
         args.ws = static_cast<uint64_t *>(workspace);
         const int64_t words = (int64_t)(l.ws_bytes / sizeof(uint64_t));
-        hipLaunchKernelGGL(scan_ws_clear_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, s, args.ws,
-                           words);
-        if (hipGetLastError() != hipSuccess) return SCANSCAM_ELAUNCH;
+        if (clear_workspace(args.ws, words, s) != hipSuccess) return SCANSCAM_ELAUNCH;
     }
     hipError_t e = hipErrorInvalidValue;
     switch (dtype) {

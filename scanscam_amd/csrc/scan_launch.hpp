@@ -27,6 +27,18 @@ struct Launch {
 // Largest workgroup (threads) a kernel with U chunks per wave is compiled for.
 constexpr int max_threads_for_unroll(int unroll) { return unroll <= 4 ? 1024 : 256; }
 
+// Launches `kernel(args)` and returns what the launch call itself returns (the runtime's sticky "last error" is
+// neither read nor cleared, so an error the host application left there is not taken for this launch's, and
+// stays there for the application to find). `start` / `stop` (may be null) receive the kernel's own time stamps.
+template <typename Kernel, typename Args>
+inline hipError_t launch_kernel(Kernel kernel, dim3 grid, dim3 block, size_t lds_bytes, hipStream_t stream,
+                                hipEvent_t start, hipEvent_t stop, const Args &args)
+{
+    Args copy = args;
+    void *params[] = {&copy};
+    return hipExtLaunchKernel(reinterpret_cast<const void *>(kernel), grid, block, params, lds_bytes, stream, start, stop, 0);
+}
+
 // One per storage type, defined in scan_f32.hip / scan_bf16.hip / scan_f16.hip.
 // Returns hipErrorInvalidValue when (vec, unroll) is not an instantiated pair. `start` / `stop`
 // (may be null) receive the kernel's own start and end time stamps.
@@ -37,34 +49,36 @@ hipError_t launch_scan(const ScanArgs &args, const Launch &l, bool rev, hipStrea
 #define SCANSCAM_LAUNCH_CASE(ST, VEC, U)                                                             \
     if (l.vec == (VEC) && l.unroll == (U)) {                                                         \
         constexpr int MAXT = max_threads_for_unroll(U);                                              \
+        hipError_t err = hipErrorInvalidValue;                                                       \
         if (l.mode == kModeSmall) {                                                                  \
-            if (rev) hipExtLaunchKernelGGL((scan_small_kernel<ST, VEC, U, true, MAXT>), grid, block, 0, stream, start, stop, 0, args);    \
-            else     hipExtLaunchKernelGGL((scan_small_kernel<ST, VEC, U, false, MAXT>), grid, block, 0, stream, start, stop, 0, args);   \
+            if (rev) err = launch_kernel(scan_small_kernel<ST, VEC, U, true, MAXT>, grid, block, 0, stream, start, stop, args);    \
+            else     err = launch_kernel(scan_small_kernel<ST, VEC, U, false, MAXT>, grid, block, 0, stream, start, stop, args);   \
         } else if (l.mode == kModeRow) {                                                             \
-            if (rev) hipExtLaunchKernelGGL((scan_row_kernel<ST, VEC, U, true, MAXT>), grid, block, 0, stream, start, stop, 0, args);      \
-            else     hipExtLaunchKernelGGL((scan_row_kernel<ST, VEC, U, false, MAXT>), grid, block, 0, stream, start, stop, 0, args);     \
+            if (rev) err = launch_kernel(scan_row_kernel<ST, VEC, U, true, MAXT>, grid, block, 0, stream, start, stop, args);      \
+            else     err = launch_kernel(scan_row_kernel<ST, VEC, U, false, MAXT>, grid, block, 0, stream, start, stop, args);     \
         } else {                                                                                     \
-            if (rev) hipExtLaunchKernelGGL((scan_lookback_kernel<ST, VEC, U, true, MAXT>), grid, block, 0, stream, start, stop, 0, args); \
-            else     hipExtLaunchKernelGGL((scan_lookback_kernel<ST, VEC, U, false, MAXT>), grid, block, 0, stream, start, stop, 0, args);\
+            if (rev) err = launch_kernel(scan_lookback_kernel<ST, VEC, U, true, MAXT>, grid, block, 0, stream, start, stop, args); \
+            else     err = launch_kernel(scan_lookback_kernel<ST, VEC, U, false, MAXT>, grid, block, 0, stream, start, stop, args);\
         }                                                                                            \
-        return hipGetLastError();                                                                    \
+        return err;                                                                    \
     }
 
 // The same for rows that are only element-aligned (full vector, U = 2 or 4).
 #define SCANSCAM_RAGGED_CASE(ST, VEC, U)                                                             \
     if (l.ragged && l.vec == (VEC) && l.unroll == (U)) {                                             \
         constexpr int MAXT = max_threads_for_unroll(U);                                              \
+        hipError_t err = hipErrorInvalidValue;                                                       \
         if (l.mode == kModeRow) {                                                                    \
-            if (rev) hipExtLaunchKernelGGL((scan_row_kernel<ST, VEC, U, true, MAXT, true>), grid, block, 0, stream, start, stop, 0, args);      \
-            else     hipExtLaunchKernelGGL((scan_row_kernel<ST, VEC, U, false, MAXT, true>), grid, block, 0, stream, start, stop, 0, args);     \
+            if (rev) err = launch_kernel(scan_row_kernel<ST, VEC, U, true, MAXT, true>, grid, block, 0, stream, start, stop, args);      \
+            else     err = launch_kernel(scan_row_kernel<ST, VEC, U, false, MAXT, true>, grid, block, 0, stream, start, stop, args);     \
         } else if (l.mode == kModeLookback) {                                                        \
-            if (rev) hipExtLaunchKernelGGL((scan_lookback_kernel<ST, VEC, U, true, MAXT, true>), grid, block, 0, stream, start, stop, 0, args); \
-            else     hipExtLaunchKernelGGL((scan_lookback_kernel<ST, VEC, U, false, MAXT, true>), grid, block, 0, stream, start, stop, 0, args);\
+            if (rev) err = launch_kernel(scan_lookback_kernel<ST, VEC, U, true, MAXT, true>, grid, block, 0, stream, start, stop, args); \
+            else     err = launch_kernel(scan_lookback_kernel<ST, VEC, U, false, MAXT, true>, grid, block, 0, stream, start, stop, args);\
         } else {                                                                                     \
-            if (rev) hipExtLaunchKernelGGL((scan_small_kernel<ST, VEC, U, true, MAXT, true>), grid, block, 0, stream, start, stop, 0, args);    \
-            else     hipExtLaunchKernelGGL((scan_small_kernel<ST, VEC, U, false, MAXT, true>), grid, block, 0, stream, start, stop, 0, args);   \
+            if (rev) err = launch_kernel(scan_small_kernel<ST, VEC, U, true, MAXT, true>, grid, block, 0, stream, start, stop, args);    \
+            else     err = launch_kernel(scan_small_kernel<ST, VEC, U, false, MAXT, true>, grid, block, 0, stream, start, stop, args);   \
         }                                                                                            \
-        return hipGetLastError();                                                                    \
+        return err;                                                                    \
     }
 
 #define SCANSCAM_DEFINE_LAUNCH(ST)                                                                   \
@@ -96,9 +110,10 @@ hipError_t launch_scan_flat(const FlatArgs &args, int unroll, int waves, bool re
 
 #define SCANSCAM_FLAT_CASE(ST, U)                                                                     \
     if (unroll == (U)) {                                                                              \
-        if (rev) hipExtLaunchKernelGGL((scan_flat_kernel<ST, FULL, U, true, 1024>), grid, block, 0, stream, start, stop, 0, args);  \
-        else     hipExtLaunchKernelGGL((scan_flat_kernel<ST, FULL, U, false, 1024>), grid, block, 0, stream, start, stop, 0, args); \
-        return hipGetLastError();                                                                     \
+        hipError_t err = hipErrorInvalidValue;                                                        \
+        if (rev) err = launch_kernel(scan_flat_kernel<ST, FULL, U, true, 1024>, grid, block, 0, stream, start, stop, args);  \
+        else     err = launch_kernel(scan_flat_kernel<ST, FULL, U, false, 1024>, grid, block, 0, stream, start, stop, args); \
+        return err;                                                                     \
     }
 
 #define SCANSCAM_DEFINE_FLAT_LAUNCH(ST)                                                               \
@@ -139,24 +154,25 @@ hipError_t launch_scan_cl(const ClArgs &args, const ClLaunch &l, bool rev, hipSt
 #define SCANSCAM_CL_CASE(ST, VEC, S)                                                                   \
     if (l.vec == (VEC) && l.steps == (S)) {                                                            \
         constexpr int MAXT = cl_max_threads(VEC, S);                                                   \
+        hipError_t err = hipErrorInvalidValue;                                                         \
         if (l.kind == 2) {                                                                             \
-            if (rev) hipLaunchKernelGGL((scan_cl_lookback_kernel<ST, VEC, S, true, MAXT>), grid, block, l.lds_bytes, stream, args);  \
-            else     hipLaunchKernelGGL((scan_cl_lookback_kernel<ST, VEC, S, false, MAXT>), grid, block, l.lds_bytes, stream, args); \
+            if (rev) err = launch_kernel(scan_cl_lookback_kernel<ST, VEC, S, true, MAXT>, grid, block, l.lds_bytes, stream, nullptr, nullptr, args);  \
+            else     err = launch_kernel(scan_cl_lookback_kernel<ST, VEC, S, false, MAXT>, grid, block, l.lds_bytes, stream, nullptr, nullptr, args); \
         } else if (l.group < kWave) {                                                                  \
-            if (rev) hipLaunchKernelGGL((scan_cl_packed_kernel<ST, VEC, S, true, MAXT>), grid, block, l.lds_bytes, stream, args);  \
-            else     hipLaunchKernelGGL((scan_cl_packed_kernel<ST, VEC, S, false, MAXT>), grid, block, l.lds_bytes, stream, args); \
+            if (rev) err = launch_kernel(scan_cl_packed_kernel<ST, VEC, S, true, MAXT>, grid, block, l.lds_bytes, stream, nullptr, nullptr, args);  \
+            else     err = launch_kernel(scan_cl_packed_kernel<ST, VEC, S, false, MAXT>, grid, block, l.lds_bytes, stream, nullptr, nullptr, args); \
         } else if (l.ragged) {                                                                         \
             if constexpr ((VEC) > 1) {                                                                 \
-                if (rev) hipLaunchKernelGGL((scan_cl_kernel<ST, VEC, S, true, MAXT, true>), grid, block, l.lds_bytes, stream, args);  \
-                else     hipLaunchKernelGGL((scan_cl_kernel<ST, VEC, S, false, MAXT, true>), grid, block, l.lds_bytes, stream, args); \
+                if (rev) err = launch_kernel(scan_cl_kernel<ST, VEC, S, true, MAXT, true>, grid, block, l.lds_bytes, stream, nullptr, nullptr, args);  \
+                else     err = launch_kernel(scan_cl_kernel<ST, VEC, S, false, MAXT, true>, grid, block, l.lds_bytes, stream, nullptr, nullptr, args); \
             } else {                                                                                   \
                 return hipErrorInvalidValue;                                                           \
             }                                                                                          \
         } else {                                                                                       \
-            if (rev) hipLaunchKernelGGL((scan_cl_kernel<ST, VEC, S, true, MAXT>), grid, block, l.lds_bytes, stream, args);  \
-            else     hipLaunchKernelGGL((scan_cl_kernel<ST, VEC, S, false, MAXT>), grid, block, l.lds_bytes, stream, args); \
+            if (rev) err = launch_kernel(scan_cl_kernel<ST, VEC, S, true, MAXT>, grid, block, l.lds_bytes, stream, nullptr, nullptr, args);  \
+            else     err = launch_kernel(scan_cl_kernel<ST, VEC, S, false, MAXT>, grid, block, l.lds_bytes, stream, nullptr, nullptr, args); \
         }                                                                                              \
-        return hipGetLastError();                                                                      \
+        return err;                                                                      \
     }
 
 #define SCANSCAM_DEFINE_CL_LAUNCH(ST)                                                                  \
