@@ -575,16 +575,21 @@ int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y
 }
 
 // Channels-last: choice of vector width, steps per wave and waves per workgroup.
-int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, int dtype, bool aligned16, bool aligned4,
+// `align`: the largest of 16, 8, 4 and the element size that every tensor's base and strides are multiples of (bytes).
+int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, int dtype, int align, bool rev,
                scanscam::ClLaunch *l)
 {
     const int esize = elem_size(dtype);
     const int full = 16 / esize;
+    const bool aligned16 = align >= 16, aligned4 = align >= 4;
     scanscam_plan u = {0, 0, 0, 0, 0, 0};
     if (user) u = *user;
     const bool vec_possible = aligned16 && (C % full == 0);
     // The narrow lane: one channel, or two for 16-bit storage (4 bytes, like one fp32 channel).
     const bool pair_possible = esize == 2 && aligned4 && (C % 2 == 0);
+    // The 8-byte lane: two fp32 channels, four 16-bit ones.
+    const int half = esize <= 4 ? full / 2 : 0;
+    const bool half_possible = half > 0 && align >= 8 && (C % half == 0);
     auto groups = [&](int vec) { return (C + (int64_t)kWave * vec - 1) / ((int64_t)kWave * vec); };
     // Pairs halve the number of workgroups: not where single channels just reach 256 of them and pairs do not.
     const int narrow = pair_possible && (batch * groups(2) >= 256 || batch * groups(1) < 256) ? 2 : 1;
@@ -603,6 +608,11 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
             if (ragged_fits(full)) {
                 l->vec = full;
                 l->ragged = true;
+            } else if (half_possible && ragged_fits(half)) {
+                l->vec = half;  // whole 8-byte lanes, nothing element-aligned about them
+            } else if (half > 1 && ragged_fits(half)) {
+                l->vec = half;
+                l->ragged = true;
             } else if (esize == 2 && !pair_possible && ragged_fits(2)) {
                 l->vec = 2;
                 l->ragged = true;
@@ -616,6 +626,17 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         // [1, 262144, 256] to [8, 4096, 512]; 16-bit storage 2.5-16 times, its 16-byte lanes leave
         // 8 times fewer chains).
         l->vec = batch * groups(full) >= 256 ? full : narrow;
+        // 8-byte lanes, where they still give 256 workgroups and fill their waves to three quarters: they
+        // stream as fast as 16-byte lanes or faster at equal shapes (two or four times the waves per byte in
+        // flight: fp32 [256, 1024, 1024] 71 / 76 -> 80 / 74 % of peak, [128, 2048, 512] 72 / 70 -> 78 / 75 %, bf16
+        // [256, 1024, 1024] 69 / 68 -> 75 / 74 %, [160, 2048, 1024] 59 / 57 -> 70 / 69 %) and reach shapes where 16-byte
+        // lanes leave too few workgroups and narrow lanes were the only choice (fp32 [32, 2048, 1024] 67 / 65 ->
+        // 73 / 78 %, [64, 2048, 512] 67 / 66 -> 75 / 70 %, bf16 [32, 4096, 2048] 66 / 62 -> 69 / 72 %).
+        // (Time steps that are not whole 128-byte lines keep 16-byte lanes where those give 256 workgroups:
+        // fp32 [64, 2048, 1016] backward 57 % against 50 %.)
+        if (half_possible && C >= (int64_t)kWave * half && C * 4 >= groups(half) * kWave * half * 3 &&
+            batch * groups(half) >= 256 && (l->vec != full || (C * esize) % 128 == 0))
+            l->vec = half;
         // Few channels (the packed kernel, below): a wide lane leaves more steps per instruction to scan
         // across with lane shuffles, which costs more than the wider loads gain -- except where C is not a
         // power of two and one channel per lane would leave a quarter of 32 lanes idle (fp32 [256, 8192, 24]:
@@ -629,9 +650,10 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         // instruction, against 33 / 29 %).
         if (esize == 2 && C > 32 && C < (int64_t)kWave * full) l->vec = (C == kWave || !pair_possible) ? 1 : 2;
     }
-    if (l->vec != 1 && l->vec != full && !(l->vec == 2 && esize == 2)) return SCANSCAM_EPLAN;
+    if (l->vec != 1 && l->vec != full && !(l->vec == 2 && esize == 2) && !(half > 1 && l->vec == half)) return SCANSCAM_EPLAN;
     // A forced wide lane that the alignment or C does not allow as it stands: element-aligned, where that kernel applies.
-    if (u.vec && ((l->vec == full && full > 1 && !vec_possible) || (l->vec == 2 && esize == 2 && full != 2 && !pair_possible))) {
+    if (u.vec && ((l->vec == full && full > 1 && !vec_possible) || (l->vec == 2 && esize == 2 && full != 2 && !pair_possible) ||
+                  (half > 1 && l->vec == half && !half_possible))) {
         if (C < (int64_t)kWave * l->vec || u.mode == kModeLookback) return SCANSCAM_EPLAN;
         l->ragged = true;
     }
@@ -639,10 +661,19 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // workgroups as well. kind 0: one workgroup walks all of T. kind 2: tiles by ticket with a
     // look-back chain of per-channel pairs (mode = SCANSCAM_MODE_LOOKBACK forces it,
     // SCANSCAM_MODE_ROW forbids it).
-    const int64_t rowgroups = batch * groups(l->vec);
+    int64_t rowgroups = batch * groups(l->vec);
     l->kind = 0;
     if (u.mode == kModeLookback || (u.mode == SCANSCAM_MODE_AUTO && rowgroups < 256)) l->kind = 2;
     if (u.mode == kModeSmall) return SCANSCAM_EPLAN;
+    // Tiles over workgroups, lanes chosen here: 8-byte lanes where C fills whole waves of them, in the
+    // direction in which they measured faster than the narrow lane (16 steps per wave either way) -- the
+    // backward pass of 16-bit storage (bf16 [8, 4096, 512] 48 -> 38 us, [8, 4096, 2048] 166 -> 140 us,
+    // [1, 262144, 256] 198 -> 167 us; forward 3 to 10 % slower) and the forward pass of fp32
+    // ([8, 4096, 512] 47 -> 44 us, [1, 262144, 256] 203 -> 182 us; backward 15 to 25 % slower).
+    if (l->kind == 2 && !u.vec && half_possible && C % ((int64_t)kWave * half) == 0 && (esize == 2 ? rev : !rev)) {
+        l->vec = half;
+        rowgroups = batch * groups(half);
+    }
     if (l->ragged && l->kind != 0) return SCANSCAM_EPLAN;  // (the automatic choice never gets here: it asked for 256 workgroups)
 
     // Steps per wave per tile: with one channel per lane and tiles over workgroups, 16 (8 measured 1.2-1.4
@@ -662,7 +693,7 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // fill such tiles, it costs 2 to 10 points; fp32 gains nothing from it.
     const bool narrow_lane = l->vec < full;
     // (element-aligned pairs of 16-bit channels likewise: bf16 [64, 2048, 1001] 36 / 34 -> 39 / 38 % of peak)
-    const bool long_steps = l->kind != 0 || (esize == 2 && T >= 1024 && (rowgroups < 512 || (l->ragged && l->vec == 2)));
+    const bool long_steps = l->kind != 0 || (esize == 2 && l->vec <= 2 && T >= 1024 && (rowgroups < 512 || (l->ragged && l->vec == 2)));
     l->steps = u.unroll ? u.unroll : (narrow_lane ? (long_steps ? 16 : 8) : ((l->kind != 0 && full <= 4) ? 8 : 4));
     if (!u.unroll && l->group <= 16 && narrow_lane) l->steps = 4;  // packed, 4 or more steps per instruction
     const bool steps_ok = (l->vec == full) ? (l->steps == 2 || l->steps == 4 || l->steps == 8)
@@ -690,7 +721,7 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         // would be mostly empty (320 workgroups = 1.25 rounds), 4-wave workgroups, several per CU, finish
         // together instead: fp32 [80, 2048, 1024] 445 / 699 us -> 361 / 661 us, [64, 2048, 1032] 494 / 766 ->
         // 413 / 734 us. (16-byte lanes only: narrow lanes need the waves to keep enough bytes in flight.)
-        if (l->kind == 0 && l->group == kWave && l->vec == full && l->waves > 4 && rowgroups > kComputeUnits) {
+        if (l->kind == 0 && l->group == kWave && l->vec * esize >= 8 && l->waves > 4 && rowgroups > kComputeUnits) {
             const int64_t rounds = (rowgroups + kComputeUnits - 1) / kComputeUnits;
             if (rowgroups * 100 < rounds * kComputeUnits * 85) l->waves = 4;
         }
@@ -733,20 +764,19 @@ int run_cl(bool rev, const void *a, const void *x, const void *h, void *y0, void
     // Tensor order a, x, h, y0, y1; the forward pass has no h and no y1 (they alias a and y0).
     const void *ptrs[5] = {a, x, rev ? h : a, y0, rev ? y1 : y0};
     const int src[5] = {0, 1, rev ? 2 : 0, 3, rev ? 4 : 3};
-    const int full = 16 / esize;
     int64_t sB[5], sT[5];
-    bool aligned16 = true, aligned4 = true;  // aligned4: what two-channel lanes of 16-bit storage need
+    int align = 16;  // bytes every base and stride is a multiple of: 16, 8, 4 or the element size
     for (int k = 0; k < 5; k++) {
         const scanscam_strides *t = st[src[k]];
         sB[k] = batch == 1 ? 0 : (t ? t->outer : T * C);
         sT[k] = T == 1 ? 0 : (t ? t->row : C);
         if (sB[k] < 0 || sT[k] < 0 || sT[k] >= kMaxT) return SCANSCAM_EINVAL;
         if (!aligned_to(ptrs[k], (size_t)esize)) return SCANSCAM_EALIGN;
-        aligned16 = aligned16 && aligned_to(ptrs[k], 16) && sB[k] % full == 0 && sT[k] % full == 0;
-        aligned4 = aligned4 && aligned_to(ptrs[k], 4) && sB[k] % 2 == 0 && sT[k] % 2 == 0;
+        while (align > esize && !(aligned_to(ptrs[k], (size_t)align) && (sB[k] * esize) % align == 0 && (sT[k] * esize) % align == 0))
+            align >>= 1;
     }
     scanscam::ClLaunch l;
-    const int rc = resolve_cl(plan, batch, T, C, dtype, aligned16, aligned4, &l);
+    const int rc = resolve_cl(plan, batch, T, C, dtype, align, rev, &l);
     if (rc != SCANSCAM_OK) return rc;
     // A wave addresses its steps (at most 16, and one neighbour on either side backwards) with 32-bit byte
     // offsets from its first one, the lane's channel included.
@@ -885,13 +915,14 @@ int scanscam_scan_bwd_cl(const void *a, const void *h, const void *gh, void *ga,
 size_t scanscam_workspace_bytes_cl(int64_t batch, int64_t T, int64_t C, int dtype, int direction,
                                    const scanscam_plan *plan)
 {
-    (void)direction;
-    if (elem_size(dtype) == 0 || batch <= 0 || T <= 0 || C <= 0 || T >= kMaxT || C >= kMaxT) return 0;
+    const int esize = elem_size(dtype);
+    if (esize == 0 || batch <= 0 || T <= 0 || C <= 0 || T >= kMaxT || C >= kMaxT) return 0;
     size_t need = 0;
-    for (int al = 0; al < 3; al++) {
+    // The caller's pointers are not known yet: every alignment the tensors may turn out to have.
+    for (int align = 16; align >= esize; align >>= 1) {
         scanscam::ClLaunch l;
-        // al: 0 = element-aligned only, 1 = 4-byte aligned (16-bit pairs), 2 = 16-byte aligned
-        if (resolve_cl(plan, batch, T, C, dtype, al == 2, al >= 1, &l) == SCANSCAM_OK && l.ws_bytes > need) need = l.ws_bytes;
+        if (resolve_cl(plan, batch, T, C, dtype, align, direction == SCANSCAM_BACKWARD, &l) == SCANSCAM_OK && l.ws_bytes > need)
+            need = l.ws_bytes;
     }
     return need;
 }

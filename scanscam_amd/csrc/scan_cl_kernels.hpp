@@ -157,6 +157,12 @@ __device__ __forceinline__ typename Vec<ST, VEC>::raw_t cl_shift_down(typename V
 {
     if constexpr (sizeof(r) == 16) {
         return Vec<ST, VEC>::shift_components(r, -s);
+    } else if constexpr (sizeof(r) == 8) {
+        const uint64_t v = ((uint64_t)r.x | ((uint64_t)r.y << 32)) >> (s * (int)sizeof(ST) * 8);
+        decltype(r) out;
+        out.x = (uint32_t)v;
+        out.y = (uint32_t)(v >> 32);
+        return out;
     } else if constexpr (sizeof(r) == 4) {
         return r >> (s * (int)sizeof(ST) * 8);
     } else {

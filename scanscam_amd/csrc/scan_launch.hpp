@@ -192,6 +192,12 @@ hipError_t launch_scan_cl(const ClArgs &args, const ClLaunch &l, bool rev, hipSt
             SCANSCAM_CL_CASE(ST, 2, 8)                                                                 \
             SCANSCAM_CL_CASE(ST, 2, 16)                                                                \
         }                                                                                              \
+        if constexpr (sizeof(ST) <= 4) { /* lanes of 8 bytes: two fp32 channels, four 16-bit ones */   \
+            constexpr int HALF = FULL / 2;                                                             \
+            SCANSCAM_CL_CASE(ST, HALF, 4)                                                              \
+            SCANSCAM_CL_CASE(ST, HALF, 8)                                                              \
+            SCANSCAM_CL_CASE(ST, HALF, 16)                                                             \
+        }                                                                                              \
         return hipErrorInvalidValue;                                                                   \
     }
 

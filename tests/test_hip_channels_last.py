@@ -81,7 +81,8 @@ def test_forced_plans(gpu, dtype):
         ga, gb = oracle.bwd(as_rows(a), as_rows(hs), as_rows(gh))
         cases.append((shape, a.to(gpu), b.to(gpu), gh.to(gpu), hs.to(gpu), h, ga, gb, prev_abs(as_rows(hs))))
     n = 0
-    for vec in ((full, 2, 1) if full == 8 else (full, 1)):  # 16-bit storage also has lanes of two channels
+    # Lanes of 16 bytes, of 8 bytes (two fp32 channels, four 16-bit ones), of two 16-bit channels, of one channel.
+    for vec in {8: (8, 4, 2, 1), 4: (4, 2, 1), 2: (2, 1)}[full]:
         for steps in ((2, 4, 8) if vec == full else (4, 8, 16)):
             csize = 8 if dtype == torch.float64 else 4
             max_waves = min(16, 65536 // (4 * vec * 64 * csize), (512 if (vec > 1 and steps >= 8) else 1024) // 64)
@@ -101,7 +102,7 @@ def test_forced_plans(gpu, dtype):
                     assert rel_err(as_rows(got_gb), gb) <= bar, (plan, shape)
                     assert rel_err(as_rows(got_ga), ga, hp) <= bar, (plan, shape)
                     n += 1
-    assert n > 60
+    assert n > 90
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16, torch.float16])
@@ -127,7 +128,7 @@ def test_element_aligned_lanes(gpu, dtype):
                 v.copy_(t)
                 return v
             da, db, dgh, dhs = view_of(a), view_of(b), view_of(gh), view_of(hs)
-            for vec in ((full, 2) if full == 8 else (full,)):
+            for vec in {8: (8, 4, 2), 4: (4, 2), 2: (2,)}[full]:
                 if shape[-1] < 64 * vec:
                     continue
                 for steps in ((2, 4, 8) if vec == full else (4, 8, 16)):
@@ -284,6 +285,14 @@ MANY_WORKGROUPS = [
     (torch.bfloat16, (257, 64, 256), None),
     (torch.bfloat16, (9, 3000, 64), None),      # the same with time split over workgroups
     (torch.bfloat16, (16, 1100, 1024), None),
+    (torch.float32, (260, 60, 256), None),      # 8-byte lanes: chosen ahead of 16-byte lanes ...
+    (torch.bfloat16, (130, 70, 1024), None),
+    (torch.float32, (130, 70, 512), None),      # ... and where only they and narrower ones give 256 workgroups
+    (torch.float16, (64, 100, 1016), None),
+    (torch.bfloat16, (64, 90, 1001), None),     # element-aligned 8-byte lanes (16-byte ones: 128 workgroups)
+    (torch.float32, (70, 50, 501), None),
+    (torch.float32, (8, 2100, 512), None),      # time split over workgroups: 8-byte lanes forwards (fp32) ...
+    (torch.bfloat16, (8, 1500, 1024), None),    # ... and backwards (16-bit storage)
 ]
 
 
