@@ -650,6 +650,15 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         // instruction, against 33 / 29 %).
         if (esize == 2 && C > 32 && C < (int64_t)kWave * full) l->vec = (C == kWave || !pair_possible) ? 1 : 2;
     }
+    // fp32 with fewer than 128 channels and a workgroup per batch element: pairs of channels (8-byte lanes) with 8
+    // steps per wave, whether a time step fills a wave or several steps share one; a single channel per lane
+    // at exactly 64. Against 16-byte lanes with 4 steps: [2048, 512, 40] 41 / 56 -> 56 / 56 % of peak, [1024, 1024, 48]
+    // 47 / 59 -> 60 / 59 %, [512, 2048, 96] 54 / 61 -> 64 / 64 %, [256, 4096, 64] 60 / 68 -> 73 / 67 %; against single
+    // channels with 4 steps: [4096, 1024, 8] 63 / 65 -> 73 / 72 %.
+    if (!u.vec && esize == 4 && C < 2 * kWave && batch >= 256 && u.mode != kModeLookback) {
+        if (C == kWave) l->vec = 1;
+        else if (half_possible) l->vec = 2;
+    }
     if (l->vec != 1 && l->vec != full && !(l->vec == 2 && esize == 2) && !(half > 1 && l->vec == half)) return SCANSCAM_EPLAN;
     // A forced wide lane that the alignment or C does not allow as it stands: element-aligned, where that kernel applies.
     if (u.vec && ((l->vec == full && full > 1 && !vec_possible) || (l->vec == 2 && esize == 2 && full != 2 && !pair_possible) ||
@@ -695,7 +704,9 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // (element-aligned pairs of 16-bit channels likewise: bf16 [64, 2048, 1001] 36 / 34 -> 39 / 38 % of peak)
     const bool long_steps = l->kind != 0 || (esize == 2 && l->vec <= 2 && T >= 1024 && (rowgroups < 512 || (l->ragged && l->vec == 2)));
     l->steps = u.unroll ? u.unroll : (narrow_lane ? (long_steps ? 16 : 8) : ((l->kind != 0 && full <= 4) ? 8 : 4));
-    if (!u.unroll && l->group <= 16 && narrow_lane) l->steps = 4;  // packed, 4 or more steps per instruction
+    // Packed, 4 or more steps per instruction: 4 instructions per wave with one channel per lane; lanes of two
+    // channels keep 8 (bf16 [4096, 1024, 8] 41 / 41 -> 47 / 60 % of peak, [512, 4096, 24] 31 / 33 -> 37 / 44 %).
+    if (!u.unroll && l->group <= 16 && l->vec == 1) l->steps = 4;
     const bool steps_ok = (l->vec == full) ? (l->steps == 2 || l->steps == 4 || l->steps == 8)
                                            : (l->steps == 4 || l->steps == 8 || l->steps == 16);
     if (!steps_ok) return SCANSCAM_EPLAN;

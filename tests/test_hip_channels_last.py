@@ -291,6 +291,12 @@ MANY_WORKGROUPS = [
     (torch.float16, (64, 100, 1016), None),
     (torch.bfloat16, (64, 90, 1001), None),     # element-aligned 8-byte lanes (16-byte ones: 128 workgroups)
     (torch.float32, (70, 50, 501), None),
+    (torch.float32, (300, 100, 40), None),      # fp32 below 128 channels: pairs of channels, 8 steps per wave ...
+    (torch.float32, (257, 64, 96), None),
+    (torch.float32, (300, 200, 8), None),
+    (torch.float32, (260, 90, 64), None),       # ... one channel per lane at exactly 64
+    (torch.bfloat16, (300, 200, 8), None),      # 16-bit pairs, several time steps per instruction, 8 instructions
+    (torch.float16, (300, 100, 24), None),
     (torch.float32, (8, 2100, 512), None),      # time split over workgroups: 8-byte lanes forwards (fp32) ...
     (torch.bfloat16, (8, 1500, 1024), None),    # ... and backwards (16-bit storage)
 ]
