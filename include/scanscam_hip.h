@@ -67,7 +67,7 @@ enum {
  * family on a small input. Zero in any field means "choose for me".
  *   vec            elements per lane per load: 16/sizeof(storage) or 1
  *   unroll         64-lane chunks per wave per tile: 1, 2, 3, 4 or 8 (1 or 4 when vec == 1)
- *   waves          waves per workgroup, 1..16 (at most 4 when unroll == 8)
+ *   waves          waves per workgroup, 1..16 (at most 8 when unroll == 8)
  *   waves_per_row  ROW only: a divisor of `waves` (waves / waves_per_row rows share a workgroup)
  *   spin_limit     kernels that wait for another workgroup's carry poll at most this many times
  *                  (0 = 2^20, about a second); a wait that expires sets word 1 of the workspace to 1

@@ -308,6 +308,13 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
         // 2^26 fp32 elements; from 12 rows on the 32-chunk tile is 4 to 6 points faster).
         l.unroll = u.unroll ? u.unroll : 4;
         l.waves = u.waves ? u.waves : (rows <= 8 && l.unroll <= 4 ? 16 : 8);
+        // Forward fp32 with up to 16 rows: the 64-chunk tile as 8 waves of 8 chunks (two workgroups per CU
+        // instead of one of 16 waves): [1, 2^26] 61 -> 64 % of peak, [16, 2^22] 64 -> 66 %, [8, 2^21] 53 -> 57 %;
+        // backward and 16-bit storage gain nothing from it.
+        if (!u.waves && !u.unroll && !rev && esize == 4 && l.vec == full && !l.ragged && rows <= 16) {
+            l.unroll = 8;
+            l.waves = 8;
+        }
         if (!u.waves && !u.unroll && rows > 8) {
             // As many tiles as 8-wave tiles would take, but with only the waves they need: 75 chunks are 3
             // tiles of 7 waves (84 chunk slots), not of 8 (96).

@@ -25,7 +25,7 @@ struct Launch {
 };
 
 // Largest workgroup (threads) a kernel with U chunks per wave is compiled for.
-constexpr int max_threads_for_unroll(int unroll) { return unroll <= 4 ? 1024 : 256; }
+constexpr int max_threads_for_unroll(int unroll) { return unroll <= 4 ? 1024 : 512; }
 
 // Launches `kernel(args)` and returns what the launch call itself returns (the runtime's sticky "last error" is
 // neither read nor cleared, so an error the host application left there is not taken for this launch's, and

@@ -79,7 +79,7 @@ def test_argument_errors_are_reported_before_any_launch():
     assert L.scanscam_scan_fwd(fake, fake, fake, 4, 1 << 20, 0, fake, 64, None) == E_WORKSPACE
     # Bad explicit plans.
     for bad in (hip.Plan(mode=9), hip.Plan(vec=3), hip.Plan(mode=hip.MODE_ROW, unroll=5),
-                hip.Plan(mode=hip.MODE_ROW, unroll=8, waves=8), hip.Plan(mode=hip.MODE_ROW, waves=4, waves_per_row=3),
+                hip.Plan(mode=hip.MODE_ROW, unroll=8, waves=9), hip.Plan(mode=hip.MODE_ROW, waves=4, waves_per_row=3),
                 hip.Plan(mode=hip.MODE_SMALL), hip.Plan(waves=17)):
         rc = L.scanscam_scan_fwd_plan(fake, fake, fake, 4, 4096, 0, None, 0, None, ctypes.byref(bad))
         assert rc == E_PLAN, bad

@@ -237,7 +237,7 @@ def plans_for(dtype):
     for vec in (full, 1):
         unrolls = (1, 2, 4, 8) if vec == full else (1, 4)
         for unroll in unrolls:
-            max_waves = 16 if unroll <= 4 else 4
+            max_waves = 16 if unroll <= 4 else 8
             for waves in sorted({1, 4, max_waves}):
                 for wpr in sorted({1, 2, waves} & {1, 2, 4, 8, 16}):
                     if waves % wpr == 0:
@@ -376,6 +376,7 @@ AUTO_REGIMES = [
     (512, 140000, (ROW, 16, 4), None),        # 18 tiles per row in full rounds: the row kernel
     (300, 16640, (ROW, 9, 4), None),          # few rows, 65 chunks: 2 steps of 9 waves
     (255, 16640, (LOOKBACK, 0, 4), None),     # fewer than 256 rows: tiles in tile-major order
+    (12, 300000, (LOOKBACK, 0, 8), (LOOKBACK, 0, 4)),  # up to 16 rows: forward tiles of 8 waves x 8 chunks
 ]
 
 
