@@ -160,9 +160,10 @@ int scanscam_scan_bwd_timed(const void *a, const void *h, const void *gh, void *
  * src/scanscam_cuda.cu:556-582, and transposed_linear_scan_backward(gate,
  * output, outGrad, gateGradOut, valueGradOut, channelsPerBlock), :687-723. The
  * reference's trailing tuning argument has its counterpart in `plan` (NULL =
- * automatic): vec = channels per lane (16/sizeof(storage) or 1; also 2 for
- * 16-bit storage), unroll = time
- * steps per wave per tile (2, 4, 8 for the full vector; 4, 8, 16 for vec 1;
+ * automatic): vec = channels per lane (16/sizeof(storage) or 1; also half of
+ * the former, an 8-byte lane, for fp32 and 16-bit storage, and 2 for 16-bit
+ * storage), unroll = time
+ * steps per wave per tile (2, 4, 8 for the full vector; 4, 8, 16 for narrower lanes;
  * with at most 32 * vec channels a wave holds several time steps per load and
  * `unroll` counts those loads), waves = waves per workgroup (1..16). When
  * batch * C is too small to fill the
