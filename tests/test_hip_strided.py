@@ -221,6 +221,22 @@ def test_channels_last_batch_slices_and_lookback(gpu):
         check_forward_backward(a, b, gh, plan=plan, layout="cl")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_channels_last_views_on_the_8_byte_grid(gpu, dtype):
+    """Views whose starts and strides are multiples of 8 bytes but not of 16: lanes of 8 bytes are the widest that fit."""
+    half = 8 // torch.empty(0, dtype=dtype).element_size()   # channels of an 8-byte lane
+    for B, T, C, forced in [(260, 40, 64 * half, None), (3, 300, 64 * half, hip.Plan(mode=hip.MODE_LOOKBACK, vec=half)),
+                            (2, 70, 128 * half + half, hip.Plan(mode=hip.MODE_ROW, vec=half, unroll=8, waves=3))]:
+        width = 2 * C + 3 * half   # time stride: a multiple of 8 bytes, not of 16
+        x = randn(gpu, (B, T, width), B + T + C, dtype)
+        x[..., half:half + C] = torch.sigmoid(x[..., half:half + C].float()).to(dtype)
+        a, b = x[..., half:half + C].mT, x[..., half + C:half + 2 * C].mT   # start 8 bytes into a time step
+        assert a.data_ptr() % 16 == 8 and (a.stride(-1) * x.element_size()) % 16 == 8
+        gh = randn(gpu, (B, T, C), 5, dtype).mT
+        print(f"case strided channels-last 8-byte grid B={B} T={T} C={C} {dtype} {forced}", flush=True)
+        check_forward_backward(a, b, gh, dtype, plan=forced, layout="cl")
+
+
 def test_channels_last_gradient_of_another_layout_is_converted(gpu):
     a = randn(gpu, (2, 50, 70), 41, gate=True).mT
     b = randn(gpu, (2, 50, 70), 42).mT
