@@ -299,6 +299,7 @@ MANY_WORKGROUPS = [
     (torch.float16, (300, 100, 24), None),
     (torch.float32, (8, 2100, 512), None),      # time split over workgroups: 8-byte lanes forwards (fp32) ...
     (torch.bfloat16, (8, 1500, 1024), None),    # ... and backwards (16-bit storage)
+    (torch.float16, (8, 1100, 2048), None),     # 256 workgroups of single channels forwards, tiles of four-channel lanes backwards
 ]
 
 
