@@ -632,8 +632,13 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         // win: more, narrower carry chains (fp32 1.1-1.7 times faster than 16-byte lanes, measured from
         // [1, 262144, 256] to [8, 4096, 512]; 16-bit storage 2.5-16 times, its 16-byte lanes leave
         // 8 times fewer chains).
-        l->vec = batch * groups(full) >= 256 ? full : narrow;
-        // 8-byte lanes, where they still give 256 workgroups and fill their waves to three quarters: they
+        // A lane width whose last channel group is partly empty moves fewer bytes per workgroup in the same time
+        // (the kernels run at 1 / fill of their speed: fp32 C = 320, 83 % fill in pairs and 63 % in fours, 199 / 338 us
+        // and 225 / 375 us against 179 / 316 us with single channels), so a wider lane has to fill its groups
+        // within 5 % of the narrow one.
+        auto fills = [&](int vec) { return 21 * groups(narrow) * narrow >= 20 * groups(vec) * vec; };
+        l->vec = (batch * groups(full) >= 256 && fills(full)) ? full : narrow;
+        // 8-byte lanes, where they still give 256 workgroups and fill their waves as well: they
         // stream as fast as 16-byte lanes or faster at equal shapes (two or four times the waves per byte in
         // flight: fp32 [256, 1024, 1024] 71 / 76 -> 80 / 74 % of peak, [128, 2048, 512] 72 / 70 -> 78 / 75 %, bf16
         // [256, 1024, 1024] 69 / 68 -> 75 / 74 %, [160, 2048, 1024] 59 / 57 -> 70 / 69 %) and reach shapes where 16-byte
@@ -641,8 +646,8 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         // 73 / 78 %, [64, 2048, 512] 67 / 66 -> 75 / 70 %, bf16 [32, 4096, 2048] 66 / 62 -> 69 / 72 %).
         // (Time steps that are not whole 128-byte lines keep 16-byte lanes where those give 256 workgroups:
         // fp32 [64, 2048, 1016] backward 57 % against 50 %.)
-        if (half_possible && C >= (int64_t)kWave * half && C * 4 >= groups(half) * kWave * half * 3 &&
-            batch * groups(half) >= 256 && (l->vec != full || (C * esize) % 128 == 0))
+        if (half_possible && C >= (int64_t)kWave * half && fills(half) && batch * groups(half) >= 256 &&
+            (l->vec != full || (C * esize) % 128 == 0))
             l->vec = half;
         // Few channels (the packed kernel, below): a wide lane leaves more steps per instruction to scan
         // across with lane shuffles, which costs more than the wider loads gain -- except where C is not a
@@ -681,6 +686,18 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     l->kind = 0;
     if (u.mode == kModeLookback || (u.mode == SCANSCAM_MODE_AUTO && rowgroups < 256)) l->kind = 2;
     if (u.mode == kModeSmall) return SCANSCAM_EPLAN;
+    // A few more than 256 workgroups (up to 340) leave some CUs with twice the work of the others. Tiles over
+    // workgroups are taken instead, with the lanes that measure best there in each direction (below): fp32
+    // [20, 4096, 2048] forward 430 -> 354 us, [24, 2048, 1536] 194 / 360 -> 170 / 273 us, [68, 2048, 512] forward 183 ->
+    // 153 us, bf16 [24, 2048, 3072] backward 374 -> 305 us, [12, 4096, 3072] 231 / 399 -> 191 / 286 us. Exactly 256
+    // workgroups are one per CU, and from 350 on the walk is the faster one.
+    const bool few_too_many = l->kind == 0 && !u.vec && u.mode == SCANSCAM_MODE_AUTO && !l->ragged && rowgroups > 256 &&
+                              rowgroups < 340 && groups(l->vec) > 1 && T >= 1024;
+    if (few_too_many) {
+        l->kind = 2;
+        l->vec = narrow;
+        rowgroups = batch * groups(narrow);
+    }
     // Tiles over workgroups, lanes chosen here: 8-byte lanes where C fills whole waves of them, in the
     // direction in which they measured faster than the narrow lane (16 steps per wave either way) -- the
     // backward pass of 16-bit storage (bf16 [8, 4096, 512] 48 -> 38 us, [8, 4096, 2048] 166 -> 140 us,

@@ -300,6 +300,9 @@ MANY_WORKGROUPS = [
     (torch.float32, (8, 2100, 512), None),      # time split over workgroups: 8-byte lanes forwards (fp32) ...
     (torch.bfloat16, (8, 1500, 1024), None),    # ... and backwards (16-bit storage)
     (torch.float16, (8, 1100, 2048), None),     # 256 workgroups of single channels forwards, tiles of four-channel lanes backwards
+    (torch.float32, (36, 1100, 512), None),     # 288 workgroups of 8-byte lanes: tiles over workgroups instead
+    (torch.bfloat16, (36, 1100, 1024), None),
+    (torch.float32, (260, 50, 320), None),      # lanes that would leave their last group half empty: single channels
 ]
 
 
