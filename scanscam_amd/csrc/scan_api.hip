@@ -598,8 +598,13 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     const int half = esize <= 4 ? full / 2 : 0;
     const bool half_possible = half > 0 && align >= 8 && (C % half == 0);
     auto groups = [&](int vec) { return (C + (int64_t)kWave * vec - 1) / ((int64_t)kWave * vec); };
-    // Pairs halve the number of workgroups: not where single channels just reach 256 of them and pairs do not.
-    const int narrow = pair_possible && (batch * groups(2) >= 256 || batch * groups(1) < 256) ? 2 : 1;
+    // Workgroups that lanes of 4 or 8 bytes need before a workgroup walks all of T with them: three quarters of
+    // the CUs (two thirds backwards), not all 256 -- at 176 to 255 workgroups they still beat twice as many
+    // workgroups of the next narrower lane (fp32 [28, 4096, 1024] 287 / 473 -> 261 / 388 us, [24, 4096, 1024] 261 / 442 ->
+    // 228 / 361 us, bf16 [28, 4096, 2048] 300 / 513 -> 278 / 430 us, [56, 2048, 512] forward 81 -> 70 us).
+    const int64_t enough = rev ? 168 : 192;
+    // Pairs halve the number of workgroups: not where single channels reach 256 of them and pairs fall short.
+    const int narrow = pair_possible && (batch * groups(2) >= enough || batch * groups(1) < 256) ? 2 : 1;
     // Element-aligned lanes: where C is no multiple of the lane's channels, or the tensors are only element-aligned,
     // wider lanes are still possible in the kernel in which a workgroup walks all of T -- vectors loaded and
     // stored at element alignment, the last lane of a time step on the window of channels that ends with it.
@@ -646,8 +651,13 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         // 73 / 78 %, [64, 2048, 512] 67 / 66 -> 75 / 70 %, bf16 [32, 4096, 2048] 66 / 62 -> 69 / 72 %).
         // (Time steps that are not whole 128-byte lines keep 16-byte lanes where those give 256 workgroups:
         // fp32 [64, 2048, 1016] backward 57 % against 50 %.)
-        if (half_possible && C >= (int64_t)kWave * half && fills(half) && batch * groups(half) >= 256 &&
-            (l->vec != full || (C * esize) % 128 == 0))
+        // (16-bit storage keeps 256 for its four-channel lanes: bf16 [28, 4096, 2048] gains with 224 workgroups of
+        // them, [72, 2048, 768] loses 15 % with 216.)
+        // (And the backward pass of fp32 with 2048 or more channels, where 16-byte lanes give 256 workgroups:
+        // [32, 2048, 2048] 437 us against 505-530 us, [40, 4096, 2048] level.)
+        if (half_possible && C >= (int64_t)kWave * half && fills(half) &&
+            batch * groups(half) >= (esize == 2 ? 256 : enough) && (l->vec != full || (C * esize) % 128 == 0) &&
+            !(l->vec == full && esize == 4 && rev && C >= 2048))
             l->vec = half;
         // Few channels (the packed kernel, below): a wide lane leaves more steps per instruction to scan
         // across with lane shuffles, which costs more than the wider loads gain -- except where C is not a
@@ -660,7 +670,18 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         // channels (a full wave: 61 / 62 %), two otherwise (66 / 68 % at 256 channels; 47 / 48 % at 96, where single
         // channels would split a step into a full and a half-empty wave: 33 / 31 %; 46 / 46 % at 56, two steps per
         // instruction, against 33 / 29 %).
-        if (esize == 2 && C > 32 && C < (int64_t)kWave * full) l->vec = (C == kWave || !pair_possible) ? 1 : 2;
+        if (esize == 2 && C > 32 && C < (int64_t)kWave * full) {
+            l->vec = (C == kWave || !pair_possible) ? 1 : 2;
+            // Measured later, over rotated buffers at 512 or more batch elements: 129 to 256 channels fill one wave
+            // of four-channel lanes, and a batch element is then one workgroup's contiguous block (C = 200: 201 / 376
+            // -> 121 / 248 us, C = 256: 147 / 261 -> 141 / 249 us); 320 or 448 channels are whole waves of single
+            // channels but leave the last wave of pairs half empty (C = 320: 215 / 358 -> 186 / 353 us, C = 448: 302 /
+            // 504 -> 264 / 494 us); at exactly 64 channels the backward pass is faster in pairs (98 -> 70 us).
+            // (pairs that fill their two waves keep them: C = 256 at 256 batch elements 73 / 128 us against 87 / 137 us)
+            if (C > 2 * kWave && C <= 4 * kWave && C % (2 * kWave) != 0 && half_possible && batch >= 384) l->vec = half;
+            else if (C > 4 * kWave && C % kWave == 0 && C % (2 * kWave) != 0) l->vec = 1;
+            else if (C == kWave && rev && pair_possible && batch >= 256) l->vec = 2;
+        }
     }
     // fp32 with fewer than 128 channels and a workgroup per batch element: pairs of channels (8-byte lanes) with 8
     // steps per wave, whether a time step fills a wave or several steps share one; a single channel per lane
@@ -684,26 +705,41 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // SCANSCAM_MODE_ROW forbids it).
     int64_t rowgroups = batch * groups(l->vec);
     l->kind = 0;
-    if (u.mode == kModeLookback || (u.mode == SCANSCAM_MODE_AUTO && rowgroups < 256)) l->kind = 2;
+    const bool wide_enough = esize == 2 ? l->vec == 2 : l->vec > 1;  // pairs of 16-bit channels, 8- or 16-byte fp32 lanes
+    if (u.mode == kModeLookback || (u.mode == SCANSCAM_MODE_AUTO && rowgroups < (wide_enough ? enough : 256))) l->kind = 2;
     if (u.mode == kModeSmall) return SCANSCAM_EPLAN;
     // A few more than 256 workgroups (up to 340) leave some CUs with twice the work of the others. Tiles over
     // workgroups are taken instead, with the lanes that measure best there in each direction (below): fp32
     // [20, 4096, 2048] forward 430 -> 354 us, [24, 2048, 1536] 194 / 360 -> 170 / 273 us, [68, 2048, 512] forward 183 ->
     // 153 us, bf16 [24, 2048, 3072] backward 374 -> 305 us, [12, 4096, 3072] 231 / 399 -> 191 / 286 us. Exactly 256
     // workgroups are one per CU, and from 350 on the walk is the faster one.
+    // (The same one round later: 520 workgroups are 2.03 rounds. And with few channels, where a batch element is a
+    // workgroup, as long as single channels or pairs fill three quarters of their waves: fp32 [260, 4000, 48]
+    // 207 / 348 -> 139 / 237 us, bf16 204 / 307 -> 108 / 201 us.)
+    const int64_t rounds_up = (rowgroups + kComputeUnits - 1) / kComputeUnits;
     const bool few_too_many = l->kind == 0 && !u.vec && u.mode == SCANSCAM_MODE_AUTO && !l->ragged && rowgroups > 256 &&
-                              rowgroups < 340 && groups(l->vec) > 1 && T >= 1024;
-    if (few_too_many) {
+                              rowgroups * 10 < rounds_up * kComputeUnits * 7 && T >= 1024 &&
+                              C * 4 >= groups(1) * kWave * 3;
+    // (16-bit storage backwards only where four-channel lanes, the ones its tiles need, fill their waves.)
+    // (filling them to 85 %: bf16 C = 1600, 89 %, gains 11 % backwards in such tiles, C = 640, 83 %, loses 8 %)
+    const bool half_fits = half_possible && C >= (int64_t)kWave * half && C * 20 >= groups(half) * kWave * half * 17;
+    // Its pairs make poor tiles backwards, so without four-channel lanes it stays with the walk -- bf16 [300, 2048, 128]
+    // 189 us against 218 us in tiles -- unless the pairs leave most of a wave empty: [260, 4000, 48] 308 -> 201 us in
+    // tiles of single channels.)
+    const bool pairs_fill = groups(2) * kWave * 2 * 7 <= C * 10;
+    if (few_too_many && !(esize == 2 && rev && !half_fits && pairs_fill)) {
         l->kind = 2;
-        l->vec = narrow;
-        rowgroups = batch * groups(narrow);
+        if (l->vec == full && full > 1) l->vec = narrow;
+        // single channels where the lane chosen so far would leave more than 30 % of its waves empty
+        if (groups(l->vec) * kWave * l->vec * 7 > C * 10) l->vec = 1;
+        rowgroups = batch * groups(l->vec);
     }
     // Tiles over workgroups, lanes chosen here: 8-byte lanes where C fills whole waves of them, in the
     // direction in which they measured faster than the narrow lane (16 steps per wave either way) -- the
     // backward pass of 16-bit storage (bf16 [8, 4096, 512] 48 -> 38 us, [8, 4096, 2048] 166 -> 140 us,
     // [1, 262144, 256] 198 -> 167 us; forward 3 to 10 % slower) and the forward pass of fp32
     // ([8, 4096, 512] 47 -> 44 us, [1, 262144, 256] 203 -> 182 us; backward 15 to 25 % slower).
-    if (l->kind == 2 && !u.vec && half_possible && C % ((int64_t)kWave * half) == 0 && (esize == 2 ? rev : !rev)) {
+    if (l->kind == 2 && !u.vec && half_fits && (esize == 2 ? rev : !rev)) {
         l->vec = half;
         rowgroups = batch * groups(half);
     }
@@ -711,8 +747,8 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // 511 workgroups of single-channel lanes walking all of T (a wave's access is 128 bytes there): bf16
     // [4, 8192, 4096] 292 -> 265 us, [2, 16384, 8192] 584 -> 510 us, [16, 4096, 1024] 144 -> 140 us, [8, 4096, 2048]
     // 148-185 -> 150 us over rotated buffers; forwards the single channels are 5 to 20 % faster.
-    if (l->kind == 0 && !u.vec && u.mode == SCANSCAM_MODE_AUTO && esize == 2 && rev && l->vec == 1 && !l->ragged &&
-        half_possible && C % ((int64_t)kWave * half) == 0 && batch * groups(half) < 256 && T >= 1024) {
+    if (l->kind == 0 && !u.vec && u.mode == SCANSCAM_MODE_AUTO && esize == 2 && rev && l->vec <= 2 && !l->ragged &&
+        (l->vec == 1 || rowgroups < 256) && half_fits && batch * groups(half) < 256 && T >= 1024) {
         l->kind = 2;
         l->vec = half;
         rowgroups = batch * groups(half);
@@ -738,6 +774,9 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // (element-aligned pairs of 16-bit channels likewise: bf16 [64, 2048, 1001] 36 / 34 -> 39 / 38 % of peak)
     const bool long_steps = l->kind != 0 || (esize == 2 && l->vec <= 2 && T >= 1024 && (rowgroups < 512 || (l->ragged && l->vec == 2)));
     l->steps = u.unroll ? u.unroll : (narrow_lane ? (long_steps ? 16 : 8) : ((l->kind != 0 && full <= 4) ? 8 : 4));
+    // Tiles of 8-byte fp32 lanes backwards (kept from the choice above where there are a few workgroups too many):
+    // 8 steps, which fit 104 registers where 16 need 129 (fp32 [520, 2000, 96] 504 -> 438 us).
+    if (!u.unroll && l->kind == 2 && esize == 4 && l->vec == 2 && rev) l->steps = 8;
     // Packed, 4 or more steps per instruction: 4 instructions per wave with one channel per lane; lanes of two
     // channels keep 8 (bf16 [4096, 1024, 8] 41 / 41 -> 47 / 60 % of peak, [512, 4096, 24] 31 / 33 -> 37 / 44 %).
     if (!u.unroll && l->group <= 16 && l->vec == 1) l->steps = 4;
@@ -769,6 +808,15 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         if (l->kind == 0 && l->group == kWave && l->vec * esize >= 8 && l->waves > 4 && rowgroups > kComputeUnits) {
             const int64_t rounds = (rowgroups + kComputeUnits - 1) / kComputeUnits;
             if (rowgroups * 100 < rounds * kComputeUnits * 85) l->waves = 4;
+        }
+        // 16-bit storage, a workgroup per batch element or several: 4-wave workgroups for four-channel lanes that
+        // fill one wave per step and for pairs at 64 channels (above), and for the backward pass of single channels
+        // over two or more waves per step (C = 256: 374 -> 296 us, C = 320: 456 -> 353 us; forwards 16 waves are
+        // 5 to 10 % faster).
+        if (l->kind == 0 && esize == 2 && l->waves > 4 && !l->ragged) {
+            if (l->vec == half && l->group == kWave && groups(half) == 1) l->waves = 4;
+            if (l->vec == 2 && C == kWave) l->waves = 4;
+            if (l->vec == 1 && rev && groups(1) >= 2) l->waves = 4;
         }
         while (l->waves > max_waves) l->waves >>= 1;
     }

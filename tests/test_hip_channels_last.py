@@ -303,6 +303,11 @@ MANY_WORKGROUPS = [
     (torch.float32, (36, 1100, 512), None),     # 288 workgroups of 8-byte lanes: tiles over workgroups instead
     (torch.bfloat16, (36, 1100, 1024), None),
     (torch.float32, (260, 50, 320), None),      # lanes that would leave their last group half empty: single channels
+    (torch.float32, (50, 1100, 512), None),     # 200 workgroups of 8-byte lanes are enough for a walk of all of T
+    (torch.float32, (260, 1100, 48), None),     # a workgroup per batch element, a few too many: tiles of single channels
+    (torch.bfloat16, (260, 1100, 48), None),
+    (torch.bfloat16, (400, 60, 200), None),     # 16-bit storage: 129-256 channels in four-channel lanes, 4-wave workgroups
+    (torch.float16, (300, 50, 320), None),      # 320 channels: whole waves of single channels
 ]
 
 
