@@ -617,12 +617,21 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     } else if (!vec_possible) {
         l->vec = narrow;
         if (u.mode != kModeLookback) {
-            if (ragged_fits(full)) {
+            // A lane's fill is C / (groups(vec) * 64 * vec): the wide lanes only where they fill their waves to 65 %,
+            // whole (aligned) 8-byte lanes ahead of element-aligned 16-byte ones where they fill theirs 1.15 times
+            // better, and no element-aligned lane that fills worse than aligned pairs would (fp32 [700, 300, 257]
+            // 221 / 351 -> 179 / 328 us, [90, 2048, 514] 323 / 642 -> 308 / 540 us, bf16 241 / 406 -> 180 / 349 us).
+            auto fills65 = [&](int vec) { return C * 20 >= groups(vec) * kWave * vec * 13; };
+            const bool full_fits = ragged_fits(full) && fills65(full);
+            const bool half_whole = half_possible && ragged_fits(half);
+            const bool half_ragged = half > 1 && !half_possible && ragged_fits(half) && fills65(half) &&
+                                     !(pair_possible && groups(half) * half > groups(2) * 2);
+            if (half_whole && (!full_fits || groups(full) * full * 20 >= groups(half) * half * 23)) {
+                l->vec = half;  // whole 8-byte lanes, nothing element-aligned about them
+            } else if (full_fits) {
                 l->vec = full;
                 l->ragged = true;
-            } else if (half_possible && ragged_fits(half)) {
-                l->vec = half;  // whole 8-byte lanes, nothing element-aligned about them
-            } else if (half > 1 && ragged_fits(half)) {
+            } else if (half_ragged) {
                 l->vec = half;
                 l->ragged = true;
             } else if (esize == 2 && !pair_possible && ragged_fits(2)) {
@@ -653,11 +662,12 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         // fp32 [64, 2048, 1016] backward 57 % against 50 %.)
         // (16-bit storage keeps 256 for its four-channel lanes: bf16 [28, 4096, 2048] gains with 224 workgroups of
         // them, [72, 2048, 768] loses 15 % with 216.)
-        // (And the backward pass of fp32 with 2048 or more channels, where 16-byte lanes give 256 workgroups:
-        // [32, 2048, 2048] 437 us against 505-530 us, [40, 4096, 2048] level.)
+        // (And the backward pass of fp32 with 2048 or more channels, where 16-byte lanes give 256 to 511 workgroups:
+        // [32, 2048, 2048] 437 us against 505-530 us, [40, 4096, 2048] level; with 1024 of them, [64, 512, 4096], the
+        // 8-byte lanes are 7 % ahead again.)
         if (half_possible && C >= (int64_t)kWave * half && fills(half) &&
             batch * groups(half) >= (esize == 2 ? 256 : enough) && (l->vec != full || (C * esize) % 128 == 0) &&
-            !(l->vec == full && esize == 4 && rev && C >= 2048))
+            !(l->vec == full && esize == 4 && rev && C >= 2048 && batch * groups(full) < 512))
             l->vec = half;
         // Few channels (the packed kernel, below): a wide lane leaves more steps per instruction to scan
         // across with lane shuffles, which costs more than the wider loads gain -- except where C is not a
@@ -714,12 +724,11 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // 153 us, bf16 [24, 2048, 3072] backward 374 -> 305 us, [12, 4096, 3072] 231 / 399 -> 191 / 286 us. Exactly 256
     // workgroups are one per CU, and from 350 on the walk is the faster one.
     // (The same one round later: 520 workgroups are 2.03 rounds. And with few channels, where a batch element is a
-    // workgroup, as long as single channels or pairs fill three quarters of their waves: fp32 [260, 4000, 48]
-    // 207 / 348 -> 139 / 237 us, bf16 204 / 307 -> 108 / 201 us.)
+    // workgroup, from 40 channels on (below that several time steps share a wave): fp32 [260, 4000, 48]
+    // 207 / 348 -> 139 / 237 us, bf16 204 / 307 -> 108 / 201 us, fp32 [300, 1000, 77] 113 / 205 -> 93 / 168 us.)
     const int64_t rounds_up = (rowgroups + kComputeUnits - 1) / kComputeUnits;
     const bool few_too_many = l->kind == 0 && !u.vec && u.mode == SCANSCAM_MODE_AUTO && !l->ragged && rowgroups > 256 &&
-                              rowgroups * 10 < rounds_up * kComputeUnits * 7 && T >= 1024 &&
-                              C * 4 >= groups(1) * kWave * 3;
+                              rowgroups * 10 < rounds_up * kComputeUnits * 7 && T >= 512 && C >= 40;
     // (16-bit storage backwards only where four-channel lanes, the ones its tiles need, fill their waves.)
     // (filling them to 85 %: bf16 C = 1600, 89 %, gains 11 % backwards in such tiles, C = 640, 83 %, loses 8 %)
     const bool half_fits = half_possible && C >= (int64_t)kWave * half && C * 20 >= groups(half) * kWave * half * 17;
@@ -727,11 +736,12 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // 189 us against 218 us in tiles -- unless the pairs leave most of a wave empty: [260, 4000, 48] 308 -> 201 us in
     // tiles of single channels.)
     const bool pairs_fill = groups(2) * kWave * 2 * 7 <= C * 10;
-    if (few_too_many && !(esize == 2 && rev && !half_fits && pairs_fill)) {
+    // (With many channel groups per batch element the tiles of pairs win all the same: bf16 [16, 4096, 2050] 572 -> 403 us.)
+    if (few_too_many && !(esize == 2 && rev && !half_fits && pairs_fill && groups(2) < 8)) {
         l->kind = 2;
         if (l->vec == full && full > 1) l->vec = narrow;
-        // single channels where the lane chosen so far would leave more than 30 % of its waves empty
-        if (groups(l->vec) * kWave * l->vec * 7 > C * 10) l->vec = 1;
+        // single channels where the lane chosen so far leaves more than 30 % of its waves empty and they do better
+        if (groups(l->vec) * kWave * l->vec * 7 > C * 10 && groups(l->vec) * l->vec > groups(1)) l->vec = 1;
         rowgroups = batch * groups(l->vec);
     }
     // Tiles over workgroups, lanes chosen here: 8-byte lanes where C fills whole waves of them, in the
@@ -742,6 +752,14 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     if (l->kind == 2 && !u.vec && half_fits && (esize == 2 ? rev : !rev)) {
         l->vec = half;
         rowgroups = batch * groups(half);
+    }
+    // fp32 backwards on time steps that are no whole 128-byte lines: pairs of channels with 8 steps, where they
+    // fill their waves as well as single channels do ([20, 8192, 250] 265 -> 214 us, [48, 2048, 1500] 860 -> 706 us,
+    // [8, 4096, 1000] 178 -> 155 us, [260, 2000, 66] 305 -> 244 us; with whole lines single channels are level or ahead).
+    if (l->kind == 2 && !u.vec && esize == 4 && rev && half_possible && (C * esize) % 128 != 0 &&
+        groups(2) * 2 <= groups(1)) {
+        l->vec = 2;
+        rowgroups = batch * groups(2);
     }
     // The backward pass of 16-bit storage takes the same tiles of four-channel lanes where the alternative is 256 to
     // 511 workgroups of single-channel lanes walking all of T (a wave's access is 128 bytes there): bf16
