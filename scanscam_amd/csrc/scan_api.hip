@@ -310,8 +310,10 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
         l.waves = u.waves ? u.waves : (rows <= 8 && l.unroll <= 4 ? 16 : 8);
         // Forward fp32 with up to 16 rows: the 64-chunk tile as 8 waves of 8 chunks (two workgroups per CU
         // instead of one of 16 waves): [1, 2^26] 61 -> 64 % of peak, [16, 2^22] 64 -> 66 %, [8, 2^21] 53 -> 57 %;
-        // backward and 16-bit storage gain nothing from it.
-        if (!u.waves && !u.unroll && !rev && esize == 4 && l.vec == full && !l.ragged && rows <= 16) {
+        // the backward pass gains nothing from it, 16-bit storage with 2 to 8 rows (bf16 [8, 2^22] 50 -> 43 us,
+        // [4, 2^23] 48 -> 46 us, [2, 2^24] 49 -> 46 us; [1, 2^26] level, [16, 2^21] 47 -> 51 us).
+        if (!u.waves && !u.unroll && !rev && l.vec == full && !l.ragged &&
+            (esize == 4 ? rows <= 16 : (esize == 2 && rows >= 2 && rows <= 8))) {
             l.unroll = 8;
             l.waves = 8;
         }
