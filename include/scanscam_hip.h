@@ -239,6 +239,16 @@ int scanscam_workspace_timed_out(const void *workspace, void *stream, int *timed
 int scanscam_resolve_plan(int64_t rows, int64_t T, int dtype, int direction, const scanscam_plan *plan,
                           scanscam_plan *out);
 
+/*
+ * The same for the channels-last calls on dense [batch, T, C] tensors whose bases are 16-byte
+ * aligned: mode SCANSCAM_MODE_ROW where a workgroup walks all of T, SCANSCAM_MODE_LOOKBACK where
+ * tiles of time steps chain through the workspace; vec channels per lane, unroll time steps per
+ * wave and tile, waves per workgroup. No counterpart in the reference, whose kernel has one launch
+ * shape (scanscam/cuda.py:100-148 passes channels_per_block only).
+ */
+int scanscam_resolve_plan_cl(int64_t batch, int64_t T, int64_t C, int dtype, int direction,
+                             const scanscam_plan *plan, scanscam_plan *out);
+
 /* Static, never-freed description of an error code. */
 const char *scanscam_strerror(int code);
 

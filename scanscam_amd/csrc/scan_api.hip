@@ -628,7 +628,18 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
             const bool half_whole = half_possible && ragged_fits(half);
             const bool half_ragged = half > 1 && !half_possible && ragged_fits(half) && fills65(half) &&
                                      !(pair_possible && groups(half) * half > groups(2) * 2);
-            if (half_whole && (!full_fits || groups(full) * full * 20 >= groups(half) * half * 23)) {
+            // 16-bit storage with 256 to 384 workgroups of 16-byte lanes (one to one and a half per CU): twice as many
+            // of 8-byte lanes, whole or element-aligned, where those fill their waves as well (bf16 [128, 1024, 1003]
+            // 224 / 408 -> 200 / 358 us, [160, 1024, 1003] backward 660 -> 508 us, [128, 1024, 1501] backward 817 -> 557 us,
+            // [128, 1024, 777] 202 / 332 -> 151 / 280 us, [160, 1024, 1004] 271 / 673 -> 251 / 447 us; from 400 workgroups
+            // on the 16-byte lanes are ahead again, and fp32 keeps them throughout).
+            const bool half_instead = esize == 2 && full_fits && batch * groups(full) <= 384 &&
+                                      groups(half) * half <= groups(full) * full &&
+                                      (half_whole || (half > 1 && ragged_fits(half) && fills65(half)));
+            if (half_instead) {
+                l->vec = half;
+                l->ragged = !half_possible;
+            } else if (half_whole && (!full_fits || groups(full) * full * 20 >= groups(half) * half * 23)) {
                 l->vec = half;  // whole 8-byte lanes, nothing element-aligned about them
             } else if (full_fits) {
                 l->vec = full;
@@ -729,8 +740,12 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // workgroup, from 40 channels on (below that several time steps share a wave): fp32 [260, 4000, 48]
     // 207 / 348 -> 139 / 237 us, bf16 204 / 307 -> 108 / 201 us, fp32 [300, 1000, 77] 113 / 205 -> 93 / 168 us.)
     const int64_t rounds_up = (rowgroups + kComputeUnits - 1) / kComputeUnits;
+    // (Up to 0.8 of the rounds they start, from 64 channels on, for the forward pass of fp32 and for lanes of a single
+    // channel -- of 16-bit storage backwards only: fp32 [300, 1024, 256] forward 192 -> 167 us, [400, 1024, 256] 247 ->
+    // 216 us, [150, 2048, 512] 351 -> 324 us, [300, 1000, 77] 112 / 206 -> 92 / 169 us, bf16 backward 147 -> 125 us.)
+    const bool to_08 = C >= 64 && (esize == 4 ? (!rev || l->vec == 1) : (rev && l->vec == 1));
     const bool few_too_many = l->kind == 0 && !u.vec && u.mode == SCANSCAM_MODE_AUTO && !l->ragged && rowgroups > 256 &&
-                              rowgroups * 10 < rounds_up * kComputeUnits * 7 && T >= 512 && C >= 40;
+                              rowgroups * 10 < rounds_up * kComputeUnits * (to_08 ? 8 : 7) && T >= 512 && C >= 40;
     // (16-bit storage backwards only where four-channel lanes, the ones its tiles need, fill their waves.)
     // (filling them to 85 %: bf16 C = 1600, 89 %, gains 11 % backwards in such tiles, C = 640, 83 %, loses 8 %)
     const bool half_fits = half_possible && C >= (int64_t)kWave * half && C * 20 >= groups(half) * kWave * half * 17;
@@ -838,6 +853,12 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
             if (l->vec == 2 && C == kWave) l->waves = 4;
             if (l->vec == 1 && rev && groups(1) >= 2) l->waves = 4;
         }
+        // Element-aligned four-channel lanes of 16-bit storage, more than one and up to two workgroups per CU: 4 waves
+        // (bf16 [128, 1024, 1003] 206 / 370 -> 200 / 358 us, [128, 1024, 777] 175 / 305 -> 151 / 280 us; with one per CU
+        // 8 waves: [64, 2048, 1001] 216 / 386 us against 250 / 434 us).
+        if (l->kind == 0 && esize == 2 && l->ragged && l->vec == half && l->waves > 4 && rowgroups > kComputeUnits &&
+            rowgroups <= 2 * kComputeUnits)
+            l->waves = 4;
         while (l->waves > max_waves) l->waves >>= 1;
     }
     if (l->waves < 1 || l->waves > max_waves) return SCANSCAM_EPLAN;
@@ -1106,6 +1127,28 @@ int scanscam_resolve_plan(int64_t rows, int64_t T, int dtype, int direction, con
     out->unroll = r.l.unroll;
     out->waves = r.l.waves;
     out->waves_per_row = r.l.mode == kModeRow ? r.l.wpr : 0;
+    out->spin_limit = (plan && plan->spin_limit > 0) ? plan->spin_limit : scanscam::kSpinLimit;
+    return SCANSCAM_OK;
+}
+
+int scanscam_resolve_plan_cl(int64_t batch, int64_t T, int64_t C, int dtype, int direction,
+                             const scanscam_plan *plan, scanscam_plan *out)
+{
+    if (!out) return SCANSCAM_EINVAL;
+    const int esize = elem_size(dtype);
+    if (esize == 0) return SCANSCAM_EDTYPE;
+    if (batch <= 0 || T <= 0 || C <= 0 || T >= kMaxT || C >= kMaxT) return SCANSCAM_EINVAL;
+    // Dense tensors on allocation borders: every time step starts on the largest power of two that divides C elements.
+    int align = 16;
+    while (align > esize && !(batch == 1 && T == 1) && (C * esize) % align != 0) align >>= 1;
+    scanscam::ClLaunch l;
+    const int rc = resolve_cl(plan, batch, T, C, dtype, align, direction == SCANSCAM_BACKWARD, &l);
+    if (rc != SCANSCAM_OK) return rc;
+    out->mode = l.kind == 2 ? kModeLookback : kModeRow;
+    out->vec = l.vec;
+    out->unroll = l.steps;
+    out->waves = l.waves;
+    out->waves_per_row = 0;
     out->spin_limit = (plan && plan->spin_limit > 0) ? plan->spin_limit : scanscam::kSpinLimit;
     return SCANSCAM_OK;
 }

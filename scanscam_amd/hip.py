@@ -105,6 +105,8 @@ def _bind(path: str) -> ctypes.CDLL:
     lib.scanscam_workspace_timed_out.restype = i32
     lib.scanscam_resolve_plan.argtypes = [i64, i64, i32, i32, plan_p, plan_p]
     lib.scanscam_resolve_plan.restype = i32
+    lib.scanscam_resolve_plan_cl.argtypes = [i64, i64, i64, i32, i32, plan_p, plan_p]
+    lib.scanscam_resolve_plan_cl.restype = i32
     lib.scanscam_strerror.argtypes = [i32]
     lib.scanscam_strerror.restype = ctypes.c_char_p
     lib.scanscam_abi_version.argtypes = []
@@ -425,6 +427,16 @@ def workspace_bytes_cl(batch: int, T: int, C: int, dtype: torch.dtype, direction
     if plan is None:
         return _workspace_bytes_cl_auto(batch, T, C, _dtype_code(dtype), direction)
     return int(lib().scanscam_workspace_bytes_cl(batch, T, C, _dtype_code(dtype), direction, ctypes.byref(plan)))
+
+
+def resolve_plan_cl(batch: int, T: int, C: int, dtype: torch.dtype, direction: int = FORWARD,
+                    plan: Optional[Plan] = None) -> Plan:
+    """The plan the channels-last calls would run for dense ``[batch, T, C]`` tensors (no GPU needed)."""
+    out = Plan()
+    rc = lib().scanscam_resolve_plan_cl(batch, T, C, _dtype_code(dtype), direction, _plan_ref(plan), ctypes.byref(out))
+    if rc != 0:
+        raise RuntimeError(f"scanscam_resolve_plan_cl: {strerror(rc)}")
+    return out
 
 
 def _workspace_cl(L, batch: int, T: int, C: int, dtype: torch.dtype, direction: int, plan: Optional[Plan],

@@ -1,0 +1,199 @@
+"""
+Time the library's automatic launch plan for a shape against a set of forced plans.
+
+    python -m scanscam_amd.plan_search rows 8192x4096 2047x16385:bf16 ...
+    python -m scanscam_amd.plan_search cl 8x4096x512:bf16 64x2048x1001 ...
+    python -m scanscam_amd.plan_search --suite cl-a | cl-b | cl-odd | rows-23 | rows-25 | rows-26
+
+``rows`` shapes are contiguous ``[rows, T]`` tensors scanned along ``T`` (the layout of
+``simple_linear_scan`` and its siblings, ``scanscam/cuda.py:28-64`` in the reference), ``cl`` shapes are
+contiguous ``[batch, T, C]`` tensors scanned along ``T`` (``transposed_linear_scan``, ``cuda.py:100-148``).
+dtype is f32 (default), bf16 or f16.
+
+One line per shape and dtype: the automatic plan's forward / backward microseconds and fraction of the 8 TB/s
+HBM peak in algorithmic bytes (3 and 5 elements per scanned element), then the fastest plan of the set for each
+direction, and a mark where the automatic plan (shown in brackets: mode, vec, unroll, waves, waves per row) is
+more than 8 % behind it. The automatic plan is timed first
+and again last and the faster of the two is kept, so that warm-up does not count against it. Buffer sets rotate
+over at least 512 MiB so that the 256 MB Infinity Cache does not serve them. A plan the library rejects for a
+shape is skipped.
+
+The same search serves a caller who wants the best plan for one fixed shape: pass the printed plan to the
+``plan=`` argument of the calls in ``scanscam_amd.hip`` (``struct scanscam_plan`` in the C interface).
+"""
+import argparse
+import sys
+
+import torch
+
+from . import hip
+
+P = hip.Plan
+DTYPES = {"": torch.float32, "f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
+HBM_PEAK_GBPS = 8000.0
+
+SUITES = {
+    "cl-a": ("cl", [(8, 4096, 512), (64, 2048, 1024), (256, 1024, 256), (32, 2048, 2048), (16, 8192, 512),
+                    (128, 1024, 768), (4, 32768, 512), (512, 512, 512), (24, 2048, 1536), (96, 1024, 1280),
+                    (12, 4096, 3072), (2, 65536, 1024), (1024, 256, 384), (48, 4096, 640), (200, 1024, 896),
+                    (20, 8192, 256), (320, 1024, 512), (6, 16384, 2048), (40, 2048, 4096), (700, 512, 192)]),
+    "cl-b": ("cl", [(1024, 1024, 64), (300, 2048, 128), (2000, 128, 256), (64, 512, 4096), (16, 2048, 8192),
+                    (100, 3000, 300), (256, 333, 1000), (512, 700, 200), (28, 4096, 1024), (72, 2048, 768),
+                    (3, 50000, 640), (5, 30000, 1280), (1, 100000, 1024), (150, 1500, 448), (4096, 256, 32),
+                    (260, 4000, 48), (520, 2000, 96), (130, 8000, 64), (66, 3000, 1344), (10, 12000, 1600)]),
+    "cl-odd": ("cl", [(64, 2048, 1001), (256, 1024, 1001), (128, 1024, 1003), (32, 4096, 999), (512, 512, 333),
+                      (300, 1000, 77), (1000, 500, 130), (20, 8192, 250), (48, 2048, 1500), (8, 4096, 1000),
+                      (90, 2048, 514), (700, 300, 257), (16, 4096, 2050), (260, 2000, 66)]),
+}
+
+
+def _row_suite(log_n):
+    n = 1 << log_n
+    lengths = (32, 70, 128, 256, 300, 512, 800, 1024, 1600, 2048, 3000, 4096, 6000, 8192, 10000, 16384, 20000,
+               32768, 50000, 65536, 100000)
+    shapes = [(n // t, t) for t in lengths]
+    shapes += [(n >> 17, 1 << 17), (n >> 18, 1 << 18), (n >> 19, 1 << 19), (n >> 20, 1 << 20), (n >> 22, 1 << 22)]
+    shapes += [(r * n >> 25, t) for r, t in ((131071, 255), (43690, 767), (9999, 3333), (2047, 16385), (513, 65537),
+                                              (70000, 480), (26000, 1290), (7000, 4800), (1200, 28000))]
+    return "rows", [s for s in shapes if s[0] >= 1]
+
+
+for _log_n in (23, 25, 26):
+    SUITES[f"rows-{_log_n}"] = _row_suite(_log_n)
+
+
+def row_plans(dtype, T):
+    """Forced plans for the row layout: workgroups of whole rows, time-split tiles, and for short rows the others."""
+    full = 16 // torch.empty(0, dtype=dtype).element_size()
+    out = [P(mode=hip.MODE_ROW, vec=full, unroll=u, waves=w, waves_per_row=r)
+           for u, w, r in ((4, 4, 1), (4, 4, 4), (2, 4, 1), (4, 8, 8), (4, 16, 16), (2, 8, 8), (4, 4, 2), (1, 4, 1),
+                           (2, 4, 2), (3, 3, 3), (4, 2, 2), (8, 4, 4), (4, 12, 12), (2, 16, 16))]
+    out += [P(mode=hip.MODE_LOOKBACK, vec=full, unroll=u, waves=w)
+            for u, w in ((4, 8), (4, 4), (8, 8), (4, 16), (2, 8), (4, 6))]
+    if T <= 64 * full:
+        out += [P(mode=hip.MODE_SMALL, vec=full, unroll=u, waves=4) for u in (1, 2, 4)]
+        out += [P(mode=hip.MODE_FLAT, vec=full, unroll=4, waves=4), P(mode=hip.MODE_FLAT, vec=full, unroll=2, waves=8)]
+    return out
+
+
+def cl_plans(dtype, C):
+    """Forced plans for channels-last storage: every lane width over a few tile shapes, whole-T walks and time-split tiles."""
+    full = 16 // torch.empty(0, dtype=dtype).element_size()
+    half, narrow = full // 2, (1 if full == 4 else 2)
+    walk, split = hip.MODE_ROW, hip.MODE_LOOKBACK
+    most = 16 if full == 4 else 8  # waves that the kernels' LDS arrays allow with 16-byte lanes
+    out = [P(vec=v, unroll=s, waves=w, mode=walk)
+           for v, s, w in ((full, 4, most), (full, 4, 4), (half, 8, 8), (half, 8, 4), (half, 16, 8), (half, 16, 4),
+                           (narrow, 8, 8 * (3 - narrow)), (narrow, 16, 8), (1, 8, 16)) if C % v == 0]
+    if C % full != 0:  # lanes wider than the channel count divides: taken where a time step fills a wave of them
+        out += [P(vec=v, unroll=s, waves=w, mode=walk)
+                for v, s, w in ((full, 4, most), (full, 4, 4), (half, 8, 8), (half, 8, 4), (2, 16, 8), (2, 8, 8))
+                if C % v != 0 and C >= 64 * v]
+    out += [P(vec=v, unroll=s, waves=w, mode=split)
+            for v, s, w in ((narrow, 16, 8), (half, 16, 8), (half, 8, 8), (1, 16, 8)) if C % v == 0]
+    return out
+
+
+def _time(calls, reps, warm):
+    n = len(calls)
+    for i in range(max(warm, 1)):
+        calls[i % n]()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for i in range(reps):
+        calls[i % n]()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / reps * 1e3
+
+
+def _short(plan):
+    if plan is None:
+        return "auto"
+    s = f"m{plan.mode} v{plan.vec} u{plan.unroll} w{plan.waves}"
+    return s + (f" r{plan.waves_per_row}" if plan.waves_per_row else "")
+
+
+def search(layout, shape, dtype, reps=24, warm=4, out=sys.stdout, every=False):
+    """Time every plan of the set on ``shape``; returns {direction: (auto_us, best_us, best_plan)}."""
+    dev = torch.device("cuda:0")
+    esize = torch.empty(0, dtype=dtype).element_size()
+    n = 1
+    for d in shape:
+        n *= d
+    nsets = max(1, min(8, -(-(1 << 29) // (6 * n * esize))))
+    g = torch.Generator(device=dev).manual_seed(0)
+    sets = []
+    for _ in range(nsets):
+        a = (0.9 + 0.1 * torch.rand(shape, generator=g, device=dev)).to(dtype)
+        b, gh = (torch.randn(shape, generator=g, device=dev).to(dtype) for _ in range(2))
+        sets.append((a, b, gh, torch.empty_like(a), torch.empty_like(a), torch.empty_like(a)))
+    if layout == "rows":
+        plans, fwd, bwd = row_plans(dtype, shape[-1]), hip.prepare_forward, hip.prepare_backward
+    else:
+        plans, fwd, bwd = cl_plans(dtype, shape[-1]), hip.prepare_forward_cl, hip.prepare_backward_cl
+    times = {"fwd": [], "bwd": []}
+    for plan in [None] + plans + [None]:
+        try:
+            f = [fwd(a, b, h, plan=plan) for a, b, gh, h, ga, gb in sets]
+            f[0]()  # fills h for the backward pass, and shows whether the library takes this plan here
+            r = [bwd(a, h, gh, ga, gb, plan=plan) for a, b, gh, h, ga, gb in sets]
+            r[0]()
+        except RuntimeError:
+            continue
+        times["fwd"].append((_time(f, reps, warm), plan))
+        times["bwd"].append((_time(r, reps, warm), plan))
+    res, text = {}, []
+    if layout == "rows":
+        chosen = [hip.resolve_plan(*shape, dtype, d) for d in (hip.FORWARD, hip.BACKWARD)]
+    else:
+        chosen = [hip.resolve_plan_cl(*shape, dtype, d) for d in (hip.FORWARD, hip.BACKWARD)]
+    for (name, per_elem), auto_plan in zip((("fwd", 3), ("bwd", 5)), chosen):
+        auto = min(t for t, p in times[name] if p is None)
+        best, best_plan = min(times[name], key=lambda tp: tp[0])
+        res[name] = (auto, best, best_plan)
+        frac = per_elem * esize * n / (auto * 1e-6) / 1e9 / HBM_PEAK_GBPS
+        text.append(f"{name} auto [{_short(auto_plan):16s}] {auto:7.1f} us {100 * frac:4.1f} %  best {best:7.1f} {_short(best_plan):16s}"
+                    + (" BEHIND" if auto > 1.08 * best else "       "))
+    label = "x".join(str(d) for d in shape) + ":" + str(dtype).replace("torch.", "")
+    print(f"{layout} {label:26s} {len(times['fwd']) - 2:2d} plans | " + " | ".join(text), file=out, flush=True)
+    if every:
+        for (tf, plan), (tb, _) in zip(times["fwd"], times["bwd"]):
+            print(f"    {_short(plan):18s} fwd {tf:7.1f} us  bwd {tb:7.1f} us", file=out, flush=True)
+    return res
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
+    ap.add_argument("layout", nargs="?", choices=("rows", "cl"))
+    ap.add_argument("shapes", nargs="*", metavar="SHAPE[:dtype]")
+    ap.add_argument("--suite", choices=sorted(SUITES), help="a fixed list of shapes, each in f32 and bf16")
+    ap.add_argument("--reps", type=int, default=24)
+    ap.add_argument("--every", action="store_true", help="also print every plan's timings")
+    args = ap.parse_args(argv)
+    if not hip.has_hip_ops:
+        sys.exit("plan_search: libscanscam_hip.so does not load")
+    if not torch.cuda.is_available():
+        sys.exit("plan_search: no GPU visible")
+    jobs = []
+    if args.suite:
+        layout, shapes = SUITES[args.suite]
+        jobs = [(layout, s, dt) for s in shapes for dt in (torch.float32, torch.bfloat16)]
+    elif args.layout is None:
+        ap.error("give a layout and shapes, or --suite")
+    for spec in args.shapes:
+        shape_s, _, dtype_s = spec.partition(":")
+        shape = tuple(int(v) for v in shape_s.lower().split("x"))
+        if len(shape) != (2 if args.layout == "rows" else 3):
+            ap.error(f"{spec}: a {args.layout} shape has {2 if args.layout == 'rows' else 3} sizes")
+        jobs.append((args.layout, shape, DTYPES[dtype_s]))
+    behind = 0
+    for layout, shape, dtype in jobs:
+        res = search(layout, shape, dtype, reps=args.reps, every=args.every)
+        behind += sum(auto > 1.08 * best for auto, best, _ in res.values())
+    print(f"{2 * len(jobs)} timings, automatic plan more than 8 % behind the set's best in {behind}", flush=True)
+
+
+if __name__ == "__main__":
+    main()

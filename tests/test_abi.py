@@ -32,7 +32,7 @@ def test_library_is_built_and_loads():
 
 def test_every_declared_symbol_is_exported():
     names = declared_functions()
-    assert "scanscam_scan_fwd" in names and "scanscam_scan_bwd" in names and len(names) == 20
+    assert "scanscam_scan_fwd" in names and "scanscam_scan_bwd" in names and len(names) == 21
     raw = ctypes.CDLL(hip.LIB_PATH)
     for name in names:
         assert hasattr(raw, name), f"{name} declared in scanscam_hip.h but not exported"
@@ -189,5 +189,61 @@ def test_every_automatic_plan_is_a_valid_plan():
                         assert 1 <= out.waves <= 16 and out.unroll in (1, 2, 3, 4, 8) and out.mode in (1, 2, 3, 4)
                         if out.mode == 2:
                             assert out.waves_per_row >= 1 and out.waves % out.waves_per_row == 0
+                        checked += 1
+    assert checked > 10000
+
+
+WALK, TILES = hip.MODE_ROW, hip.MODE_LOOKBACK
+
+
+@pytest.mark.parametrize(
+    "shape,dtype,fwd,bwd",
+    [
+        # (mode, channels per lane, time steps per wave, waves) forwards and backwards
+        ((8, 4096, 2048), torch.float32, (WALK, 1, 8, 16), (WALK, 1, 8, 16)),     # 256 workgroups of single channels
+        ((64, 2048, 1024), torch.float32, (WALK, 2, 8, 8), (WALK, 2, 8, 8)),      # 8-byte lanes give 512 workgroups
+        ((8, 4096, 512), torch.float32, (TILES, 2, 16, 8), (TILES, 1, 16, 8)),    # too few for a walk: tiles over time
+        ((8, 4096, 2048), torch.bfloat16, (WALK, 1, 16, 16), (TILES, 4, 16, 8)),
+        ((256, 4096, 64), torch.bfloat16, (WALK, 1, 16, 16), (WALK, 2, 16, 4)),   # 64 channels: a wave of single channels
+        ((128, 1024, 1003), torch.bfloat16, (WALK, 4, 8, 4), (WALK, 4, 8, 4)),    # element-aligned 8-byte lanes, 512 workgroups
+        ((256, 1024, 1001), torch.bfloat16, (WALK, 8, 4, 8), (WALK, 8, 4, 8)),    # ... 16-byte lanes from 400 workgroups on
+        ((96, 1024, 1003), torch.float32, (WALK, 4, 4, 4), (WALK, 4, 4, 4)),      # fp32 keeps its 16-byte lanes
+        ((300, 1024, 256), torch.float32, (TILES, 2, 16, 8), (WALK, 2, 8, 4)),    # 600 workgroups: 0.78 of three rounds
+        ((300, 1000, 77), torch.bfloat16, (WALK, 1, 8, 16), (TILES, 1, 16, 8)),
+        ((2048, 512, 40), torch.float32, (WALK, 2, 8, 8), (WALK, 2, 8, 8)),       # several time steps per instruction
+    ],
+)
+def test_automatic_channels_last_plan_per_regime(shape, dtype, fwd, bwd):
+    for direction, want in ((hip.FORWARD, fwd), (hip.BACKWARD, bwd)):
+        plan = hip.resolve_plan_cl(*shape, dtype, direction)
+        assert (plan.mode, plan.vec, plan.unroll, plan.waves) == want, (direction, plan)
+        ws = hip.workspace_bytes_cl(*shape, dtype, direction)
+        assert (ws > 0) == (want[0] == TILES)
+
+
+def test_every_automatic_channels_last_plan_is_a_valid_plan():
+    # Every plan the channels-last choice arrives at must be one the library accepts when it is forced,
+    # with the workspace the automatic call asks for being enough for it.
+    L = hip.lib()
+    channels = list(range(1, 70)) + [77, 96, 100, 127, 128, 129, 130, 200, 250, 256, 257, 300, 320, 333, 384, 448, 500,
+                                     511, 512, 513, 514, 640, 768, 1000, 1001, 1003, 1004, 1016, 1024, 1280, 1500, 1501,
+                                     2001, 2048, 2050, 4001, 4096, 8192]
+    checked = 0
+    for dtype in (torch.float32, torch.bfloat16, torch.float16, torch.float64):
+        code = hip._dtype_code(dtype)
+        for batch in (1, 8, 36, 64, 100, 128, 160, 256, 300, 400, 1024, 5000):
+            for T in (1, 50, 512, 1024, 4096):
+                for C in channels:
+                    for direction in (hip.FORWARD, hip.BACKWARD):
+                        out, again = hip.Plan(), hip.Plan()
+                        rc = L.scanscam_resolve_plan_cl(batch, T, C, code, direction, None, ctypes.byref(out))
+                        assert rc == 0, (dtype, batch, T, C, direction, hip.strerror(rc))
+                        assert out.mode in (WALK, TILES) and out.unroll in (2, 4, 8, 16) and 1 <= out.waves <= 16
+                        assert out.vec in (1, 2, 4, 8) and out.vec * torch.empty(0, dtype=dtype).element_size() <= 16
+                        rc = L.scanscam_resolve_plan_cl(batch, T, C, code, direction, ctypes.byref(out), ctypes.byref(again))
+                        assert rc == 0, (dtype, batch, T, C, direction, out, hip.strerror(rc))
+                        assert (again.vec, again.unroll, again.waves) == (out.vec, out.unroll, out.waves), (out, again)
+                        need = L.scanscam_workspace_bytes_cl(batch, T, C, code, direction, ctypes.byref(out))
+                        assert need <= hip.workspace_bytes_cl(batch, T, C, dtype, direction), (dtype, batch, T, C, out)
                         checked += 1
     assert checked > 10000

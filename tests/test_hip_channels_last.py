@@ -308,6 +308,12 @@ MANY_WORKGROUPS = [
     (torch.bfloat16, (260, 1100, 48), None),
     (torch.bfloat16, (400, 60, 200), None),     # 16-bit storage: 129-256 channels in four-channel lanes, 4-wave workgroups
     (torch.float16, (300, 50, 320), None),      # 320 channels: whole waves of single channels
+    (torch.bfloat16, (130, 70, 1003), None),    # 16-bit, 260 workgroups of 16-byte lanes: element-aligned 8-byte lanes, 4 waves
+    (torch.float16, (96, 70, 1501), None),      # ... 8 waves (576 workgroups)
+    (torch.bfloat16, (130, 70, 1004), None),    # ... whole 8-byte lanes
+    (torch.float32, (300, 600, 256), None),     # 0.78 of the rounds started: fp32 forwards in tiles over workgroups
+    (torch.float32, (300, 600, 77), None),      # ... single channels in both directions
+    (torch.bfloat16, (300, 600, 77), None),     # ... 16-bit storage backwards only
 ]
 
 

@@ -188,3 +188,24 @@ def test_package_never_imports_the_oracle():
                 text = open(os.path.join(dirpath, f)).read()
                 assert not re.search(r"^\s*(import|from)\s+oracle\b", text, flags=re.M), f
                 assert "scan_oracle" not in text, f
+
+
+def test_plan_search_sets_hold_plans_the_library_knows():
+    # The forced plans of scanscam_amd.plan_search: each is accepted for at least one of the search's own shapes.
+    import ctypes
+
+    from scanscam_amd import plan_search
+
+    L = hip.lib()
+    for dtype in (torch.float32, torch.bfloat16):
+        code = hip._dtype_code(dtype)
+        for plan in plan_search.row_plans(dtype, 64):
+            out = hip.Plan()
+            assert any(L.scanscam_resolve_plan(rows, T, code, hip.FORWARD, ctypes.byref(plan), ctypes.byref(out)) == 0
+                       for rows, T in ((4096, 64), (4096, 4096), (16, 1 << 20))), plan
+        for C in (1001, 1024):
+            for plan in plan_search.cl_plans(dtype, C):
+                out = hip.Plan()
+                assert any(L.scanscam_resolve_plan_cl(batch, 2048, C, code, hip.FORWARD, ctypes.byref(plan), ctypes.byref(out)) == 0
+                           for batch in (8, 512)), (C, plan)
+    assert {"cl-a", "cl-b", "cl-odd", "rows-25"} <= set(plan_search.SUITES)
