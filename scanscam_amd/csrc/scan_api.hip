@@ -675,12 +675,14 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         // fp32 [64, 2048, 1016] backward 57 % against 50 %.)
         // (16-bit storage keeps 256 for its four-channel lanes: bf16 [28, 4096, 2048] gains with 224 workgroups of
         // them, [72, 2048, 768] loses 15 % with 216.)
-        // (And the backward pass of fp32 with 2048 or more channels, where 16-byte lanes give 256 to 511 workgroups:
-        // [32, 2048, 2048] 437 us against 505-530 us, [40, 4096, 2048] level; with 1024 of them, [64, 512, 4096], the
-        // 8-byte lanes are 7 % ahead again.)
+        // (And the backward pass of fp32 with 2048 or more channels: [32, 2048, 2048] 437 us against 505-530 us,
+        // [64, 1024, 2048] 466 against 508 us, [128, 1024, 2048] 911 against 1025 us, [40, 2048, 4096] 1219 against 1276 us;
+        // with 512 or fewer time steps in workgroups of 4 waves (below): [256, 512, 2048] 967 against 1088 us,
+        // [64, 512, 4096] 492 against 508 us, 516 us with 16 waves; rows of 128 steps keep the 8-byte lanes:
+        // [256, 128, 4096] 460 against 495 us.)
         if (half_possible && C >= (int64_t)kWave * half && fills(half) &&
             batch * groups(half) >= (esize == 2 ? 256 : enough) && (l->vec != full || (C * esize) % 128 == 0) &&
-            !(l->vec == full && esize == 4 && rev && C >= 2048 && batch * groups(full) < 512))
+            !(l->vec == full && esize == 4 && rev && C >= 2048 && (batch * groups(full) < 512 || T >= 256)))
             l->vec = half;
         // Few channels (the packed kernel, below): a wide lane leaves more steps per instruction to scan
         // across with lane shuffles, which costs more than the wider loads gain -- except where C is not a
@@ -812,6 +814,11 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // Tiles of 8-byte fp32 lanes backwards (kept from the choice above where there are a few workgroups too many):
     // 8 steps, which fit 104 registers where 16 need 129 (fp32 [520, 2000, 96] 504 -> 438 us).
     if (!u.unroll && l->kind == 2 && esize == 4 && l->vec == 2 && rev) l->steps = 8;
+    // A walk of all of T in 8-byte fp32 lanes forwards, 2048 or more channels: 16 steps per wave ([64, 1024, 2048]
+    // 292 -> 266 us, [256, 512, 2048] 589 -> 525 us, [512, 256, 2048] 561 -> 499 us, [128, 1024, 2048] 586 -> 535 us,
+    // [40, 2048, 4096] 712 -> 658 us, [12, 4096, 8192] 831 -> 774 us; with 1024 channels 16 steps lose as much).
+    const bool wide_rows_fwd = l->kind == 0 && esize == 4 && !rev && half > 1 && l->vec == half && !l->ragged && C >= 2048;
+    if (!u.unroll && wide_rows_fwd) l->steps = 16;
     // Packed, 4 or more steps per instruction: 4 instructions per wave with one channel per lane; lanes of two
     // channels keep 8 (bf16 [4096, 1024, 8] 41 / 41 -> 47 / 60 % of peak, [512, 4096, 24] 31 / 33 -> 37 / 44 %).
     if (!u.unroll && l->group <= 16 && l->vec == 1) l->steps = 4;
@@ -853,6 +860,12 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
             if (l->vec == 2 && C == kWave) l->waves = 4;
             if (l->vec == 1 && rev && groups(1) >= 2) l->waves = 4;
         }
+        // fp32 with 2048 or more channels: the forward pass above in 4-wave workgroups from 4096 channels on
+        // ([24, 2048, 4096] 413 -> 391 us, [16, 2048, 8192] 554 -> 521 us), the backward pass in 16-byte lanes in
+        // 4-wave workgroups up to 512 time steps ([128, 512, 2048] 586 -> 478 us).
+        if (wide_rows_fwd && !u.unroll && C >= 4096 && l->waves > 4) l->waves = 4;
+        if (l->kind == 0 && esize == 4 && rev && l->vec == full && !l->ragged && C >= 2048 && T <= 512 && l->waves > 4)
+            l->waves = 4;
         // Element-aligned four-channel lanes of 16-bit storage, more than one and up to two workgroups per CU: 4 waves
         // (bf16 [128, 1024, 1003] 206 / 370 -> 200 / 358 us, [128, 1024, 777] 175 / 305 -> 151 / 280 us; with one per CU
         // 8 waves: [64, 2048, 1001] 216 / 386 us against 250 / 434 us).

@@ -211,6 +211,8 @@ WALK, TILES = hip.MODE_ROW, hip.MODE_LOOKBACK
         ((300, 1024, 256), torch.float32, (TILES, 2, 16, 8), (WALK, 2, 8, 4)),    # 600 workgroups: 0.78 of three rounds
         ((300, 1000, 77), torch.bfloat16, (WALK, 1, 8, 16), (TILES, 1, 16, 8)),
         ((2048, 512, 40), torch.float32, (WALK, 2, 8, 8), (WALK, 2, 8, 8)),       # several time steps per instruction
+        ((128, 512, 2048), torch.float32, (WALK, 2, 16, 8), (WALK, 4, 4, 4)),     # 2048 or more fp32 channels
+        ((24, 2048, 4096), torch.float32, (WALK, 2, 16, 4), (WALK, 4, 4, 4)),
     ],
 )
 def test_automatic_channels_last_plan_per_regime(shape, dtype, fwd, bwd):

@@ -314,6 +314,8 @@ MANY_WORKGROUPS = [
     (torch.float32, (300, 600, 256), None),     # 0.78 of the rounds started: fp32 forwards in tiles over workgroups
     (torch.float32, (300, 600, 77), None),      # ... single channels in both directions
     (torch.bfloat16, (300, 600, 77), None),     # ... 16-bit storage backwards only
+    (torch.float32, (20, 300, 2048), None),     # fp32, 2048 or more channels: 16 steps per wave forwards, 16-byte lanes backwards
+    (torch.float32, (10, 200, 4096), None),
 ]
 
 
