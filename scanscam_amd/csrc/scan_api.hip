@@ -949,6 +949,17 @@ int run_cl(bool rev, const void *a, const void *x, const void *h, void *y0, void
     bool lines = true;
     for (int k = 0; k < 5; k++) lines = lines && (sT[k] * esize) % 128 == 0 && aligned_to(ptrs[k], 128) && (sB[k] * esize) % 128 == 0;
     args.xcd_order = (!lines && l.grid >= 64) ? 1 : 0;
+    // Lanes of 8 bytes or less whose time steps are no whole lines write partial lines at both ends of every
+    // wave's store; non-temporal stores then cost 20 % of a plain copy's rate and stores left to the caches'
+    // normal policy nothing. Measured on the kernels: 16-bit storage 8 to 35 % faster in both directions (bf16
+    // [90, 2048, 514] 178 / 341 -> 139 / 298 us, [1000, 500, 130] 157 / 296 -> 120 / 202 us, [700, 300, 257] 112 / 217 ->
+    // 85 / 141 us; single channels backwards lose 10 %: [260, 4000, 48]), fp32 forwards and in tiles over workgroups
+    // 4 to 19 % ([8, 4096, 1000] 90 / 152 -> 83 / 128 us, [100, 3000, 300] forward 339 -> 276 us; a walk of all of T
+    // backwards loses up to 11 %); on whole lines they lose 6 to 14 %, and 16-byte lanes lose 6 to 11 % either way.
+    // (Element-aligned lanes of 8 bytes or less always store this way: the kernel's choice, not this flag's.)
+    const int lane_bytes = l.vec * esize;
+    args.cached_stores = (!lines && lane_bytes <= 8 && esize <= 4 &&
+                          (esize == 2 ? (lane_bytes > 2 || !rev) : (!rev || l.kind == 2))) ? 1 : 0;
     args.ws = nullptr;
     args.spin_limit = (plan && plan->spin_limit > 0) ? plan->spin_limit : scanscam::kSpinLimit;
 

@@ -44,6 +44,7 @@ struct ClArgs {
     int32_t segments;   // look-back kernel: tiles per (batch element, channel group)
     int32_t group;      // packed kernel: lanes per time step (power of two below 64)
     int32_t xcd_order;  // scan_cl_kernel, scan_cl_lookback_kernel: consecutive (batch element, channel group) pairs share an XCD
+    int32_t cached_stores;  // outputs through the caches' normal policy instead of non-temporal (the host decides, see run_cl)
     uint64_t *ws;       // look-back kernel: ticket counters + published pairs
     int32_t spin_limit; // look-back kernel: polls before a wait gives up
 };
@@ -60,6 +61,7 @@ template <typename ST> struct ClLane {
     int pa, px, ph, py0, py1;  // elements from one time step to the next, per tensor
     unsigned c;                // byte offset of the lane's first channel (0 for a lane without channels)
     bool c_ok;
+    bool cached;               // ClArgs::cached_stores (the same in every wave of the launch)
     // Element-aligned lanes (RAGGED): C need not be a multiple of the lane's VEC channels, so the last lane of
     // a time step may own fewer. It loads the window of VEC channels that ends with the time step instead
     // (`c` points there) and moves its components down by `shift` places; its stores go out per channel.
@@ -120,6 +122,13 @@ template <typename ST, int VEC> struct ClAccess<ST, VEC, true> {
         else if constexpr (kBytes == 4) return __builtin_amdgcn_raw_buffer_load_b32(r, lane_off, step_off, AUX);
         else return __builtin_amdgcn_raw_buffer_load_b16(r, lane_off, step_off, AUX);
     }
+    static __device__ __forceinline__ void store_cached(raw_t v, Base r, unsigned lane_off, unsigned step_off)
+    {
+        if constexpr (kBytes == 16) __builtin_amdgcn_raw_buffer_store_b128(v, r, lane_off, step_off, 0);
+        else if constexpr (kBytes == 8) __builtin_amdgcn_raw_buffer_store_b64(v, r, lane_off, step_off, 0);
+        else if constexpr (kBytes == 4) __builtin_amdgcn_raw_buffer_store_b32(v, r, lane_off, step_off, 0);
+        else __builtin_amdgcn_raw_buffer_store_b16(v, r, lane_off, step_off, 0);
+    }
     static __device__ __forceinline__ void store(raw_t v, Base r, unsigned lane_off, unsigned step_off)
     {
         if constexpr (kBytes == 16) __builtin_amdgcn_raw_buffer_store_b128(v, r, lane_off, step_off, 2);
@@ -143,6 +152,16 @@ template <typename ST, int VEC> struct ClAccess<ST, VEC, false> {
     static __device__ __forceinline__ void store(raw_t v, Base r, unsigned lane_off, unsigned step_off)
     {
         __builtin_nontemporal_store(v, reinterpret_cast<raw_elem_aligned_t *>(r + step_off + lane_off));
+    }
+    // Through the caches' normal policy. Lanes on their natural alignment take the buffer form: were both forms
+    // plain stores to one address under a run-time choice, the compiler would fold them into one and drop the hint.
+    static __device__ __forceinline__ void store_cached(raw_t v, Base r, unsigned lane_off, unsigned step_off)
+    {
+        ClAccess<ST, VEC, true>::store_cached(v, ClAccess<ST, VEC, true>::base(reinterpret_cast<const ST *>(r)), lane_off, step_off);
+    }
+    static __device__ __forceinline__ void store_cached_elem_aligned(raw_t v, Base r, unsigned lane_off, unsigned step_off)
+    {
+        *reinterpret_cast<raw_elem_aligned_t *>(r + step_off + lane_off) = v;
     }
 };
 
@@ -273,21 +292,41 @@ struct ClSteps {
 
     // A lane's vector to its channels of one time step; the last lane of an element-aligned time step stores
     // the channels it owns one by one (its window started `shift` channels early).
+    // CACHED: through the caches' normal policy instead of non-temporal. Lanes of 8 bytes or less only:
+    // element-aligned ones always (their time steps are never whole lines), the others where the host asks for it.
+    template <bool CACHED>
     static __device__ __forceinline__ void put(raw_t r, Base res, const ClLane<ST> &ln, unsigned off)
     {
         if (!RAGGED || ln.shift == 0) {
-            BV::store(r, res, ln.c, off);
+            if constexpr (RAGGED && sizeof(raw_t) <= 8) BV::store_cached_elem_aligned(r, res, ln.c, off);
+            else if constexpr (CACHED) BV::store_cached(r, res, ln.c, off);
+            else BV::store(r, res, ln.c, off);
         } else if constexpr (RAGGED) {
             using One = ClAccess<ST, 1, false>;
             const Elems<ST, VEC> e = __builtin_bit_cast(Elems<ST, VEC>, r);
 #pragma unroll
             for (int k = 0; k < VEC; k++)
                 if (k < VEC - ln.shift)
-                    One::store(__builtin_bit_cast(typename One::raw_t, e.e[k]), res, ln.c + (unsigned)((ln.shift + k) * sizeof(ST)), off);
+                    if constexpr (sizeof(raw_t) <= 8)
+                        One::store_cached_elem_aligned(__builtin_bit_cast(typename One::raw_t, e.e[k]), res, ln.c + (unsigned)((ln.shift + k) * sizeof(ST)), off);
+                    else
+                        One::store(__builtin_bit_cast(typename One::raw_t, e.e[k]), res, ln.c + (unsigned)((ln.shift + k) * sizeof(ST)), off);
         }
     }
 
+    // One copy of the store loop per policy, chosen once per call (the choice is the same for the whole launch).
     __device__ __forceinline__ void apply(const ClLane<ST> &ln, int T, CT (&mine)[VEC])
+    {
+        if constexpr (!RAGGED && sizeof(raw_t) <= 8) {
+            if (ln.cached) {
+                apply_as<true>(ln, T, mine);
+                return;
+            }
+        }
+        apply_as<false>(ln, T, mine);
+    }
+
+    template <bool CACHED> __device__ __forceinline__ void apply_as(const ClLane<ST> &ln, int T, CT (&mine)[VEC])
     {
         const Base res_y0 = BV::base(ln.y0 + (int64_t)tb * ln.py0), res_y1 = BV::base(ln.y1 + (int64_t)tb * ln.py1);
 #pragma unroll
@@ -302,15 +341,15 @@ struct ClSteps {
                 out[k] = mine[k];
             }
             if (!REV) {
-                if (in && ln.c_ok) put(V::pack(out), res_y0, ln, step_off(t, ln.py0));
+                if (in && ln.c_ok) put<CACHED>(V::pack(out), res_y0, ln, step_off(t, ln.py0));
             } else {
                 CT fh[VEC], ga[VEC];
                 V::unpack(rh[s], fh);
 #pragma unroll
                 for (int k = 0; k < VEC; k++) ga[k] = out[k] * (h_in ? fh[k] : CT(0));
                 if (in && ln.c_ok) {
-                    put(V::pack(out), res_y0, ln, step_off(t, ln.py0));
-                    put(V::pack(ga), res_y1, ln, step_off(t, ln.py1));
+                    put<CACHED>(V::pack(out), res_y0, ln, step_off(t, ln.py0));
+                    put<CACHED>(V::pack(ga), res_y1, ln, step_off(t, ln.py1));
                 }
             }
         }
@@ -375,6 +414,7 @@ __device__ __forceinline__ ClLane<ST> cl_lane(const ClArgs &p, int64_t batch_ind
 {
     const int64_t c0 = ((int64_t)group * kWave + lane) * VEC;  // first channel of this lane
     ClLane<ST> ln;
+    ln.cached = p.cached_stores != 0;
     ln.c_ok = c0 < p.C;
     ln.shift = (RAGGED && ln.c_ok && c0 + VEC > p.C) ? (int)(c0 + VEC - p.C) : 0;  // C >= VEC: the host checks it
     ln.c = ln.c_ok ? (unsigned)((c0 - ln.shift) * sizeof(ST)) : 0u;
