@@ -651,6 +651,23 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
                 l->vec = 2;
                 l->ragged = true;
             }
+            // With their stores left to the caches (below, and in the kernel for element-aligned lanes) the narrower
+            // lanes are ahead wherever they fill their waves 1.1 times better: 8-byte lanes in place of element-aligned
+            // 16-byte ones (fp32 [512, 512, 333] 290 / 469 -> 248 / 390 us, [128, 1024, 601] 249 / 440 -> 230 / 395 us,
+            // [64, 1024, 777] 148 / 246 -> 122 / 238 us), pairs of 16-bit channels in place of four-channel lanes (bf16
+            // [512, 512, 333] 143 / 247 -> 121 / 254 us, [128, 1024, 601] 150 / 253 -> 122 / 235 us).
+            // (1.2 times where the 16-byte lanes give more than 256 workgroups: fp32 [256, 1024, 777], 1.14 times, is
+            // 13 % faster forwards in 16-byte lanes and level backwards.)
+            if (l->vec == full && l->ragged && half > 1 && ragged_fits(half) &&
+                groups(full) * full * 10 >= groups(half) * half * (batch * groups(full) <= 256 ? 11 : 12)) {
+                l->vec = half;
+                l->ragged = !half_possible;
+            }
+            if (esize == 2 && l->vec == half && half > 2 && (pair_possible || ragged_fits(2)) && batch * groups(2) >= 256 &&
+                groups(half) * half * 10 >= groups(2) * 2 * 11) {
+                l->vec = 2;
+                l->ragged = !pair_possible;
+            }
         }
     } else {
         // A workgroup owns 64*vec channels of one batch element. Enough of them: 16-byte loads.
@@ -809,7 +826,9 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // fill such tiles, it costs 2 to 10 points; fp32 gains nothing from it.
     const bool narrow_lane = l->vec < full;
     // (element-aligned pairs of 16-bit channels likewise: bf16 [64, 2048, 1001] 36 / 34 -> 39 / 38 % of peak)
-    const bool long_steps = l->kind != 0 || (esize == 2 && l->vec <= 2 && T >= 1024 && (rowgroups < 512 || (l->ragged && l->vec == 2)));
+    // (and of fp32 channels: [512, 512, 333] backward 502 -> 390 us, [256, 1024, 777] 1246 -> 962 us, [128, 1024, 1003] 747 -> 664 us)
+    const bool long_steps = l->kind != 0 || (esize == 2 && l->vec <= 2 && T >= 1024 && (rowgroups < 512 || (l->ragged && l->vec == 2))) ||
+                            (esize == 4 && l->ragged && l->vec == 2);
     l->steps = u.unroll ? u.unroll : (narrow_lane ? (long_steps ? 16 : 8) : ((l->kind != 0 && full <= 4) ? 8 : 4));
     // Tiles of 8-byte fp32 lanes backwards (kept from the choice above where there are a few workgroups too many):
     // 8 steps, which fit 104 registers where 16 need 129 (fp32 [520, 2000, 96] 504 -> 438 us).
@@ -847,7 +866,9 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         // would be mostly empty (320 workgroups = 1.25 rounds), 4-wave workgroups, several per CU, finish
         // together instead: fp32 [80, 2048, 1024] 445 / 699 us -> 361 / 661 us, [64, 2048, 1032] 494 / 766 ->
         // 413 / 734 us. (16-byte lanes only: narrow lanes need the waves to keep enough bytes in flight.)
-        if (l->kind == 0 && l->group == kWave && l->vec * esize >= 8 && l->waves > 4 && rowgroups > kComputeUnits) {
+        // (Not element-aligned lanes with 16 steps per wave: fp32 [128, 1024, 601] backward 474 us with 4 waves, 395 us with 8.)
+        if (l->kind == 0 && l->group == kWave && l->vec * esize >= 8 && l->waves > 4 && rowgroups > kComputeUnits &&
+            !(l->ragged && l->steps == 16)) {
             const int64_t rounds = (rowgroups + kComputeUnits - 1) / kComputeUnits;
             if (rowgroups * 100 < rounds * kComputeUnits * 85) l->waves = 4;
         }

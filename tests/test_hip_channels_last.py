@@ -314,6 +314,9 @@ MANY_WORKGROUPS = [
     (torch.float32, (300, 600, 256), None),     # 0.78 of the rounds started: fp32 forwards in tiles over workgroups
     (torch.float32, (300, 600, 77), None),      # ... single channels in both directions
     (torch.bfloat16, (300, 600, 77), None),     # ... 16-bit storage backwards only
+    (torch.float32, (260, 70, 333), None),      # lanes that fill their waves better: element-aligned pairs of fp32 channels, 16 steps
+    (torch.bfloat16, (260, 70, 333), None),     # ... element-aligned pairs of 16-bit channels
+    (torch.float16, (130, 1030, 601), None),
     (torch.float32, (20, 300, 2048), None),     # fp32, 2048 or more channels: 16 steps per wave forwards, 16-byte lanes backwards
     (torch.float32, (10, 200, 4096), None),
 ]
