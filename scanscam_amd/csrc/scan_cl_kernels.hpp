@@ -202,6 +202,10 @@ struct ClSteps {
     int tau0;   // scan position of the first step
     int limit;  // scan positions from here on do not exist
     int tb;     // time step the resources' bases point at: no access of this wave lies before it
+    // issue() may run for the next span of steps while the folded one still awaits apply(): what it sets is kept
+    // apart (n_*) until fold() takes it over. The raw gates and values need no second copy, fold() has used them up.
+    raw_t n_rh[(REV && APPLY) ? S : 1];
+    int n_tau0, n_limit, n_tb;
 
     // Byte distance of time step t from the base, for a tensor with `stride` elements per step.
     __device__ __forceinline__ unsigned step_off(int t, int stride) const
@@ -218,12 +222,14 @@ struct ClSteps {
     // Issues every load of the wave's S steps; nothing waits for them here.
     __device__ __forceinline__ void issue(const ClLane<ST> &ln, int T, int first_step, int limit_)
     {
-        tau0 = first_step;
-        limit = limit_;
+        n_tau0 = first_step;
+        n_limit = limit_;
         // Forwards the wave touches times tau0 ... tau0+S-1; backwards T-1-tau for the same tau, plus
         // a[t+1] and h[t-1]: nothing before T-1-(tau0+S-1)-1. Clamped into the tensor.
-        const int lowest = REV ? T - 1 - (tau0 + S - 1) - 1 : tau0;
-        tb = lowest < 0 ? 0 : (lowest > T - 1 ? T - 1 : lowest);
+        const int lowest = REV ? T - 1 - (n_tau0 + S - 1) - 1 : n_tau0;
+        n_tb = lowest < 0 ? 0 : (lowest > T - 1 ? T - 1 : lowest);
+        const int tb = n_tb, tau0 = n_tau0, limit = n_limit;  // this function's own view (step_off below takes tb from here)
+        auto step_off = [tb](int t, int stride) { return (unsigned)(t - tb) * (unsigned)stride * (unsigned)sizeof(ST); };
         const Base res_a = BV::base(ln.a + (int64_t)tb * ln.pa), res_x = BV::base(ln.x + (int64_t)tb * ln.px);
         const Base res_h = BV::base(ln.h + (int64_t)tb * ln.ph);
         // Every load is issued unconditionally (a step that does not exist reads the base): no
@@ -241,7 +247,7 @@ struct ClSteps {
             if (APPLY) {
                 ra[s] = BV::template load<2>(res_a, ln.c, off_a);
                 rx[s] = BV::template load<2>(res_x, ln.c, off_x);
-                if (REV) rh[s] = BV::template load<2>(res_h, ln.c, h_in ? step_off(t - 1, ln.ph) : 0u);
+                if (REV) n_rh[s] = BV::template load<2>(res_h, ln.c, h_in ? step_off(t - 1, ln.ph) : 0u);
             } else {
                 ra[s] = BV::template load<0>(res_a, ln.c, off_a);
                 rx[s] = BV::template load<0>(res_x, ln.c, off_x);
@@ -252,6 +258,13 @@ struct ClSteps {
     // Folds the issued steps to one affine pair per channel (and keeps gate and value per step for apply()).
     __device__ __forceinline__ void fold(int T, CT (&A)[VEC], CT (&B)[VEC], int shift = 0)
     {
+        tau0 = n_tau0;
+        limit = n_limit;
+        tb = n_tb;
+        if (REV && APPLY) {
+#pragma unroll
+            for (int s = 0; s < S; s++) rh[s] = n_rh[s];
+        }
         if (RAGGED && shift != 0) {  // the last lane of a time step: its window's components into place
 #pragma unroll
             for (int s = 0; s < S; s++) {
@@ -356,50 +369,6 @@ struct ClSteps {
     }
 };
 
-// Processes the tile of W*S steps that starts at scan position tile0.
-//   APPLY = true   `run` holds the scan value entering the tile per channel; the
-//                  tile's outputs are stored and `run` advanced to its end.
-//   APPLY = false  `runA`, `run` hold the affine pair of everything folded so
-//                  far; the tile's pair is composed onto it; nothing is stored
-//                  (kept for callers that only need a pair; unused by the kernels here).
-// lds_A / lds_B: [W][VEC][64] values each; the caller alternates two buffers.
-template <typename ST, int VEC, int S, bool REV, bool APPLY, typename CT, bool RAGGED = false>
-__device__ __forceinline__ void cl_tile(const ClLane<ST> &ln, int T, int tile0, int limit, int wave, int W,
-                                        int lane, CT *lds_A, CT *lds_B, CT (&runA)[VEC], CT (&run)[VEC])
-{
-    ClSteps<ST, VEC, S, REV, APPLY, CT, false, RAGGED> steps;
-    CT A[VEC], B[VEC];
-    steps.load_fold(ln, T, tile0 + wave * S, limit, A, B);
-
-    CT mine[VEC];
-#pragma unroll
-    for (int k = 0; k < VEC; k++) mine[k] = run[k];
-    if (W > 1) {
-#pragma unroll
-        for (int k = 0; k < VEC; k++) {
-            lds_A[(wave * VEC + k) * kWave + lane] = A[k];
-            lds_B[(wave * VEC + k) * kWave + lane] = B[k];
-        }
-        __syncthreads();
-        for (int q = 0; q < W; q++) {
-#pragma unroll
-            for (int k = 0; k < VEC; k++) {
-                const CT Aq = lds_A[(q * VEC + k) * kWave + lane], Bq = lds_B[(q * VEC + k) * kWave + lane];
-                if (APPLY && q == wave) mine[k] = run[k];
-                run[k] = fma_(Aq, run[k], Bq);
-                if (!APPLY) runA[k] = Aq * runA[k];
-            }
-        }
-    } else {
-#pragma unroll
-        for (int k = 0; k < VEC; k++) {
-            run[k] = fma_(A[k], run[k], B[k]);
-            if (!APPLY) runA[k] = A[k] * runA[k];
-        }
-    }
-    if (APPLY) steps.apply(ln, T, mine);
-}
-
 // Index r of n, dealt round-robin to the 8 XCDs (r % 8), mapped so that every XCD holds one contiguous run
 // of the n indices: a permutation of 0 ... n-1.
 __device__ __forceinline__ int xcd_contiguous(int r, int n)
@@ -454,14 +423,48 @@ __global__ __launch_bounds__(MAXT) void scan_cl_kernel(const ClArgs p)
     const int tile_steps = W * S;
     const int ntiles = (p.T + tile_steps - 1) / tile_steps;
     const int plane = W * VEC * kWave;  // values per LDS array
-    CT carry[VEC], unused[VEC];
+    CT carry[VEC];
 #pragma unroll
     for (int k = 0; k < VEC; k++) carry[k] = CT(0);
 
+    // AHEAD: the loads of tile it + 1 are issued as soon as tile it is folded, so that they are in flight while the
+    // waves exchange their pairs, wait at the barrier, and compute and store tile it. Both tiles' registers are live
+    // then (the next one's packed gates and values beside this one's unpacked ones): taken for 16-bit storage in
+    // lanes of up to 8 bytes, where the packed half is small and the kernels wait most -- bf16 [64, 2048, 1024]
+    // 151 / 228 -> 129 / 220 us, [32, 2048, 2048] 148 / 231 -> 131 / 222 us, [256, 1024, 1024] backward 447 -> 424 us,
+    // [8, 4096, 2048] forward 93 -> 90 us. fp32 pays 30 to 120 registers for it and is level on average (+28 % to -10 %),
+    // 16-byte lanes of 16-bit storage spill.
+    constexpr bool AHEAD = sizeof(ST) == 2 && VEC <= 4 && VEC * S <= 32;
+    ClSteps<ST, VEC, S, REV, true, CT, false, RAGGED> steps;
+    if (AHEAD) steps.issue(ln, p.T, wave * S, p.T);
     for (int it = 0; it < ntiles; it++) {
-        CT *lds_A = lds + (it & 1) * 2 * plane;
-        cl_tile<ST, VEC, S, REV, true, CT, RAGGED>(ln, p.T, it * tile_steps, p.T, wave, W, lane, lds_A, lds_A + plane,
-                                                   unused, carry);
+        CT *lds_A = lds + (it & 1) * 2 * plane, *lds_B = lds_A + plane;
+        CT A[VEC], B[VEC], mine[VEC];
+        if (!AHEAD) steps.issue(ln, p.T, it * tile_steps + wave * S, p.T);
+        steps.fold(p.T, A, B, ln.shift);
+        if (AHEAD && it + 1 < ntiles) steps.issue(ln, p.T, (it + 1) * tile_steps + wave * S, p.T);
+#pragma unroll
+        for (int k = 0; k < VEC; k++) mine[k] = carry[k];
+        if (W > 1) {
+#pragma unroll
+            for (int k = 0; k < VEC; k++) {
+                lds_A[(wave * VEC + k) * kWave + lane] = A[k];
+                lds_B[(wave * VEC + k) * kWave + lane] = B[k];
+            }
+            __syncthreads();
+            for (int q = 0; q < W; q++) {
+#pragma unroll
+                for (int k = 0; k < VEC; k++) {
+                    const CT Aq = lds_A[(q * VEC + k) * kWave + lane], Bq = lds_B[(q * VEC + k) * kWave + lane];
+                    if (q == wave) mine[k] = carry[k];
+                    carry[k] = fma_(Aq, carry[k], Bq);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < VEC; k++) carry[k] = fma_(A[k], carry[k], B[k]);
+        }
+        steps.apply(ln, p.T, mine);
     }
 }
 
