@@ -697,9 +697,15 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         // with 512 or fewer time steps in workgroups of 4 waves (below): [256, 512, 2048] 967 against 1088 us,
         // [64, 512, 4096] 492 against 508 us, 516 us with 16 waves; rows of 128 steps keep the 8-byte lanes:
         // [256, 128, 4096] 460 against 495 us.)
+        // (16-bit storage likewise from 4096 channels on: bf16 [16, 2048, 8192] backward 548 -> 465 us, [32, 2048, 4096]
+        // 486 -> 448 us, [64, 1024, 4096] 486 -> 462 us; with 2048 channels the four-channel lanes are 10 % ahead, and so
+        // they are with 512 time steps or where the 16-byte lanes' workgroups are no whole rounds of 256:
+        // [64, 512, 4096] 241 against 280 us, [40, 2048, 4096] 645 against 765 us.)
         if (half_possible && C >= (int64_t)kWave * half && fills(half) &&
             batch * groups(half) >= (esize == 2 ? 256 : enough) && (l->vec != full || (C * esize) % 128 == 0) &&
-            !(l->vec == full && esize == 4 && rev && C >= 2048 && (batch * groups(full) < 512 || T >= 256)))
+            !(l->vec == full && esize == 4 && rev && C >= 2048 && (batch * groups(full) < 512 || T >= 256)) &&
+            !(l->vec == full && esize == 2 && rev && C >= 4096 && T >= 1024 &&
+              batch * groups(full) * 10 >= ((batch * groups(full) + kComputeUnits - 1) / kComputeUnits) * kComputeUnits * 9))
             l->vec = half;
         // Few channels (the packed kernel, below): a wide lane leaves more steps per instruction to scan
         // across with lane shuffles, which costs more than the wider loads gain -- except where C is not a
@@ -720,7 +726,9 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
             // channels but leave the last wave of pairs half empty (C = 320: 215 / 358 -> 186 / 353 us, C = 448: 302 /
             // 504 -> 264 / 494 us); at exactly 64 channels the backward pass is faster in pairs (98 -> 70 us).
             // (pairs that fill their two waves keep them: C = 256 at 256 batch elements 73 / 128 us against 87 / 137 us)
-            if (C > 2 * kWave && C <= 4 * kWave && C % (2 * kWave) != 0 && half_possible && batch >= 384) l->vec = half;
+            // (With the next tile's loads issued ahead, four-channel lanes also at exactly 256 channels and from 256
+            // batch elements: bf16 [256, 1024, 256] 72 / 132 -> 72 / 118 us, [512, 1024, 256] 146 / 258 -> 144 / 244 us.)
+            if (C > 2 * kWave && C <= 4 * kWave && half_possible && batch >= 256) l->vec = half;
             else if (C > 4 * kWave && C % kWave == 0 && C % (2 * kWave) != 0) l->vec = 1;
             else if (C == kWave && rev && pair_possible && batch >= 256) l->vec = 2;
         }
@@ -878,7 +886,7 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         // 5 to 10 % faster).
         if (l->kind == 0 && esize == 2 && l->waves > 4 && !l->ragged) {
             if (l->vec == half && l->group == kWave && groups(half) == 1) l->waves = 4;
-            if (l->vec == 2 && C == kWave) l->waves = 4;
+            if (l->vec == 2 && C == kWave && rowgroups >= 2 * kComputeUnits) l->waves = 4;  // ([256, 4096, 64] backward: 220 us with 4 waves, 154 us with 8)
             if (l->vec == 1 && rev && groups(1) >= 2) l->waves = 4;
         }
         // fp32 with 2048 or more channels: the forward pass above in 4-wave workgroups from 4096 channels on
@@ -886,12 +894,6 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         // 4-wave workgroups up to 512 time steps ([128, 512, 2048] 586 -> 478 us).
         if (wide_rows_fwd && !u.unroll && C >= 4096 && l->waves > 4) l->waves = 4;
         if (l->kind == 0 && esize == 4 && rev && l->vec == full && !l->ragged && C >= 2048 && T <= 512 && l->waves > 4)
-            l->waves = 4;
-        // Element-aligned four-channel lanes of 16-bit storage, more than one and up to two workgroups per CU: 4 waves
-        // (bf16 [128, 1024, 1003] 206 / 370 -> 200 / 358 us, [128, 1024, 777] 175 / 305 -> 151 / 280 us; with one per CU
-        // 8 waves: [64, 2048, 1001] 216 / 386 us against 250 / 434 us).
-        if (l->kind == 0 && esize == 2 && l->ragged && l->vec == half && l->waves > 4 && rowgroups > kComputeUnits &&
-            rowgroups <= 2 * kComputeUnits)
             l->waves = 4;
         while (l->waves > max_waves) l->waves >>= 1;
     }

@@ -204,8 +204,8 @@ WALK, TILES = hip.MODE_ROW, hip.MODE_LOOKBACK
         ((64, 2048, 1024), torch.float32, (WALK, 2, 8, 8), (WALK, 2, 8, 8)),      # 8-byte lanes give 512 workgroups
         ((8, 4096, 512), torch.float32, (TILES, 2, 16, 8), (TILES, 1, 16, 8)),    # too few for a walk: tiles over time
         ((8, 4096, 2048), torch.bfloat16, (WALK, 1, 16, 16), (TILES, 4, 16, 8)),
-        ((256, 4096, 64), torch.bfloat16, (WALK, 1, 16, 16), (WALK, 2, 16, 4)),   # 64 channels: a wave of single channels
-        ((128, 1024, 1003), torch.bfloat16, (WALK, 4, 8, 4), (WALK, 4, 8, 4)),    # element-aligned 8-byte lanes, 512 workgroups
+        ((256, 4096, 64), torch.bfloat16, (WALK, 1, 16, 16), (WALK, 2, 16, 8)),   # 64 channels: a wave of single channels
+        ((128, 1024, 1003), torch.bfloat16, (WALK, 4, 8, 8), (WALK, 4, 8, 8)),    # element-aligned 8-byte lanes, 512 workgroups
         ((256, 1024, 1001), torch.bfloat16, (WALK, 8, 4, 8), (WALK, 8, 4, 8)),    # ... 16-byte lanes from 400 workgroups on
         ((96, 1024, 1003), torch.float32, (WALK, 4, 4, 4), (WALK, 4, 4, 4)),      # fp32 keeps its 16-byte lanes
         ((300, 1024, 256), torch.float32, (TILES, 2, 16, 8), (WALK, 2, 8, 4)),    # 600 workgroups: 0.78 of three rounds

@@ -317,6 +317,8 @@ MANY_WORKGROUPS = [
     (torch.float32, (260, 70, 333), None),      # lanes that fill their waves better: element-aligned pairs of fp32 channels, 16 steps
     (torch.bfloat16, (260, 70, 333), None),     # ... element-aligned pairs of 16-bit channels
     (torch.float16, (130, 1030, 601), None),
+    (torch.bfloat16, (260, 130, 256), None),    # 16-bit, 129-256 channels: four-channel lanes, 4 waves
+    (torch.bfloat16, (32, 1100, 4096), None),   # 16-bit, 4096 or more channels: 16-byte lanes backwards
     (torch.float32, (20, 300, 2048), None),     # fp32, 2048 or more channels: 16 steps per wave forwards, 16-byte lanes backwards
     (torch.float32, (10, 200, 4096), None),
 ]
