@@ -4,6 +4,7 @@ with the CPU oracle, through the C ABI. Shapes and the N(0,1) gates follow the
 reference's tests of its transposed kernels (scanscam/cuda_test.py:129-163); the
 oracle sees the same values as contiguous [batch, C, T] arrays.
 """
+import ctypes
 import itertools
 
 import numpy as np
@@ -352,3 +353,75 @@ def test_automatic_plans_on_many_workgroups(gpu, dtype, shape, window):
     got_ga, got_gb = hip.scan_backward(a.mT, hs.mT, gh.mT)
     assert rel_err(as_rows(got_gb.mT), gb) <= bar
     assert rel_err(as_rows(got_ga.mT), ga, prev_abs(as_rows(hs))) <= bar
+
+
+CHANNEL_EDGES = [1, 2, 3, 5, 8, 24, 31, 32, 33, 40, 63, 64, 65, 66, 77, 96, 100, 127, 128, 129, 130, 192, 200, 250, 256,
+                 257, 300, 320, 333, 384, 448, 500, 511, 512, 513, 514, 600, 601, 640, 768, 777, 896, 1000, 1001, 1002,
+                 1003, 1004, 1016, 1024, 1100]
+
+
+@pytest.mark.parametrize("block", range(8))
+def test_random_channels_last_shapes(gpu, block):
+    """
+    Seeded random [batch, T, C] shapes, storage types and windows: batch sizes on both sides of 256 workgroups
+    for every lane width, channel counts on and off every lane's multiple and the 128-byte line, windows of a
+    wider buffer that start at any element. Whatever lies around a window holds NaN, inputs and outputs alike, so a
+    lane that reads or writes a channel it does not own shows either in the result or in the surroundings.
+    """
+    rng = np.random.default_rng(5000 + block)
+    g = torch.Generator().manual_seed(6000 + block)
+    for i in range(24):
+        dtype = [torch.float32, torch.bfloat16, torch.float16, torch.float32, torch.bfloat16, torch.float64][rng.integers(6)]
+        C = int(CHANNEL_EDGES[rng.integers(len(CHANNEL_EDGES))]) if rng.random() < 0.8 else int(rng.integers(1, 1200))
+        regime = rng.integers(3)  # many batch elements and few steps, a few of each, few batch elements and many steps
+        B = int([rng.integers(200, 600), rng.integers(16, 200), rng.integers(1, 16)][regime])
+        budget = (1 << 22) // (B * C)
+        T = int(rng.integers(1, max(2, min([160, 1200, 6000][regime], budget))))
+        first, extra = (int(rng.integers(0, 9)), int(rng.integers(0, 9))) if rng.random() < 0.5 else (0, 0)
+        width = first + C + extra
+        bar = {torch.float32: 1e-5, torch.float64: 1e-13}.get(dtype, 1e-2)
+        print(f"case cl random block={block} i={i} {dtype} B={B} T={T} C={C} window=({first}, {width})", flush=True)
+
+        def place(values):
+            buf = torch.full((B, T, width), float("nan"), dtype=dtype, device=gpu)
+            buf[..., first:first + C] = values.to(dtype).to(gpu)
+            return buf, buf[..., first:first + C]
+
+        def surroundings_are_nan(buf):
+            return bool(torch.isnan(buf[..., :first]).all()) and bool(torch.isnan(buf[..., first + C:]).all())
+
+        shape = (B, T, C)
+        _, a = place(torch.rand(shape, generator=g, dtype=torch.float64))
+        _, b = place(torch.randn(shape, generator=g, dtype=torch.float64))
+        _, gh = place(torch.randn(shape, generator=g, dtype=torch.float64))
+        want_h = oracle.fwd(as_rows(a), as_rows(b))
+        got_h = hip.scan_forward(a.mT, b.mT)
+        assert rel_err(as_rows(got_h.mT), want_h) <= bar, "forward"
+        _, hs = place(torch.from_numpy(want_h).mT)
+        want_ga, want_gb = oracle.bwd(as_rows(a), as_rows(hs), as_rows(gh))
+        got_ga, got_gb = hip.scan_backward(a.mT, hs.mT, gh.mT)
+        assert rel_err(as_rows(got_gb.mT), want_gb) <= bar, "grad of value"
+        assert rel_err(as_rows(got_ga.mT), want_ga, prev_abs(as_rows(hs))) <= bar, "grad of gate"
+        # The same through the C ABI's strided calls with the outputs inside NaN-filled buffers of their own.
+        L = hip.lib()
+        code = hip._dtype_code(dtype)
+        outs = [place(torch.zeros(shape, dtype=torch.float64)) for _ in range(3)]
+        st = hip.Strides(outer=T * width, row=width)
+        # (the workspace size the library reports covers every alignment a window may turn out to have)
+        ws_n = max(hip.workspace_bytes_cl(B, T, C, dtype, d) for d in (hip.FORWARD, hip.BACKWARD))
+        ws = torch.empty(max(ws_n, 8), dtype=torch.uint8, device=gpu)
+        stream = torch.cuda.current_stream().cuda_stream
+        refs = [ctypes.byref(st)] * 5
+        rc = L.scanscam_scan_fwd_cl_strided(a.data_ptr(), b.data_ptr(), outs[0][1].data_ptr(), refs[0], refs[1], refs[2],
+                                            B, T, C, code, ws.data_ptr(), ws.numel(), stream, None)
+        assert rc == 0, hip.strerror(rc)
+        rc = L.scanscam_scan_bwd_cl_strided(a.data_ptr(), hs.data_ptr(), gh.data_ptr(), outs[1][1].data_ptr(),
+                                            outs[2][1].data_ptr(), refs[0], refs[1], refs[2], refs[3], refs[4],
+                                            B, T, C, code, ws.data_ptr(), ws.numel(), stream, None)
+        assert rc == 0, hip.strerror(rc)
+        torch.cuda.synchronize()
+        assert rel_err(as_rows(outs[0][1]), want_h) <= bar, "forward into a window"
+        assert rel_err(as_rows(outs[2][1]), want_gb) <= bar, "grad of value into a window"
+        assert rel_err(as_rows(outs[1][1]), want_ga, prev_abs(as_rows(hs))) <= bar, "grad of gate into a window"
+        for buf, _ in outs:
+            assert surroundings_are_nan(buf), "a store outside the window"
