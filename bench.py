@@ -34,6 +34,10 @@ Prints ONE JSON line. Besides the contract fields it carries
   long_rows     many rows of 16K to 96K elements (long-context shapes);
   odd_lengths   row lengths that are no multiple of a 128-byte line or of the
                 16-byte vector;
+  channels_last contiguous [B, T, C] tensors scanned along T (the reference's
+                transposed kernels): its timing shape, many channels, many batch
+                elements, channel counts off the 128-byte line and below a wave,
+                fp32 and bf16, with the launch plan each direction takes;
   autograd_op   the same step through the op a model calls,
                 scanscam_amd.scan(a, b).backward(grad_h), outputs allocated per call;
   configs       forward and forward+backward GB/s of the other four synthetic
@@ -515,16 +519,11 @@ def launch_shapes(args, hip, torch):
     print(json.dumps(out))
 
 
-def channels_last_workload(spec, args, hip, torch):
-    """--channels-last BxTxC[:dtype]: forward and backward over contiguous [B, T, C] tensors (scanned along T).
+def time_channels_last(B, T, C, dtype, steps, warmup, hip, torch):
+    """Forward and backward over contiguous [B, T, C] tensors (scanned along T): milliseconds per launch, buffer sets.
 
-    Buffer sets rotate over >= 1 GiB; mean microseconds per launch over back-to-back launches. Used for the
-    rocprofv3 summaries of the channels-last kernels under profiles/; prints its own JSON line.
+    Buffer sets rotate over >= 1 GiB; mean over back-to-back launches.
     """
-    shape_s, _, dtype_s = spec.partition(":")
-    B, T, C = (int(v) for v in shape_s.lower().split("x"))
-    dtype = {"": torch.float32, "f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16,
-             "f64": torch.float64}[dtype_s]
     dev = torch.device("cuda:0")
     g = torch.Generator(device=dev).manual_seed(0)
     n = B * T * C
@@ -540,24 +539,66 @@ def channels_last_workload(spec, args, hip, torch):
         bwd.append(hip.prepare_backward_cl(a, h, gh, ga, gb))
     ms = []
     for calls in (fwd, bwd):
-        for i in range(max(args.warmup, nsets)):
+        for i in range(max(warmup, nsets)):
             calls[i % nsets]()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         e0.record()
-        for i in range(args.steps):
+        for i in range(steps):
             calls[i % nsets]()
         e1.record()
         torch.cuda.synchronize()
-        ms.append(e0.elapsed_time(e1) / args.steps)
+        ms.append(e0.elapsed_time(e1) / steps)
+    del fwd, bwd
+    torch.cuda.empty_cache()
+    return ms[0], ms[1], nsets
+
+
+def channels_last_workload(spec, args, hip, torch):
+    """--channels-last BxTxC[:dtype]: forward and backward over contiguous [B, T, C] tensors (scanned along T).
+
+    Used for the rocprofv3 summaries of the channels-last kernels under profiles/; prints its own JSON line.
+    """
+    shape_s, _, dtype_s = spec.partition(":")
+    B, T, C = (int(v) for v in shape_s.lower().split("x"))
+    dtype = {"": torch.float32, "f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16,
+             "f64": torch.float64}[dtype_s]
+    f_ms, b_ms, nsets = time_channels_last(B, T, C, dtype, args.steps, args.warmup, hip, torch)
+    n = B * T * C
+    esize = torch.empty(0, dtype=dtype).element_size()
     print(json.dumps({
         "workload": f"channels-last [B={B}, T={T}, C={C}] {str(dtype).replace('torch.', '')}, a ~ U(0,1), b, grad_h ~ N(0,1)",
         "buffer_sets": nsets, "steps": args.steps,
-        "fwd_us": round(ms[0] * 1e3, 2), "bwd_us": round(ms[1] * 1e3, 2),
-        "fwd_frac": round(FWD_BYTES[esize] * n / (ms[0] * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-        "bwd_frac": round(BWD_BYTES[esize] * n / (ms[1] * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+        "fwd_us": round(f_ms * 1e3, 2), "bwd_us": round(b_ms * 1e3, 2),
+        "fwd_frac": round(FWD_BYTES[esize] * n / (f_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+        "bwd_frac": round(BWD_BYTES[esize] * n / (b_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
         "fwd_bytes": FWD_BYTES[esize] * n, "bwd_bytes": BWD_BYTES[esize] * n,
     }))
+
+
+def channels_last_table(args, hip, torch):
+    """Contiguous [B, T, C] tensors scanned along T (the layout of the reference's transposed kernels,
+    scanscam/cuda.py:100-148): its timing shape, many-channel and many-batch shapes in fp32 and bf16, channel
+    counts that are no whole 128-byte lines or fewer than a wave. Rotated buffer sets, prepared calls."""
+    shapes = [(8, 4096, 512, torch.float32), (8, 4096, 2048, torch.float32), (64, 2048, 1024, torch.float32),
+              (256, 1024, 1024, torch.float32), (8, 4096, 512, torch.bfloat16), (8, 4096, 2048, torch.bfloat16),
+              (64, 2048, 1024, torch.bfloat16), (256, 1024, 1024, torch.bfloat16), (8, 4096, 1000, torch.float32),
+              (64, 2048, 1001, torch.float32), (64, 2048, 1001, torch.bfloat16), (2048, 512, 40, torch.float32),
+              (2048, 512, 40, torch.bfloat16)]
+    out = {}
+    for B, T, C, dtype in shapes:
+        f_ms, b_ms, nsets = time_channels_last(B, T, C, dtype, max(20, args.steps // 2), max(3, args.warmup // 2), hip, torch)
+        n, esize = B * T * C, torch.empty(0, dtype=dtype).element_size()
+        short = lambda p: f"mode={p.mode} vec={p.vec} steps={p.unroll} waves={p.waves}"
+        out[f"{B}x{T}x{C}_{str(dtype).replace('torch.', '')}"] = {
+            "fwd_us": round(f_ms * 1e3, 1), "bwd_us": round(b_ms * 1e3, 1),
+            "fwd_frac": round(FWD_BYTES[esize] * n / (f_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+            "bwd_frac": round(BWD_BYTES[esize] * n / (b_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+            "buffer_sets": nsets,
+            "plan_fwd": short(hip.resolve_plan_cl(B, T, C, dtype, hip.FORWARD)),
+            "plan_bwd": short(hip.resolve_plan_cl(B, T, C, dtype, hip.BACKWARD)),
+        }
+    return out
 
 
 def cpu_baseline(a, b, gh, reps):
@@ -835,6 +876,7 @@ def main():
         out["strided_views"] = strided_views(dev, args, hip, torch)
         out["long_rows"] = long_rows(dev, args, hip, torch)
         out["odd_lengths"] = odd_lengths(dev, args, hip, torch)
+        out["channels_last"] = channels_last_table(args, hip, torch)
 
     if not args.no_cpu:
         # 16-bit workloads: the reference has no 16-bit path, so its loop runs on the exact fp32 upcast.
