@@ -425,3 +425,19 @@ def test_random_channels_last_shapes(gpu, block):
         assert rel_err(as_rows(outs[1][1]), want_ga, prev_abs(as_rows(hs))) <= bar, "grad of gate into a window"
         for buf, _ in outs:
             assert surroundings_are_nan(buf), "a store outside the window"
+
+
+def test_plan_search_runs_and_reports_both_directions(gpu):
+    # The tuning tool on two small shapes: every plan it keeps is one the library ran, the automatic plan is among them.
+    import io
+
+    from scanscam_amd import plan_search
+
+    for layout, shape in (("cl", (4, 300, 96)), ("rows", (64, 1000))):
+        text = io.StringIO()
+        res = plan_search.search(layout, shape, torch.float32, reps=3, warm=1, out=text, every=True)
+        assert set(res) == {"fwd", "bwd"}
+        for auto_us, best_us, _ in res.values():
+            assert 0 < best_us <= auto_us
+        lines = text.getvalue().splitlines()
+        assert lines[0].startswith(layout) and sum(line.strip().startswith("auto") for line in lines[1:]) == 2
