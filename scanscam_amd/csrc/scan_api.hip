@@ -162,7 +162,14 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
     Launch &l = out->l;
     l = Launch{0, 0, 0, 0, 1, 64, 0, false, 1};
     const bool flat_possible = flat_ok && T >= full && T <= (int64_t)kWave * full && flat_rows(rows, T, full) > 0;
-    if (u.mode == kModeFlat || (u.mode == SCANSCAM_MODE_AUTO && flat_possible && !u.vec && prefer_flat(T, full, esize))) {
+    // Up to 32 MiB per tensor the flat kernel's larger workgroups (16 chunks each, a halo chunk and an LDS exchange
+    // per workgroup) cost more than the lanes it fills gain: rows of four vectors or more stay with the small kernel's
+    // element-aligned vectors there (fp32 [16513, 127] forward 9.2 -> 7.4 us, bf16 [33554, 250] 15.6 -> 12.7 us over 200
+    // launches; [8224, 255], 64 vectors per row, 6.7 against 7.0 us; at 100 MB, [200000, 127], the flat kernel is
+    // ahead, 49 against 58 us).
+    const bool small_problem = rows * T * esize <= (int64_t(1) << 25) && T >= 4 * full;
+    if (u.mode == kModeFlat ||
+        (u.mode == SCANSCAM_MODE_AUTO && flat_possible && !u.vec && !small_problem && prefer_flat(T, full, esize))) {
         if (!flat_possible) return SCANSCAM_EPLAN;
         if (u.vec && u.vec != full) return SCANSCAM_EPLAN;
         l.mode = kModeFlat;

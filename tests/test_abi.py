@@ -143,11 +143,12 @@ def test_empty_inputs_are_a_successful_noop():
         (131072, 64, torch.float32, hip.MODE_SMALL, 4),     # many short rows
         (32, 1025, torch.float32, hip.MODE_ROW, 4),         # odd length: element-aligned 16-byte vectors
         (32, 5, torch.float32, hip.MODE_FLAT, 4),           # short rows of any length, dense: one flat stream
-        (32, 70, torch.float32, hip.MODE_FLAT, 4),
-        (32, 48, torch.float32, hip.MODE_FLAT, 4),          # 12 vectors: no power-of-two group of lanes
+        (200000, 70, torch.float32, hip.MODE_FLAT, 4),
+        (200000, 48, torch.float32, hip.MODE_FLAT, 4),      # 12 vectors: no power-of-two group of lanes
+        (32, 70, torch.float32, hip.MODE_SMALL, 4),         # ... up to 32 MiB per tensor: element-aligned vectors, several rows per wave
         (32, 3, torch.float32, hip.MODE_SMALL, 1),          # shorter than a vector
-        (32, 100, torch.bfloat16, hip.MODE_FLAT, 8),
-        (32, 104, torch.bfloat16, hip.MODE_SMALL, 8),       # 16-bit storage keeps groups that are at least 0.6 full
+        (200000, 100, torch.bfloat16, hip.MODE_FLAT, 8),
+        (200000, 104, torch.bfloat16, hip.MODE_SMALL, 8),   # 16-bit storage keeps groups that are at least 0.6 full
         (3, 5, torch.float32, hip.MODE_SMALL, 1),           # too few rows for a whole number of vectors
     ],
 )

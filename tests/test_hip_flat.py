@@ -50,8 +50,9 @@ def test_forced_flat_plans_over_row_lengths(gpu, dtype):
 
 
 def test_flat_is_the_automatic_choice_for_odd_short_rows(gpu):
-    for rows, T, dtype in ((4099, 70, torch.float32), (5000, 101, torch.float32), (3000, 100, torch.bfloat16),
-                           (2048, 33, torch.float64)):
+    # (beyond 32 MiB per tensor: below that, rows of four vectors or more stay with the small kernel)
+    for rows, T, dtype in ((120003, 70, torch.float32), (90000, 101, torch.float32), (170000, 100, torch.bfloat16),
+                           (130000, 33, torch.float64), (2048, 9, torch.float32)):
         assert hip.resolve_plan(rows, T, dtype, hip.FORWARD).mode == hip.MODE_FLAT
         assert hip.resolve_plan(rows, T, dtype, hip.BACKWARD).mode == hip.MODE_FLAT
         g = seeded(T)
