@@ -163,20 +163,26 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
     l = Launch{0, 0, 0, 0, 1, 64, 0, false, 1};
     const bool flat_possible = flat_ok && T >= full && T <= (int64_t)kWave * full && flat_rows(rows, T, full) > 0;
     // Up to 32 MiB per tensor the flat kernel's larger workgroups (16 chunks each, a halo chunk and an LDS exchange
-    // per workgroup) cost more than the lanes it fills gain: rows of four vectors or more stay with the small kernel's
+    // per workgroup) cost more than the few lanes it still fills gain: rows of four vectors or more stay with the small kernel's
     // element-aligned vectors there (fp32 [16513, 127] forward 9.2 -> 7.4 us, bf16 [33554, 250] 15.6 -> 12.7 us over 200
     // launches; [8224, 255], 64 vectors per row, 6.7 against 7.0 us; at 100 MB, [200000, 127], the flat kernel is
     // ahead, 49 against 58 us).
-    const bool small_problem = rows * T * esize <= (int64_t(1) << 25) && T >= 4 * full;
+    // (Only where the rows fill nine tenths of their lane group: at bf16 [119837, 70], 9 vectors in 16 lanes, the flat
+    // kernel is 15 / 38 % ahead at 16 MB too.)
+    const int64_t row_vectors = (T + full - 1) / full;
+    const bool small_problem = rows * T * esize <= (int64_t(1) << 25) && T >= 4 * full &&
+                               row_vectors * 10 >= (int64_t)pow2_ceil((int)row_vectors) * 9;
     if (u.mode == kModeFlat ||
         (u.mode == SCANSCAM_MODE_AUTO && flat_possible && !u.vec && !small_problem && prefer_flat(T, full, esize))) {
         if (!flat_possible) return SCANSCAM_EPLAN;
         if (u.vec && u.vec != full) return SCANSCAM_EPLAN;
         l.mode = kModeFlat;
         l.vec = full;
-        // 4 waves x 4 chunks; 16-bit storage (twice the registers per chunk) 8 waves x 2 chunks.
-        l.unroll = u.unroll ? u.unroll : (esize == 2 ? 2 : 4);
-        l.waves = u.waves ? u.waves : (esize == 2 ? 8 : 4);
+        // 4 waves x 4 chunks; 16-bit storage (twice the registers per chunk) 8 waves x 2 chunks -- from 16 MiB per
+        // tensor on: below, 4 x 4 there too (bf16 [119837, 70] forward 16.0 -> 14.3 us, [27962, 300] 12.7 -> 11.2 us).
+        const bool halves = esize == 2 && rows * T * esize > (int64_t(1) << 24);
+        l.unroll = u.unroll ? u.unroll : (halves ? 2 : 4);
+        l.waves = u.waves ? u.waves : (halves ? 8 : 4);
         if ((l.unroll != 2 && l.unroll != 4) || l.waves < 1 || l.waves > scanscam::kMaxWaves) return SCANSCAM_EPLAN;
         out->nch = 1;
         out->tiles_per_row = 0;
@@ -319,12 +325,15 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
         // instead of one of 16 waves): [1, 2^26] 61 -> 64 % of peak, [16, 2^22] 64 -> 66 %, [8, 2^21] 53 -> 57 %;
         // the backward pass gains nothing from it, 16-bit storage with 2 to 8 rows (bf16 [8, 2^22] 50 -> 43 us,
         // [4, 2^23] 48 -> 46 us, [2, 2^24] 49 -> 46 us; [1, 2^26] level, [16, 2^21] 47 -> 51 us).
+        // (fp32 with 17 to 64 rows likewise while the whole problem is 8 M elements or less, i.e. up to 512 such tiles:
+        // [32, 262144] forward 26.1 -> 20.0 us, [64, 131072] 25.4 -> 21.4 us; at 32 M elements the 32-chunk tile is level.)
+        const bool few_tiles = esize == 4 && rows > 16 && rows <= 64 && rows * (int64_t)nch <= 32768;
         if (!u.waves && !u.unroll && !rev && l.vec == full && !l.ragged &&
-            (esize == 4 ? rows <= 16 : (esize == 2 && rows >= 2 && rows <= 8))) {
+            (esize == 4 ? (rows <= 16 || few_tiles) : (esize == 2 && rows >= 2 && rows <= 8))) {
             l.unroll = 8;
             l.waves = 8;
         }
-        if (!u.waves && !u.unroll && rows > 8) {
+        if (!u.waves && !u.unroll && rows > 8 && !(few_tiles && l.unroll == 8)) {
             // As many tiles as 8-wave tiles would take, but with only the waves they need: 75 chunks are 3
             // tiles of 7 waves (84 chunk slots), not of 8 (96).
             int tiles = (nch + kTileChunks - 1) / kTileChunks;

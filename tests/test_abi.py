@@ -145,7 +145,9 @@ def test_empty_inputs_are_a_successful_noop():
         (32, 5, torch.float32, hip.MODE_FLAT, 4),           # short rows of any length, dense: one flat stream
         (200000, 70, torch.float32, hip.MODE_FLAT, 4),
         (200000, 48, torch.float32, hip.MODE_FLAT, 4),      # 12 vectors: no power-of-two group of lanes
-        (32, 70, torch.float32, hip.MODE_SMALL, 4),         # ... up to 32 MiB per tensor: element-aligned vectors, several rows per wave
+        (32, 70, torch.float32, hip.MODE_FLAT, 4),
+        (32, 61, torch.float32, hip.MODE_SMALL, 4),         # ... up to 32 MiB per tensor, rows that fill their lane group: element-aligned vectors, several rows per wave
+        (200000, 61, torch.float32, hip.MODE_FLAT, 4),
         (32, 3, torch.float32, hip.MODE_SMALL, 1),          # shorter than a vector
         (200000, 100, torch.bfloat16, hip.MODE_FLAT, 8),
         (200000, 104, torch.bfloat16, hip.MODE_SMALL, 8),   # 16-bit storage keeps groups that are at least 0.6 full

@@ -50,7 +50,7 @@ def test_forced_flat_plans_over_row_lengths(gpu, dtype):
 
 
 def test_flat_is_the_automatic_choice_for_odd_short_rows(gpu):
-    # (beyond 32 MiB per tensor: below that, rows of four vectors or more stay with the small kernel)
+    # (rows that fill nine tenths of their lane group take it beyond 32 MiB per tensor only: 101 fp32 elements are 26 of 32 lanes)
     for rows, T, dtype in ((120003, 70, torch.float32), (90000, 101, torch.float32), (170000, 100, torch.bfloat16),
                            (130000, 33, torch.float64), (2048, 9, torch.float32)):
         assert hip.resolve_plan(rows, T, dtype, hip.FORWARD).mode == hip.MODE_FLAT

@@ -377,6 +377,7 @@ AUTO_REGIMES = [
     (300, 16640, (ROW, 9, 4), None),          # few rows, 65 chunks: 2 steps of 9 waves
     (255, 16640, (LOOKBACK, 0, 4), None),     # fewer than 256 rows: tiles in tile-major order
     (12, 300000, (LOOKBACK, 0, 8), (LOOKBACK, 0, 4)),  # up to 16 rows: forward tiles of 8 waves x 8 chunks
+    (48, 100000, (LOOKBACK, 0, 8), (LOOKBACK, 0, 4)),  # ... and 17 to 64 rows of a problem of 8 M elements or less
 ]
 
 
