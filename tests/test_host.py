@@ -209,3 +209,16 @@ def test_plan_search_sets_hold_plans_the_library_knows():
                 assert any(L.scanscam_resolve_plan_cl(batch, 2048, C, code, hip.FORWARD, ctypes.byref(plan), ctypes.byref(out)) == 0
                            for batch in (8, 512)), (C, plan)
     assert {"cl-a", "cl-b", "cl-odd", "rows-25"} <= set(plan_search.SUITES)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    # This build runs on one GPU: asking for more ends with a message that says so, before anything touches a device.
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    done = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                          timeout=120)
+    assert done.returncode != 0
+    assert "one GPU" in done.stderr and done.stdout.strip() == ""
