@@ -125,6 +125,23 @@ static int check_case(const char *name, long rows, long T, long C, int channels_
     /* gates and values in [0,1) x [-1,1): |h|, |grad_b| stay small, so 1e-5 (2e-5 for the product) is ample */
     if (!(eh <= 1e-5) || !(egb <= 1e-5) || !(ega <= 2e-5)) failures++;
 
+    if (channels_last) {
+        /* The plan the channels-last call resolves to, handed back in: bit-identical output, no larger workspace. */
+        scanscam_plan plan;
+        float *again = (float *)malloc(n * 4);
+        if (scanscam_resolve_plan_cl(batch, T, C, SCANSCAM_F32, SCANSCAM_FORWARD, NULL, &plan) != SCANSCAM_OK) failures++;
+        if (scanscam_workspace_bytes_cl(batch, T, C, SCANSCAM_F32, SCANSCAM_FORWARD, &plan) > ws_bytes) failures++;
+        HIP_OK(hipMemset(o0, 0, n * 4));
+        if (scanscam_scan_fwd_cl(da, db, o0, batch, T, C, SCANSCAM_F32, ws, ws_bytes, stream, NULL) != SCANSCAM_OK) failures++;
+        HIP_OK(hipStreamSynchronize(stream));
+        HIP_OK(hipMemcpy(again, o0, n * 4, hipMemcpyDeviceToHost));
+        HIP_OK(hipMemset(o0, 0, n * 4));
+        if (scanscam_scan_fwd_cl(da, db, o0, batch, T, C, SCANSCAM_F32, ws, ws_bytes, stream, &plan) != SCANSCAM_OK) failures++;
+        HIP_OK(hipStreamSynchronize(stream));
+        HIP_OK(hipMemcpy(got, o0, n * 4, hipMemcpyDeviceToHost));
+        if (memcmp(got, again, n * 4) != 0 || worst(got, h, n) > 1e-5) failures++;
+        free(again);
+    }
     if (!channels_last) {
         /* The same launch through the _plan and _timed variants: a resolved plan handed back in gives
          * bit-identical output, and the caller's events hold the kernel's own duration. */
