@@ -723,6 +723,13 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
             !(l->vec == full && esize == 2 && rev && C >= 4096 && T >= 1024 &&
               batch * groups(full) * 10 >= ((batch * groups(full) + kComputeUnits - 1) / kComputeUnits) * kComputeUnits * 9))
             l->vec = half;
+        // float64: its 8-byte lane is the single channel, and the same holds (fp64 [64, 2048, 512] 283 / 446 -> 258 / 429 us,
+        // [256, 1024, 256] 272 / 456 -> 251 / 434 us with 8 waves of 8 steps).
+        // (From 128 channels on; backwards only where the 16-byte lanes give 512 workgroups: at 256 of them,
+        // [32, 2048, 1024], the backward pass is 16 % faster in 16-byte lanes.)
+        if (esize == 8 && l->vec == full && C >= 2 * kWave && batch * groups(1) >= enough &&
+            groups(1) * 20 <= groups(full) * full * 21 && (!rev || batch * groups(full) >= 512))
+            l->vec = 1;
         // Few channels (the packed kernel, below): a wide lane leaves more steps per instruction to scan
         // across with lane shuffles, which costs more than the wider loads gain -- except where C is not a
         // power of two and one channel per lane would leave a quarter of 32 lanes idle (fp32 [256, 8192, 24]:
@@ -857,6 +864,8 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // Tiles of 8-byte fp32 lanes backwards (kept from the choice above where there are a few workgroups too many):
     // 8 steps, which fit 104 registers where 16 need 129 (fp32 [520, 2000, 96] 504 -> 438 us).
     if (!u.unroll && l->kind == 2 && esize == 4 && l->vec == 2 && rev) l->steps = 8;
+    // (float64 in its 8-byte lanes likewise: [8, 4096, 512] backward 148 -> 130 us)
+    if (!u.unroll && l->kind == 2 && esize == 8 && l->vec == 1 && rev) l->steps = 8;
     // A walk of all of T in 8-byte fp32 lanes forwards, 2048 or more channels: 16 steps per wave ([64, 1024, 2048]
     // 292 -> 266 us, [256, 512, 2048] 589 -> 525 us, [512, 256, 2048] 561 -> 499 us, [128, 1024, 2048] 586 -> 535 us,
     // [40, 2048, 4096] 712 -> 658 us, [12, 4096, 8192] 831 -> 774 us; with 1024 channels 16 steps lose as much).
@@ -905,6 +914,9 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
             if (l->vec == 2 && C == kWave && rowgroups >= 2 * kComputeUnits) l->waves = 4;  // ([256, 4096, 64] backward: 220 us with 4 waves, 154 us with 8)
             if (l->vec == 1 && rev && groups(1) >= 2) l->waves = 4;
         }
+        // float64, single channels (8-byte lanes) walking all of T: 8 waves, as for the 8-byte lanes of fp32
+        // ([8, 4096, 2048] 282 / 484 us with 16 waves, 256-262 / 436-450 us with 4 or 8).
+        if (l->kind == 0 && esize == 8 && l->vec == 1 && l->group == kWave && l->waves > 8) l->waves = 8;
         // fp32 with 2048 or more channels: the forward pass above in 4-wave workgroups from 4096 channels on
         // ([24, 2048, 4096] 413 -> 391 us, [16, 2048, 8192] 554 -> 521 us), the backward pass in 16-byte lanes in
         // 4-wave workgroups up to 512 time steps ([128, 512, 2048] 586 -> 478 us).

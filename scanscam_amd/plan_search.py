@@ -8,7 +8,7 @@ Time the library's automatic launch plan for a shape against a set of forced pla
 ``rows`` shapes are contiguous ``[rows, T]`` tensors scanned along ``T`` (the layout of
 ``simple_linear_scan`` and its siblings, ``scanscam/cuda.py:28-64`` in the reference), ``cl`` shapes are
 contiguous ``[batch, T, C]`` tensors scanned along ``T`` (``transposed_linear_scan``, ``cuda.py:100-148``).
-dtype is f32 (default), bf16 or f16.
+dtype is f32 (default), bf16, f16 or f64.
 
 One line per shape and dtype: the automatic plan's forward / backward microseconds and fraction of the 8 TB/s
 HBM peak in algorithmic bytes (3 and 5 elements per scanned element), then the fastest plan of the set for each
@@ -29,7 +29,7 @@ import torch
 from . import hip
 
 P = hip.Plan
-DTYPES = {"": torch.float32, "f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
+DTYPES = {"": torch.float32, "f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16, "f64": torch.float64}
 HBM_PEAK_GBPS = 8000.0
 
 SUITES = {
@@ -78,8 +78,9 @@ def row_plans(dtype, T):
 
 def cl_plans(dtype, C):
     """Forced plans for channels-last storage: every lane width over a few tile shapes, whole-T walks and time-split tiles."""
-    full = 16 // torch.empty(0, dtype=dtype).element_size()
-    half, narrow = full // 2, (1 if full == 4 else 2)
+    esize = torch.empty(0, dtype=dtype).element_size()
+    full = 16 // esize
+    half, narrow = max(1, full // 2), (2 if esize == 2 else 1)
     walk, split = hip.MODE_ROW, hip.MODE_LOOKBACK
     most = 16 if full == 4 else 8  # waves that the kernels' LDS arrays allow with 16-byte lanes
     out = [P(vec=v, unroll=s, waves=w, mode=walk)

@@ -215,6 +215,8 @@ WALK, TILES = hip.MODE_ROW, hip.MODE_LOOKBACK
         ((300, 1000, 77), torch.bfloat16, (WALK, 1, 8, 16), (TILES, 1, 16, 8)),
         ((2048, 512, 40), torch.float32, (WALK, 2, 8, 8), (WALK, 2, 8, 8)),       # several time steps per instruction
         ((128, 512, 2048), torch.float32, (WALK, 2, 16, 8), (WALK, 4, 4, 4)),     # 2048 or more fp32 channels
+        ((256, 1024, 256), torch.float64, (WALK, 1, 8, 8), (WALK, 1, 8, 8)),      # float64: its 8-byte lane is one channel
+        ((8, 4096, 512), torch.float64, (TILES, 1, 16, 8), (TILES, 1, 8, 8)),
         ((24, 2048, 4096), torch.float32, (WALK, 2, 16, 4), (WALK, 4, 4, 4)),
     ],
 )

@@ -320,6 +320,8 @@ MANY_WORKGROUPS = [
     (torch.float16, (130, 1030, 601), None),
     (torch.bfloat16, (260, 130, 256), None),    # 16-bit, 129-256 channels: four-channel lanes, 4 waves
     (torch.bfloat16, (32, 1100, 4096), None),   # 16-bit, 4096 or more channels: 16-byte lanes backwards
+    (torch.float64, (260, 70, 256), None),      # float64: single channels (8-byte lanes) ahead of 16-byte lanes
+    (torch.float64, (8, 1100, 256), None),      # ... 8 steps per tile backwards when time is split over workgroups
     (torch.float32, (2, 40, 65536), None),      # very wide time steps
     (torch.bfloat16, (1, 7, 100001), None),
     (torch.float16, (300, 1, 1000), None),      # a single time step
