@@ -705,7 +705,9 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         // lanes leave too few workgroups and narrow lanes were the only choice (fp32 [32, 2048, 1024] 67 / 65 ->
         // 73 / 78 %, [64, 2048, 512] 67 / 66 -> 75 / 70 %, bf16 [32, 4096, 2048] 66 / 62 -> 69 / 72 %).
         // (Time steps that are not whole 128-byte lines keep 16-byte lanes where those give 256 workgroups:
-        // fp32 [64, 2048, 1016] backward 57 % against 50 %.)
+        // fp32 [64, 2048, 1016] backward 57 % against 50 %. 16-bit storage in rows of fewer than 384 steps does not: bf16
+        // [256, 333, 1000] 125 / 207 -> 100 / 194 us, [512, 256, 1000] 184 / 324 -> 149 / 296 us; [300, 400, 1512] is 6 % faster
+        // in 16-byte lanes, [256, 1024, 1000] 18 %.)
         // (16-bit storage keeps 256 for its four-channel lanes: bf16 [28, 4096, 2048] gains with 224 workgroups of
         // them, [72, 2048, 768] loses 15 % with 216.)
         // (And the backward pass of fp32 with 2048 or more channels: [32, 2048, 2048] 437 us against 505-530 us,
@@ -718,7 +720,8 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         // they are with 512 time steps or where the 16-byte lanes' workgroups are no whole rounds of 256:
         // [64, 512, 4096] 241 against 280 us, [40, 2048, 4096] 645 against 765 us.)
         if (half_possible && C >= (int64_t)kWave * half && fills(half) &&
-            batch * groups(half) >= (esize == 2 ? 256 : enough) && (l->vec != full || (C * esize) % 128 == 0) &&
+            batch * groups(half) >= (esize == 2 ? 256 : enough) &&
+            (l->vec != full || (C * esize) % 128 == 0 || (esize == 2 && T < 384)) &&
             !(l->vec == full && esize == 4 && rev && C >= 2048 && (batch * groups(full) < 512 || T >= 256)) &&
             !(l->vec == full && esize == 2 && rev && C >= 4096 && T >= 1024 &&
               batch * groups(full) * 10 >= ((batch * groups(full) + kComputeUnits - 1) / kComputeUnits) * kComputeUnits * 9))
@@ -749,11 +752,17 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
             // channels but leave the last wave of pairs half empty (C = 320: 215 / 358 -> 186 / 353 us, C = 448: 302 /
             // 504 -> 264 / 494 us); at exactly 64 channels the backward pass is faster in pairs (98 -> 70 us).
             // (pairs that fill their two waves keep them: C = 256 at 256 batch elements 73 / 128 us against 87 / 137 us)
-            // (With the next tile's loads issued ahead, four-channel lanes also at exactly 256 channels and from 256
-            // batch elements: bf16 [256, 1024, 256] 72 / 132 -> 72 / 118 us, [512, 1024, 256] 146 / 258 -> 144 / 244 us.)
-            if (C > 2 * kWave && C <= 4 * kWave && half_possible && batch >= 256) l->vec = half;
-            else if (C > 4 * kWave && C % kWave == 0 && C % (2 * kWave) != 0) l->vec = 1;
-            else if (C == kWave && rev && pair_possible && batch >= 256) l->vec = 2;
+            // (With the next tile's loads issued ahead, from 256 batch elements on; at exactly 256 channels pairs with
+            // 16 steps, below, are level at 256 batch elements and 7 % ahead backwards at 512 and 2048.)
+            // (192 channels, three whole waves of single channels, with 16 steps: [512, 2048, 192] 245 / 402 -> 233 / 389 us.)
+            const bool odd_waves = C > 2 * kWave && C % kWave == 0 && C % (2 * kWave) != 0;
+            if (odd_waves && (C > 4 * kWave || T >= 512)) l->vec = 1;
+            else if (C > 2 * kWave && C <= 4 * kWave && C % (2 * kWave) != 0 && half_possible && batch >= 256) l->vec = half;
+            // (At exactly 64 channels, with loads issued a tile ahead: single channels in both directions, 8 waves of
+            // 16 steps -- [256, 4096, 64] 78 / 153 -> 76 / 131 us, [2048, 512, 64] 74 / 130 -> 69 / 124 us, [4096, 256, 64]
+            // forward 77 -> 65 us; pairs are 0 to 15 % behind backwards now and 5 to 25 % forwards. Rows of fewer than 256
+            // steps are shorter than two such tiles and keep pairs backwards.)
+            if (C == kWave && rev && pair_possible && batch >= 256 && T < 256) l->vec = 2;
         }
     }
     // fp32 with fewer than 128 channels and a workgroup per batch element: pairs of channels (8-byte lanes) with 8
@@ -804,9 +813,16 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // tiles of single channels.)
     const bool pairs_fill = groups(2) * kWave * 2 * 7 <= C * 10;
     // (With many channel groups per batch element the tiles of pairs win all the same: bf16 [16, 4096, 2050] 572 -> 403 us.)
-    if (few_too_many && !(esize == 2 && rev && !half_fits && pairs_fill && groups(2) < 8)) {
+    // (Forwards it needs pairs that fill their waves to 85 %, from 64 channels on: bf16 [520, 2000, 96], 75 %, 138 us in the
+    // walk and 156 us in tiles, [300, 1000, 200], 78 %, 93-98 against 105 us, [100, 3000, 300] 172 against 179 us; and the
+    // tiles are of pairs, not of the four-channel lanes the walk chose: [24, 2048, 3072] 220 -> 197 us, [130, 2048, 512]
+    // 200 -> 173 us.)
+    const bool pairs_fill_fwd = C < kWave || groups(2) * kWave * 2 * 17 <= C * 20;
+    if (few_too_many && !(esize == 2 && rev && !half_fits && pairs_fill && groups(2) < 8) &&
+        !(esize == 2 && !rev && !pairs_fill_fwd)) {
         l->kind = 2;
         if (l->vec == full && full > 1) l->vec = narrow;
+        if (esize == 2 && !rev && l->vec == half) l->vec = narrow;
         // single channels where the lane chosen so far leaves more than 30 % of its waves empty and they do better
         if (groups(l->vec) * kWave * l->vec * 7 > C * 10 && groups(l->vec) * l->vec > groups(1)) l->vec = 1;
         rowgroups = batch * groups(l->vec);
@@ -859,7 +875,15 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // (element-aligned pairs of 16-bit channels likewise: bf16 [64, 2048, 1001] 36 / 34 -> 39 / 38 % of peak)
     // (and of fp32 channels: [512, 512, 333] backward 502 -> 390 us, [256, 1024, 777] 1246 -> 962 us, [128, 1024, 1003] 747 -> 664 us)
     const bool long_steps = l->kind != 0 || (esize == 2 && l->vec <= 2 && T >= 1024 && (rowgroups < 512 || (l->ragged && l->vec == 2))) ||
-                            (esize == 4 && l->ragged && l->vec == 2);
+                            (esize == 4 && l->ragged && l->vec == 2) ||
+                            // (with loads issued a tile ahead, every walk in narrow 16-bit lanes whose time step fills its
+                            // waves' lanes: bf16 [512, 1024, 256] 148 / 257 -> 145 / 238 us, [2048, 512, 128] backward 256 ->
+                            // 237 us, [512, 1024, 320] 184 / 331 -> 179 / 309 us, [1024, 1024, 64] backward 142 -> 124 us)
+                            // Rows shorter than a few such tiles lose: [4096, 128, 128] backward 114 -> 127 us, [1500, 100, 130]
+                            // 38 / 64 -> 45 / 84 us, element-aligned [700, 300, 257] 82 / 143 -> 94 / 188 us; the single channels of
+                            // 64 gain forwards from one tile on: [4096, 128, 64] 48 -> 35 us, [1024, 200, 64] 20.5 -> 18.2 us.
+                            (esize == 2 && l->vec <= 2 && l->kind == 0 && l->group == kWave && !l->ragged &&
+                             T >= (l->vec == 1 && C == kWave ? (rev ? 256 : 128) : 512));
     l->steps = u.unroll ? u.unroll : (narrow_lane ? (long_steps ? 16 : 8) : ((l->kind != 0 && full <= 4) ? 8 : 4));
     // Tiles of 8-byte fp32 lanes backwards (kept from the choice above where there are a few workgroups too many):
     // 8 steps, which fit 104 registers where 16 need 129 (fp32 [520, 2000, 96] 504 -> 438 us).
@@ -912,7 +936,10 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         if (l->kind == 0 && esize == 2 && l->waves > 4 && !l->ragged) {
             if (l->vec == half && l->group == kWave && groups(half) == 1) l->waves = 4;
             if (l->vec == 2 && C == kWave && rowgroups >= 2 * kComputeUnits) l->waves = 4;  // ([256, 4096, 64] backward: 220 us with 4 waves, 154 us with 8)
-            if (l->vec == 1 && rev && groups(1) >= 2) l->waves = 4;
+            if (l->vec == 1 && rev && groups(1) >= 2 && l->steps != 16) l->waves = 4;
+            // Single channels with 16 steps: 8 waves from two workgroups per CU on ([4096, 256, 64] forward 90 us
+            // with 16 waves, 65 us with 8; [256, 4096, 64], one per CU, level).
+            if (l->vec == 1 && l->steps == 16 && rowgroups >= 2 * kComputeUnits && l->waves > 8) l->waves = 8;
         }
         // float64, single channels (8-byte lanes) walking all of T: 8 waves, as for the 8-byte lanes of fp32
         // ([8, 4096, 2048] 282 / 484 us with 16 waves, 256-262 / 436-450 us with 4 or 8).

@@ -172,7 +172,7 @@ def main(argv=None):
     ap.add_argument("--suite", choices=sorted(SUITES), help="a fixed list of shapes, each in f32 and bf16")
     ap.add_argument("--reps", type=int, default=24)
     ap.add_argument("--every", action="store_true", help="also print every plan's timings")
-    args = ap.parse_args(argv)
+    args = ap.parse_intermixed_args(argv)  # options may stand between the layout and the shapes
     if not hip.has_hip_ops:
         sys.exit("plan_search: libscanscam_hip.so does not load")
     if not torch.cuda.is_available():

@@ -207,12 +207,19 @@ WALK, TILES = hip.MODE_ROW, hip.MODE_LOOKBACK
         ((64, 2048, 1024), torch.float32, (WALK, 2, 8, 8), (WALK, 2, 8, 8)),      # 8-byte lanes give 512 workgroups
         ((8, 4096, 512), torch.float32, (TILES, 2, 16, 8), (TILES, 1, 16, 8)),    # too few for a walk: tiles over time
         ((8, 4096, 2048), torch.bfloat16, (WALK, 1, 16, 16), (TILES, 4, 16, 8)),
-        ((256, 4096, 64), torch.bfloat16, (WALK, 1, 16, 16), (WALK, 2, 16, 8)),   # 64 channels: a wave of single channels
+        ((256, 4096, 64), torch.bfloat16, (WALK, 1, 16, 16), (WALK, 1, 16, 16)),  # 64 channels: a wave of single channels
+        ((4096, 256, 64), torch.bfloat16, (WALK, 1, 16, 8), (WALK, 1, 16, 8)),    # ... 8 waves from two workgroups per CU on
+        ((4096, 128, 64), torch.bfloat16, (WALK, 1, 16, 8), (WALK, 2, 8, 4)),     # ... short rows keep pairs backwards
+        ((512, 1024, 256), torch.bfloat16, (WALK, 2, 16, 8), (WALK, 2, 16, 8)),   # narrow 16-bit lanes: 16 steps from 512 steps on
+        ((2048, 256, 256), torch.bfloat16, (WALK, 2, 8, 8), (WALK, 2, 8, 8)),
+        ((512, 2048, 192), torch.bfloat16, (WALK, 1, 16, 8), (WALK, 1, 16, 8)),   # three whole waves of single channels
+        ((24, 2048, 3072), torch.bfloat16, (TILES, 2, 16, 8), (TILES, 4, 16, 8)), # 288 workgroups: tiles, pairs forwards
+        ((520, 2000, 96), torch.bfloat16, (WALK, 2, 16, 8), (WALK, 2, 16, 8)),    # ... not where the pairs leave a wave 25 % empty
         ((128, 1024, 1003), torch.bfloat16, (WALK, 4, 8, 8), (WALK, 4, 8, 8)),    # element-aligned 8-byte lanes, 512 workgroups
         ((256, 1024, 1001), torch.bfloat16, (WALK, 8, 4, 8), (WALK, 8, 4, 8)),    # ... 16-byte lanes from 400 workgroups on
         ((96, 1024, 1003), torch.float32, (WALK, 4, 4, 4), (WALK, 4, 4, 4)),      # fp32 keeps its 16-byte lanes
         ((300, 1024, 256), torch.float32, (TILES, 2, 16, 8), (WALK, 2, 8, 4)),    # 600 workgroups: 0.78 of three rounds
-        ((300, 1000, 77), torch.bfloat16, (WALK, 1, 8, 16), (TILES, 1, 16, 8)),
+        ((300, 1000, 77), torch.bfloat16, (WALK, 1, 16, 8), (TILES, 1, 16, 8)),
         ((2048, 512, 40), torch.float32, (WALK, 2, 8, 8), (WALK, 2, 8, 8)),       # several time steps per instruction
         ((128, 512, 2048), torch.float32, (WALK, 2, 16, 8), (WALK, 4, 4, 4)),     # 2048 or more fp32 channels
         ((256, 1024, 256), torch.float64, (WALK, 1, 8, 8), (WALK, 1, 8, 8)),      # float64: its 8-byte lane is one channel
