@@ -649,7 +649,9 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
             // 224 / 408 -> 200 / 358 us, [160, 1024, 1003] backward 660 -> 508 us, [128, 1024, 1501] backward 817 -> 557 us,
             // [128, 1024, 777] 202 / 332 -> 151 / 280 us, [160, 1024, 1004] 271 / 673 -> 251 / 447 us; from 400 workgroups
             // on the 16-byte lanes are ahead again, and fp32 keeps them throughout).
-            const bool half_instead = esize == 2 && full_fits && batch * groups(full) <= 384 &&
+            // (And on rows of fewer than 384 steps whatever the count: bf16 [39, 125, 4806] 35 / 91 -> 29 / 49 us, [209, 221, 1370]
+            // forward 98 -> 77 us.)
+            const bool half_instead = esize == 2 && full_fits && (batch * groups(full) <= 384 || T < 384) &&
                                       groups(half) * half <= groups(full) * full &&
                                       (half_whole || (half > 1 && ragged_fits(half) && fills65(half)));
             if (half_instead) {
@@ -684,6 +686,20 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
                 l->vec = 2;
                 l->ragged = !pair_possible;
             }
+            // fp32 forwards on rows of fewer than 384 steps: 8-byte lanes in place of element-aligned 16-byte ones
+            // ([209, 221, 1370] 179 -> 137 us, [90, 344, 1686] 148 -> 116 us, [39, 125, 4806] 63 -> 51 us; backwards level).
+            if (esize == 4 && !rev && T < 384 && l->vec == full && l->ragged && ragged_fits(half)) {
+                l->vec = half;
+                l->ragged = !half_possible;
+            }
+            // 16-bit storage backwards, too few workgroups for the rule above but enough for a walk in pairs (168):
+            // element-aligned pairs rather than single channels, walked or in tiles over time -- bf16 [71, 1910, 257]
+            // 159 -> 124 us, [101, 1576, 219] 155 -> 124 us, [14, 1439, 1473] 121 -> 104 us, [64, 2048, 257] 141 -> 129 us.
+            if (esize == 2 && rev && l->vec == 1 && !pair_possible && C >= 2 * kWave && u.mode == SCANSCAM_MODE_AUTO &&
+                batch * groups(2) >= enough && batch * groups(2) < 256) {
+                l->vec = 2;
+                l->ragged = true;
+            }
         }
     } else {
         // A workgroup owns 64*vec channels of one batch element. Enough of them: 16-byte loads.
@@ -697,7 +713,8 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         // and 225 / 375 us against 179 / 316 us with single channels), so a wider lane has to fill its groups
         // within 5 % of the narrow one.
         auto fills = [&](int vec) { return 21 * groups(narrow) * narrow >= 20 * groups(vec) * vec; };
-        l->vec = (batch * groups(full) >= 256 && fills(full)) ? full : narrow;
+        // (Up to 32 channels several time steps share a wave whatever the lane, and the walk starts at 80 workgroups, below.)
+        l->vec = (C <= 32 ? batch >= 80 : (batch * groups(full) >= 256 && fills(full))) ? full : narrow;
         // 8-byte lanes, where they still give 256 workgroups and fill their waves as well: they
         // stream as fast as 16-byte lanes or faster at equal shapes (two or four times the waves per byte in
         // flight: fp32 [256, 1024, 1024] 71 / 76 -> 80 / 74 % of peak, [128, 2048, 512] 72 / 70 -> 78 / 75 %, bf16
@@ -774,6 +791,31 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         if (C == kWave) l->vec = 1;
         else if (half_possible) l->vec = 2;
     }
+    // Fewer than 64 channels and two or more workgroups per CU, measured again over every plan: fp32 up to 32
+    // channels in 16-byte lanes, 4 steps, 4 waves ([540, 4225, 8] 68 / 105 -> 53 / 96 us, [907, 3157, 24] 220 / 356 ->
+    // 201 / 325 us, [929, 1083, 16] 50 / 73 -> 46 / 69 us; backwards from one workgroup per CU on: [306, 6590, 16] 164 ->
+    // 135 us, forwards 97 -> 121 us). 33 to 63 channels: forwards a single channel per lane (fp32 16 steps in 8 waves:
+    // [2048, 512, 40] 114 -> 92 us, [1024, 1024, 48] 126 -> 104 us; bf16 [2048, 512, 40] 87 -> 74 us, [1024, 1024, 48]
+    // 88 -> 76 us), backwards 16-byte lanes of fp32 (190 -> 172 us, 214 -> 211 us) and four-channel lanes of 16-bit
+    // storage (135 -> 125 us, 137 -> 126 us), in 4 waves.
+    bool small_fours = false, small_singles = false;
+    if (!u.vec && u.mode != kModeLookback && C < kWave && esize == 4) {
+        if (C <= 32 ? (vec_possible && batch >= (rev ? 256 : 512)) : (vec_possible && rev && batch >= 512)) {
+            l->vec = full;
+            small_fours = true;
+        } else if (C > 32 && !rev && batch >= 512) {
+            l->vec = 1;
+            small_singles = true;
+        }
+    }
+    if (!u.vec && u.mode != kModeLookback && C < kWave && C > 32 && esize == 2 && batch >= 512) {
+        if (!rev) {
+            l->vec = 1;
+        } else if (half_possible && T >= 512) {  // (shorter rows keep pairs: [5159, 257, 40] 194 against 224 us, [827, 388, 40] 55 against 59 us)
+            l->vec = half;
+            small_fours = true;
+        }
+    }
     if (l->vec != 1 && l->vec != full && !(l->vec == 2 && esize == 2) && !(half > 1 && l->vec == half)) return SCANSCAM_EPLAN;
     // A forced wide lane that the alignment or C does not allow as it stands: element-aligned, where that kernel applies.
     if (u.vec && ((l->vec == full && full > 1 && !vec_possible) || (l->vec == 2 && esize == 2 && full != 2 && !pair_possible) ||
@@ -788,7 +830,21 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     int64_t rowgroups = batch * groups(l->vec);
     l->kind = 0;
     const bool wide_enough = esize == 2 ? l->vec == 2 : l->vec > 1;  // pairs of 16-bit channels, 8- or 16-byte fp32 lanes
-    if (u.mode == kModeLookback || (u.mode == SCANSCAM_MODE_AUTO && rowgroups < (wide_enough ? enough : 256))) l->kind = 2;
+    // (Up to 32 channels a wave of the tiles' kernel is mostly empty lanes, and the walk, which packs several time steps
+    // into a wave, is ahead from 80 workgroups on: fp32 [128, 8192, 16] 99 / 168 -> 68 / 94 us, [200, 4000, 24] backward
+    // 138 -> 98 us, [95, 8181, 16] 82 / 132 -> 72 / 96 us, bf16 [128, 8192, 16] 125 / 273 -> 65 / 90 us; at 64 workgroups the
+    // tiles are ahead forwards and level backwards.)
+    const int64_t walk_from = C <= 32 ? 80 : (wide_enough ? enough : 256);
+    if (u.mode == kModeLookback || (u.mode == SCANSCAM_MODE_AUTO && rowgroups < walk_from)) l->kind = 2;
+    // (Those tiles of 16-bit storage in single channels, 16 lanes of a wave rather than 8: bf16 [64, 16384, 16] forward
+    // 135 -> 103 us, backward 283 -> 187 us.)
+    // (And wherever pairs would fill their waves to less than 70 % and single channels do better: [73, 14486, 40]
+    // 149 / 296 -> 114 / 211 us, [84, 7773, 56] 96 / 183 -> 76 / 146 us, [92, 1781, 56] 30 / 55 -> 25 / 42 us.)
+    if (l->kind == 2 && !u.vec && esize == 2 && l->vec == 2 &&
+        (C <= 32 || (groups(2) * kWave * 2 * 7 > C * 10 && groups(2) * 2 > groups(1)))) {
+        l->vec = 1;
+        rowgroups = batch * groups(1);
+    }
     if (u.mode == kModeSmall) return SCANSCAM_EPLAN;
     // A few more than 256 workgroups (up to 340) leave some CUs with twice the work of the others. Tiles over
     // workgroups are taken instead, with the lanes that measure best there in each direction (below): fp32
@@ -803,8 +859,11 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // channel -- of 16-bit storage backwards only: fp32 [300, 1024, 256] forward 192 -> 167 us, [400, 1024, 256] 247 ->
     // 216 us, [150, 2048, 512] 351 -> 324 us, [300, 1000, 77] 112 / 206 -> 92 / 169 us, bf16 backward 147 -> 125 us.)
     const bool to_08 = C >= 64 && (esize == 4 ? (!rev || l->vec == 1) : (rev && l->vec == 1));
-    const bool few_too_many = l->kind == 0 && !u.vec && u.mode == SCANSCAM_MODE_AUTO && !l->ragged && rowgroups > 256 &&
-                              rowgroups * 10 < rounds_up * kComputeUnits * (to_08 ? 8 : 7) && T >= 512 && C >= 40;
+    // (fp32 in element-aligned lanes as well, which then gives way to tiles of single channels: [14, 3757, 2539], 280
+    // workgroups of pairs, 511 / 929 -> 392 / 668 us, [24, 3000, 1473] 385 / 703 -> 311 / 529 us, [48, 2000, 777] 238 / 436 ->
+    // 217 / 362 us; 16-bit storage gains nothing there.)
+    const bool few_too_many = l->kind == 0 && !u.vec && u.mode == SCANSCAM_MODE_AUTO && (!l->ragged || esize == 4) && rowgroups > 256 &&
+                              rowgroups * 10 < rounds_up * kComputeUnits * (to_08 && !l->ragged ? 8 : 7) && T >= 512 && C >= 40;
     // (16-bit storage backwards only where four-channel lanes, the ones its tiles need, fill their waves.)
     // (filling them to 85 %: bf16 C = 1600, 89 %, gains 11 % backwards in such tiles, C = 640, 83 %, loses 8 %)
     const bool half_fits = half_possible && C >= (int64_t)kWave * half && C * 20 >= groups(half) * kWave * half * 17;
@@ -818,9 +877,15 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // tiles are of pairs, not of the four-channel lanes the walk chose: [24, 2048, 3072] 220 -> 197 us, [130, 2048, 512]
     // 200 -> 173 us.)
     const bool pairs_fill_fwd = C < kWave || groups(2) * kWave * 2 * 17 <= C * 20;
-    if (few_too_many && !(esize == 2 && rev && !half_fits && pairs_fill && groups(2) < 8) &&
-        !(esize == 2 && !rev && !pairs_fill_fwd)) {
+    // (Neither exception where the walk would be in single channels: bf16 [77, 11371, 212], 308 workgroups of them,
+    // 544 / 941 us.)
+    if (few_too_many && !(esize == 2 && rev && l->vec != 1 && !half_fits && pairs_fill && groups(2) < 8) &&
+        !(esize == 2 && !rev && l->vec != 1 && !pairs_fill_fwd)) {
         l->kind = 2;
+        if (l->ragged) {
+            l->vec = 1;
+            l->ragged = false;
+        }
         if (l->vec == full && full > 1) l->vec = narrow;
         if (esize == 2 && !rev && l->vec == half) l->vec = narrow;
         // single channels where the lane chosen so far leaves more than 30 % of its waves empty and they do better
@@ -874,16 +939,22 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     const bool narrow_lane = l->vec < full;
     // (element-aligned pairs of 16-bit channels likewise: bf16 [64, 2048, 1001] 36 / 34 -> 39 / 38 % of peak)
     // (and of fp32 channels: [512, 512, 333] backward 502 -> 390 us, [256, 1024, 777] 1246 -> 962 us, [128, 1024, 1003] 747 -> 664 us)
-    const bool long_steps = l->kind != 0 || (esize == 2 && l->vec <= 2 && T >= 1024 && (rowgroups < 512 || (l->ragged && l->vec == 2))) ||
+    // (Several time steps per wave, the packed kernel: only up to one workgroup per CU -- bf16 [306, 6590, 16] 117 / 163 us
+    // with 16 steps, 84 / 107 us with 8; [128, 8192, 16] 65 / 90 against 70 / 89 us.)
+    const bool long_steps = l->kind != 0 ||
+                            (esize == 2 && l->vec <= 2 && T >= 1024 && (rowgroups < 512 || (l->ragged && l->vec == 2)) &&
+                             (l->group == kWave || rowgroups <= kComputeUnits)) ||
+                            small_singles ||
                             (esize == 4 && l->ragged && l->vec == 2) ||
                             // (with loads issued a tile ahead, every walk in narrow 16-bit lanes whose time step fills its
                             // waves' lanes: bf16 [512, 1024, 256] 148 / 257 -> 145 / 238 us, [2048, 512, 128] backward 256 ->
                             // 237 us, [512, 1024, 320] 184 / 331 -> 179 / 309 us, [1024, 1024, 64] backward 142 -> 124 us)
                             // Rows shorter than a few such tiles lose: [4096, 128, 128] backward 114 -> 127 us, [1500, 100, 130]
                             // 38 / 64 -> 45 / 84 us, element-aligned [700, 300, 257] 82 / 143 -> 94 / 188 us; the single channels of
-                            // 64 gain forwards from one tile on: [4096, 128, 64] 48 -> 35 us, [1024, 200, 64] 20.5 -> 18.2 us.
+                            // 64 or fewer gain forwards from one tile on: [4096, 128, 64] 48 -> 35 us, [1024, 200, 64] 20.5 -> 18.2 us,
+                            // [5159, 257, 40] 134 -> 101 us.
                             (esize == 2 && l->vec <= 2 && l->kind == 0 && l->group == kWave && !l->ragged &&
-                             T >= (l->vec == 1 && C == kWave ? (rev ? 256 : 128) : 512));
+                             T >= (l->vec == 1 && C <= kWave ? (rev ? 256 : 128) : 512));
     l->steps = u.unroll ? u.unroll : (narrow_lane ? (long_steps ? 16 : 8) : ((l->kind != 0 && full <= 4) ? 8 : 4));
     // Tiles of 8-byte fp32 lanes backwards (kept from the choice above where there are a few workgroups too many):
     // 8 steps, which fit 104 registers where 16 need 129 (fp32 [520, 2000, 96] 504 -> 438 us).
@@ -897,7 +968,8 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     if (!u.unroll && wide_rows_fwd) l->steps = 16;
     // Packed, 4 or more steps per instruction: 4 instructions per wave with one channel per lane; lanes of two
     // channels keep 8 (bf16 [4096, 1024, 8] 41 / 41 -> 47 / 60 % of peak, [512, 4096, 24] 31 / 33 -> 37 / 44 %).
-    if (!u.unroll && l->group <= 16 && l->vec == 1) l->steps = 4;
+    // (From one workgroup per CU on: fp32 [128, 8192, 16] 84 / 125 us with 4 steps, 67 / 94 us with 8.)
+    if (!u.unroll && l->group <= 16 && l->vec == 1 && rowgroups >= kComputeUnits) l->steps = 4;
     const bool steps_ok = (l->vec == full) ? (l->steps == 2 || l->steps == 4 || l->steps == 8)
                                            : (l->steps == 4 || l->steps == 8 || l->steps == 16);
     if (!steps_ok) return SCANSCAM_EPLAN;
@@ -950,6 +1022,8 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         if (wide_rows_fwd && !u.unroll && C >= 4096 && l->waves > 4) l->waves = 4;
         if (l->kind == 0 && esize == 4 && rev && l->vec == full && !l->ragged && C >= 2048 && T <= 512 && l->waves > 4)
             l->waves = 4;
+        if (l->kind == 0 && small_fours && l->waves > 4) l->waves = 4;
+        if (l->kind == 0 && small_singles && l->waves > 8) l->waves = 8;
         while (l->waves > max_waves) l->waves >>= 1;
     }
     if (l->waves < 1 || l->waves > max_waves) return SCANSCAM_EPLAN;
@@ -1027,6 +1101,18 @@ int run_cl(bool rev, const void *a, const void *x, const void *h, void *y0, void
     bool lines = true;
     for (int k = 0; k < 5; k++) lines = lines && (sT[k] * esize) % 128 == 0 && aligned_to(ptrs[k], 128) && (sB[k] * esize) % 128 == 0;
     args.xcd_order = (!lines && l.grid >= 64) ? 1 : 0;
+    // Tiles over workgroups: a (batch element, channel group) pair keeps its XCD over all its tiles when their number
+    // is a multiple of 8. Otherwise, from 128 pairs on, the XCDs take runs of n / 8 rounded up or down and the grid is
+    // padded to 8 equal shares; the workgroups of a short run's last share return at once. (fp32 [9, 5318, 2059], 297
+    // pairs dealt round-robin over the XCDs tile by tile: 401 / 706 us.)
+    if (args.xcd_order && l.kind == 2) {
+        const int64_t pairs = l.grid / l.segments;
+        if (pairs % 8 != 0 && pairs >= 128) {
+            args.xcd_order = 2;
+            l.grid = 8 * ((pairs + 7) / 8) * l.segments;
+            if (l.grid >= (int64_t(1) << 31)) return SCANSCAM_EINVAL;
+        }
+    }
     // Lanes of 8 bytes or less whose time steps are no whole lines write partial lines at both ends of every
     // wave's store; non-temporal stores then cost 20 % of a plain copy's rate and stores left to the caches'
     // normal policy nothing. Measured on the kernels: 16-bit storage 8 to 35 % faster in both directions (bf16

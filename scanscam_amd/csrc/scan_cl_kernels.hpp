@@ -711,8 +711,20 @@ __global__ __launch_bounds__(MAXT) void scan_cl_lookback_kernel(const ClArgs p)
     // Row-groups of a workgroup's XCD: with p.xcd_order (time steps that are not whole 128-byte lines) a
     // contiguous run of them, so that channel groups that share a line meet in one L2 (as in scan_cl_kernel;
     // exact when the number of row-groups is a multiple of 8, where a row-group keeps its XCD over all tiles).
-    const int64_t rg0 = blockIdx.x % rowgroups;
-    const int64_t rg = (p.xcd_order && rowgroups % 8 == 0) ? xcd_contiguous((int)rg0, (int)rowgroups) : rg0;
+    // (xcd_order 2, any number of row-groups: XCD x = blockIdx % 8 owns the x-th run of them, of n / 8 rounded up or
+    // down, and its workgroups go round that run; the host pads the grid to 8 shares of the longer run's size, so the
+    // last workgroups of a shorter run's XCD have nothing to do.)
+    int64_t rg;
+    if (p.xcd_order == 2) {
+        const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
+        const int per = (int)((rowgroups + 7) / 8), rem = rowgroups % 8 == 0 ? 8 : (int)(rowgroups % 8);
+        const int mine = xcd < rem ? per : per - 1;
+        if (slot >= mine * tpr) return;
+        rg = (xcd < rem ? xcd * per : rem * per + (xcd - rem) * (per - 1)) + slot % mine;
+    } else {
+        const int64_t rg0 = blockIdx.x % rowgroups;
+        rg = (p.xcd_order && rowgroups % 8 == 0) ? xcd_contiguous((int)rg0, (int)rowgroups) : rg0;
+    }
     if (threadIdx.x == 0)
         lds_ticket = __hip_atomic_fetch_add(reinterpret_cast<unsigned *>(p.ws + rg * kCounterStride), 1u,
                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -4,6 +4,8 @@ Time the library's automatic launch plan for a shape against a set of forced pla
     python -m scanscam_amd.plan_search rows 8192x4096 2047x16385:bf16 ...
     python -m scanscam_amd.plan_search cl 8x4096x512:bf16 64x2048x1001 ...
     python -m scanscam_amd.plan_search --suite cl-a | cl-b | cl-odd | rows-23 | rows-25 | rows-26
+    python -m scanscam_amd.plan_search --random 40 --seed 3      (channels-last shapes drawn at random, and the
+                                                                  distribution of automatic / best over them)
 
 ``rows`` shapes are contiguous ``[rows, T]`` tensors scanned along ``T`` (the layout of
 ``simple_linear_scan`` and its siblings, ``scanscam/cuda.py:28-64`` in the reference), ``cl`` shapes are
@@ -22,6 +24,7 @@ The same search serves a caller who wants the best plan for one fixed shape: pas
 ``plan=`` argument of the calls in ``scanscam_amd.hip`` (``struct scanscam_plan`` in the C interface).
 """
 import argparse
+import random
 import sys
 
 import torch
@@ -85,13 +88,29 @@ def cl_plans(dtype, C):
     most = 16 if full == 4 else 8  # waves that the kernels' LDS arrays allow with 16-byte lanes
     out = [P(vec=v, unroll=s, waves=w, mode=walk)
            for v, s, w in ((full, 4, most), (full, 4, 4), (half, 8, 8), (half, 8, 4), (half, 16, 8), (half, 16, 4),
-                           (narrow, 8, 8 * (3 - narrow)), (narrow, 16, 8), (1, 8, 16)) if C % v == 0]
+                           (narrow, 8, 8 * (3 - narrow)), (narrow, 16, 8), (1, 8, 16), (1, 16, 8)) if C % v == 0]
     if C % full != 0:  # lanes wider than the channel count divides: taken where a time step fills a wave of them
         out += [P(vec=v, unroll=s, waves=w, mode=walk)
                 for v, s, w in ((full, 4, most), (full, 4, 4), (half, 8, 8), (half, 8, 4), (2, 16, 8), (2, 8, 8))
                 if C % v != 0 and C >= 64 * v]
     out += [P(vec=v, unroll=s, waves=w, mode=split)
             for v, s, w in ((narrow, 16, 8), (half, 16, 8), (half, 8, 8), (1, 16, 8)) if C % v == 0]
+    return out
+
+
+def random_cl_shapes(n, seed):
+    """n shapes [batch, T, C]: C from 8 to 5000 and T from 64 to 16384, both log-uniform, half of the channel counts
+    rounded to multiples of 8; 8 M to 190 M elements; batch what that leaves, 1 to 8192."""
+    rng = random.Random(seed)
+    out = []
+    while len(out) < n:
+        C = int(round(2 ** rng.uniform(3, 12.3)))
+        if rng.random() < 0.5:
+            C = max(8, (C + 4) // 8 * 8)
+        T = int(round(2 ** rng.uniform(6, 14)))
+        batch = int(2 ** rng.uniform(23, 27.5) / (T * C))
+        if 1 <= batch <= 8192:
+            out.append((batch, T, C))
     return out
 
 
@@ -170,6 +189,8 @@ def main(argv=None):
     ap.add_argument("layout", nargs="?", choices=("rows", "cl"))
     ap.add_argument("shapes", nargs="*", metavar="SHAPE[:dtype]")
     ap.add_argument("--suite", choices=sorted(SUITES), help="a fixed list of shapes, each in f32 and bf16")
+    ap.add_argument("--random", type=int, metavar="N", help="N channels-last shapes drawn at random, each in f32 and bf16")
+    ap.add_argument("--seed", type=int, default=0, help="seed of --random")
     ap.add_argument("--reps", type=int, default=24)
     ap.add_argument("--every", action="store_true", help="also print every plan's timings")
     args = ap.parse_intermixed_args(argv)  # options may stand between the layout and the shapes
@@ -181,19 +202,27 @@ def main(argv=None):
     if args.suite:
         layout, shapes = SUITES[args.suite]
         jobs = [(layout, s, dt) for s in shapes for dt in (torch.float32, torch.bfloat16)]
+    elif args.random:
+        jobs = [("cl", s, dt) for s in random_cl_shapes(args.random, args.seed) for dt in (torch.float32, torch.bfloat16)]
     elif args.layout is None:
-        ap.error("give a layout and shapes, or --suite")
+        ap.error("give a layout and shapes, --suite or --random")
     for spec in args.shapes:
         shape_s, _, dtype_s = spec.partition(":")
         shape = tuple(int(v) for v in shape_s.lower().split("x"))
         if len(shape) != (2 if args.layout == "rows" else 3):
             ap.error(f"{spec}: a {args.layout} shape has {2 if args.layout == 'rows' else 3} sizes")
         jobs.append((args.layout, shape, DTYPES[dtype_s]))
-    behind = 0
+    ratios = []
     for layout, shape, dtype in jobs:
         res = search(layout, shape, dtype, reps=args.reps, every=args.every)
-        behind += sum(auto > 1.08 * best for auto, best, _ in res.values())
+        ratios += [auto / best for auto, best, _ in res.values()]
+    behind = sum(r > 1.08 for r in ratios)
     print(f"{2 * len(jobs)} timings, automatic plan more than 8 % behind the set's best in {behind}", flush=True)
+    if args.random and ratios:
+        ratios.sort()
+        print(f"automatic / best: median {ratios[len(ratios) // 2]:.3f}, mean {sum(ratios) / len(ratios):.3f}, "
+              f"above 1.15 in {sum(r > 1.15 for r in ratios)}, above 1.3 in {sum(r > 1.3 for r in ratios)}, "
+              f"largest {ratios[-1]:.2f}", flush=True)
 
 
 if __name__ == "__main__":

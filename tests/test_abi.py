@@ -220,7 +220,14 @@ WALK, TILES = hip.MODE_ROW, hip.MODE_LOOKBACK
         ((96, 1024, 1003), torch.float32, (WALK, 4, 4, 4), (WALK, 4, 4, 4)),      # fp32 keeps its 16-byte lanes
         ((300, 1024, 256), torch.float32, (TILES, 2, 16, 8), (WALK, 2, 8, 4)),    # 600 workgroups: 0.78 of three rounds
         ((300, 1000, 77), torch.bfloat16, (WALK, 1, 16, 8), (TILES, 1, 16, 8)),
-        ((2048, 512, 40), torch.float32, (WALK, 2, 8, 8), (WALK, 2, 8, 8)),       # several time steps per instruction
+        ((2048, 512, 40), torch.float32, (WALK, 1, 16, 8), (WALK, 4, 4, 4)),      # 33 to 63 channels, two workgroups per CU or more
+        ((2048, 512, 40), torch.bfloat16, (WALK, 1, 16, 8), (WALK, 4, 8, 4)),
+        ((540, 4225, 8), torch.float32, (WALK, 4, 4, 4), (WALK, 4, 4, 4)),        # several time steps per instruction
+        ((306, 6590, 16), torch.float32, (WALK, 2, 8, 8), (WALK, 4, 4, 4)),
+        ((128, 8192, 16), torch.bfloat16, (WALK, 2, 16, 8), (WALK, 2, 16, 8)),    # ... walked from 100 workgroups on
+        ((64, 16384, 16), torch.bfloat16, (TILES, 1, 16, 8), (TILES, 1, 16, 8)),
+        ((209, 221, 1370), torch.bfloat16, (WALK, 4, 8, 8), (WALK, 4, 8, 8)),     # short rows, element-aligned: 8-byte lanes
+        ((71, 1910, 257), torch.bfloat16, (TILES, 1, 16, 8), (WALK, 2, 16, 8)),   # 213 workgroups of element-aligned pairs backwards
         ((128, 512, 2048), torch.float32, (WALK, 2, 16, 8), (WALK, 4, 4, 4)),     # 2048 or more fp32 channels
         ((256, 1024, 256), torch.float64, (WALK, 1, 8, 8), (WALK, 1, 8, 8)),      # float64: its 8-byte lane is one channel
         ((8, 4096, 512), torch.float64, (TILES, 1, 16, 8), (TILES, 1, 8, 8)),
@@ -232,7 +239,7 @@ def test_automatic_channels_last_plan_per_regime(shape, dtype, fwd, bwd):
         plan = hip.resolve_plan_cl(*shape, dtype, direction)
         assert (plan.mode, plan.vec, plan.unroll, plan.waves) == want, (direction, plan)
         ws = hip.workspace_bytes_cl(*shape, dtype, direction)
-        assert (ws > 0) == (want[0] == TILES)
+        assert ws > 0 or want[0] != TILES  # (the size covers tensors of any alignment, so it may be non-zero for a walk)
 
 
 def test_every_automatic_channels_last_plan_is_a_valid_plan():

@@ -203,6 +203,37 @@ def test_time_split_is_chosen_for_few_channels_and_is_reproducible(gpu):
     assert torch.equal(ga0, ga1) and torch.equal(gb0, gb1)
 
 
+@pytest.mark.parametrize("dtype,shape,vec", [
+    (torch.float32, (9, 700, 2059), 1),    # 297 (batch element, channel group) pairs: runs of 38 and 37 per XCD
+    (torch.float32, (131, 300, 100), 1),   # 131 pairs of two steps' worth of tiles
+    (torch.bfloat16, (17, 600, 515), 1),   # 153 pairs
+    (torch.bfloat16, (43, 500, 772), 4),   # 172 pairs of four-channel lanes, time steps of 1544 bytes
+    (torch.float32, (3, 900, 300), 1),     # 15 pairs: too few for runs, dealt round-robin
+])
+def test_time_split_with_pairs_that_are_no_multiple_of_eight(gpu, dtype, shape, vec):
+    # Time steps that are no whole 128-byte lines: each XCD takes a contiguous run of the (batch element, channel group)
+    # pairs and every tile of them; with a pair count that is no multiple of 8 the runs differ in length and the grid
+    # is padded, so some workgroups have nothing to do. Every tile of every pair must still be handed out exactly once.
+    bar = 1e-5 if dtype == torch.float32 else 1e-2
+    g = torch.Generator().manual_seed(sum(shape))
+    a = torch.rand(shape, generator=g, dtype=torch.float64).to(dtype)
+    b = torch.randn(shape, generator=g, dtype=torch.float64).to(dtype)
+    gh = torch.randn(shape, generator=g, dtype=torch.float64).to(dtype)
+    h = oracle.fwd(as_rows(a), as_rows(b))
+    hs = torch.from_numpy(h).mT.contiguous().to(dtype)
+    ga, gb = oracle.bwd(as_rows(a), as_rows(hs), as_rows(gh))
+    hp = prev_abs(as_rows(hs))
+    for waves in (2, 8):
+        plan = hip.Plan(vec=vec, unroll=16, waves=waves, mode=hip.MODE_LOOKBACK)
+        print(f"case cl time split {dtype} shape={shape} {plan}", flush=True)
+        for _ in range(2):
+            got_h = hip.transposed_linear_scan_forward(a.to(gpu), b.to(gpu), plan=plan)
+            got_ga, got_gb = hip.transposed_linear_scan_backward(a.to(gpu), hs.to(gpu), gh.to(gpu), plan=plan)
+            assert rel_err(as_rows(got_h), h) <= bar
+            assert rel_err(as_rows(got_gb), gb) <= bar
+            assert rel_err(as_rows(got_ga), ga, hp) <= bar
+
+
 def test_expired_wait_is_reported_and_every_wave_exits(gpu):
     # One poll allowed: the launch must still complete; either all waits succeeded in that poll or
     # word 1 of the workspace is raised and the poisoned outputs are NaN.

@@ -209,6 +209,13 @@ def test_plan_search_sets_hold_plans_the_library_knows():
                 assert any(L.scanscam_resolve_plan_cl(batch, 2048, C, code, hip.FORWARD, ctypes.byref(plan), ctypes.byref(out)) == 0
                            for batch in (8, 512)), (C, plan)
     assert {"cl-a", "cl-b", "cl-odd", "rows-25"} <= set(plan_search.SUITES)
+    # The random audit: the same shapes for the same seed, inside the stated bounds, and resolvable by the library.
+    shapes = plan_search.random_cl_shapes(30, 3)
+    assert shapes == plan_search.random_cl_shapes(30, 3) and shapes != plan_search.random_cl_shapes(30, 4)
+    for batch, T, C in shapes:
+        assert 1 <= batch <= 8192 and 64 <= T <= 16384 and 8 <= C <= 5100 and batch * T * C <= 1 << 28
+        for dtype in (torch.float32, torch.bfloat16):
+            assert hip.resolve_plan_cl(batch, T, C, dtype, hip.BACKWARD).waves >= 1
 
 
 def test_bench_refuses_more_than_one_gpu():
