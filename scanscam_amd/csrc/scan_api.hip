@@ -892,6 +892,22 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         if (groups(l->vec) * kWave * l->vec * 7 > C * 10 && groups(l->vec) * l->vec > groups(1)) l->vec = 1;
         rowgroups = batch * groups(l->vec);
     }
+    // fp32 backwards in single channels on time steps that are no whole 128-byte lines: the walk of all of T runs at
+    // 35-40 % of peak whatever the number of workgroups, tiles over time at 45-50 % -- [476, 1998, 113] 770 -> 587 us,
+    // [551, 3705, 59] 779 -> 557 us, [1000, 500, 130] 434 -> 358 us, [986, 969, 157] 931 -> 769 us, [438, 1181, 93] 327 ->
+    // 272 us, [100, 3000, 300] 553 -> 442 us. (Whole lines, [1024, 1024, 64], gain nothing.)
+    // (Pairs likewise, element-aligned ones giving way to single channels: [90, 2048, 514] 532 -> 442 us, [1429, 456, 202]
+    // 804 -> 677 us, [84, 1772, 216] 168 -> 137 us, [32, 4096, 999] 731 -> 652 us.)
+    // (From 384 steps on -- [1599, 379, 79] and [228, 402, 94] gain 11 and 22 % -- and element-aligned pairs from 2048:
+    // [512, 512, 333] is 13 % faster in their walk. Tiles of pairs where those fill their waves within 10 % of single
+    // channels: [1000, 500, 130] 425 us in pairs, 352 us in single channels.)
+    if (l->kind == 0 && !u.vec && u.mode == SCANSCAM_MODE_AUTO && esize == 4 && rev && l->vec <= 2 && C > 32 &&
+        T >= (l->ragged ? 2048 : 384) && (C * esize) % 128 != 0) {
+        l->kind = 2;
+        l->vec = (half_possible && groups(2) * 2 * 9 <= groups(1) * 10) ? 2 : 1;  // ([90, 2048, 514]: 436 us in pairs, 462 us in single channels)
+        l->ragged = false;
+        rowgroups = batch * groups(l->vec);
+    }
     // Tiles over workgroups, lanes chosen here: 8-byte lanes where C fills whole waves of them, in the
     // direction in which they measured faster than the narrow lane (16 steps per wave either way) -- the
     // backward pass of 16-bit storage (bf16 [8, 4096, 512] 48 -> 38 us, [8, 4096, 2048] 166 -> 140 us,
