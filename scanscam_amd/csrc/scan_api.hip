@@ -899,12 +899,16 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // (Pairs likewise, element-aligned ones giving way to single channels: [90, 2048, 514] 532 -> 442 us, [1429, 456, 202]
     // 804 -> 677 us, [84, 1772, 216] 168 -> 137 us, [32, 4096, 999] 731 -> 652 us.)
     // (From 384 steps on -- [1599, 379, 79] and [228, 402, 94] gain 11 and 22 % -- and element-aligned pairs from 2048:
-    // [512, 512, 333] is 13 % faster in their walk. Tiles of pairs where those fill their waves within 10 % of single
+    // [512, 512, 333] is 13 % faster in their walk. Tiles of pairs where those fill their waves within 20 % of single
     // channels: [1000, 500, 130] 425 us in pairs, 352 us in single channels.)
-    if (l->kind == 0 && !u.vec && u.mode == SCANSCAM_MODE_AUTO && esize == 4 && rev && l->vec <= 2 && C > 32 &&
-        T >= (l->ragged ? 2048 : 384) && (C * esize) % 128 != 0) {
+    // (Forwards the walk holds up on rows of about 1000 steps and the tiles are 10 to 20 % ahead from about 2000 on:
+    // [476, 1998, 113] 379 -> 344 us, [551, 3705, 59] 359 -> 319 us, [107, 2371, 206] 159 -> 130 us, [90, 2048, 514] 298 ->
+    // 256 us; [986, 969, 157] and [438, 1181, 93] are level, and element-aligned pairs keep their walk.)
+    if (l->kind == 0 && !u.vec && u.mode == SCANSCAM_MODE_AUTO && esize == 4 && l->vec <= 2 && C > 32 &&
+        (rev ? T >= (l->ragged ? 2048 : 384) : (T >= 1900 && !l->ragged)) && (C * esize) % 128 != 0) {
         l->kind = 2;
-        l->vec = (half_possible && groups(2) * 2 * 9 <= groups(1) * 10) ? 2 : 1;  // ([90, 2048, 514]: 436 us in pairs, 462 us in single channels)
+        // ([90, 2048, 514]: 436 us in pairs, 462 us in single channels; [100, 3000, 300], 0.83 of the fill: 265 / 439 against 288 / 476 us)
+        l->vec = (half_possible && groups(2) * 2 * 8 <= groups(1) * 10) ? 2 : 1;
         l->ragged = false;
         rowgroups = batch * groups(l->vec);
     }
