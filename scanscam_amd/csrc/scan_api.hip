@@ -973,7 +973,11 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
                             // 38 / 64 -> 45 / 84 us, element-aligned [700, 300, 257] 82 / 143 -> 94 / 188 us; the single channels of
                             // 64 or fewer gain forwards from one tile on: [4096, 128, 64] 48 -> 35 us, [1024, 200, 64] 20.5 -> 18.2 us,
                             // [5159, 257, 40] 134 -> 101 us.
+                            // (Nor do single channels backwards on an odd number of channels above 64, which stay with 16 waves of 8 steps:
+                            // [2000, 1000, 65] 664 against 810 us, [438, 1181, 93] 236 against 269 us, [1599, 379, 79] 215 us against
+                            // 256 us in 4 waves.)
                             (esize == 2 && l->vec <= 2 && l->kind == 0 && l->group == kWave && !l->ragged &&
+                             !(rev && l->vec == 1 && !pair_possible && groups(1) >= 2) &&
                              T >= (l->vec == 1 && C <= kWave ? (rev ? 256 : 128) : 512));
     l->steps = u.unroll ? u.unroll : (narrow_lane ? (long_steps ? 16 : 8) : ((l->kind != 0 && full <= 4) ? 8 : 4));
     // Tiles of 8-byte fp32 lanes backwards (kept from the choice above where there are a few workgroups too many):
@@ -1028,7 +1032,7 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         if (l->kind == 0 && esize == 2 && l->waves > 4 && !l->ragged) {
             if (l->vec == half && l->group == kWave && groups(half) == 1) l->waves = 4;
             if (l->vec == 2 && C == kWave && rowgroups >= 2 * kComputeUnits) l->waves = 4;  // ([256, 4096, 64] backward: 220 us with 4 waves, 154 us with 8)
-            if (l->vec == 1 && rev && groups(1) >= 2 && l->steps != 16) l->waves = 4;
+            if (l->vec == 1 && rev && groups(1) >= 2 && l->steps != 16 && pair_possible) l->waves = 4;
             // Single channels with 16 steps: 8 waves from two workgroups per CU on ([4096, 256, 64] forward 90 us
             // with 16 waves, 65 us with 8; [256, 4096, 64], one per CU, level).
             if (l->vec == 1 && l->steps == 16 && rowgroups >= 2 * kComputeUnits && l->waves > 8) l->waves = 8;
