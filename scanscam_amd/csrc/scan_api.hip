@@ -620,7 +620,7 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // the CUs (two thirds backwards), not all 256 -- at 176 to 255 workgroups they still beat twice as many
     // workgroups of the next narrower lane (fp32 [28, 4096, 1024] 287 / 473 -> 261 / 388 us, [24, 4096, 1024] 261 / 442 ->
     // 228 / 361 us, bf16 [28, 4096, 2048] 300 / 513 -> 278 / 430 us, [56, 2048, 512] forward 81 -> 70 us).
-    const int64_t enough = rev ? 168 : 192;
+    const int64_t enough = rev ? 168 : 176;  // (forwards 192 at first: bf16 [189, 4702, 82], 189 workgroups of pairs, 123 us against 190 us in single channels)
     // Pairs halve the number of workgroups: not where single channels reach 256 of them and pairs fall short.
     const int narrow = pair_possible && (batch * groups(2) >= enough || batch * groups(1) < 256) ? 2 : 1;
     // Element-aligned lanes: where C is no multiple of the lane's channels, or the tensors are only element-aligned,
@@ -787,7 +787,8 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // at exactly 64. Against 16-byte lanes with 4 steps: [2048, 512, 40] 41 / 56 -> 56 / 56 % of peak, [1024, 1024, 48]
     // 47 / 59 -> 60 / 59 %, [512, 2048, 96] 54 / 61 -> 64 / 64 %, [256, 4096, 64] 60 / 68 -> 73 / 67 %; against single
     // channels with 4 steps: [4096, 1024, 8] 63 / 65 -> 73 / 72 %.
-    if (!u.vec && esize == 4 && C < 2 * kWave && batch >= 256 && u.mode != kModeLookback) {
+    // (From the `enough` workgroups of above on, not only from 256: [234, 1315, 72] forward 84 -> 64 us.)
+    if (!u.vec && esize == 4 && C < 2 * kWave && batch >= enough && u.mode != kModeLookback) {
         if (C == kWave) l->vec = 1;
         else if (half_possible) l->vec = 2;
     }
@@ -965,6 +966,11 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
                             (esize == 2 && l->vec <= 2 && T >= 1024 && (rowgroups < 512 || (l->ragged && l->vec == 2)) &&
                              (l->group == kWave || rowgroups <= kComputeUnits)) ||
                             small_singles ||
+                            // (fp32 forwards in single channels from two workgroups per CU on, with 8 waves: [3237, 206, 192] 295 ->
+                            // 255 us, [1704, 67, 85] 49 -> 38 us, [2106, 99, 64] 37 -> 29 us, [5005, 328, 21] 185 -> 149 us; on rows of
+                            // fewer than 512 steps -- [1024, 1024, 64] and [700, 512, 192] are level, [986, 969, 157] loses 26 %.
+                            // Backwards 16 waves of 8 steps stay ahead with few channels.)
+                            (esize == 4 && !rev && l->vec == 1 && l->kind == 0 && rowgroups >= 2 * kComputeUnits && T < 512) ||
                             (esize == 4 && l->ragged && l->vec == 2) ||
                             // (with loads issued a tile ahead, every walk in narrow 16-bit lanes whose time step fills its
                             // waves' lanes: bf16 [512, 1024, 256] 148 / 257 -> 145 / 238 us, [2048, 512, 128] backward 256 ->
@@ -978,7 +984,7 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
                             // 256 us in 4 waves.)
                             (esize == 2 && l->vec <= 2 && l->kind == 0 && l->group == kWave && !l->ragged &&
                              !(rev && l->vec == 1 && !pair_possible && groups(1) >= 2) &&
-                             T >= (l->vec == 1 && C <= kWave ? (rev ? 256 : 128) : 512));
+                             T >= (l->vec == 1 && C <= kWave ? (rev ? 256 : 64) : 512));
     l->steps = u.unroll ? u.unroll : (narrow_lane ? (long_steps ? 16 : 8) : ((l->kind != 0 && full <= 4) ? 8 : 4));
     // Tiles of 8-byte fp32 lanes backwards (kept from the choice above where there are a few workgroups too many):
     // 8 steps, which fit 104 registers where 16 need 129 (fp32 [520, 2000, 96] 504 -> 438 us).
@@ -1048,7 +1054,20 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
             l->waves = 4;
         if (l->kind == 0 && small_fours && l->waves > 4) l->waves = 4;
         if (l->kind == 0 && small_singles && l->waves > 8) l->waves = 8;
+        if (l->kind == 0 && esize == 4 && !rev && l->vec == 1 && l->steps == 16 && l->waves > 8) l->waves = 8;
         while (l->waves > max_waves) l->waves >>= 1;
+        // Rows of one or two tiles: no more waves than make those tiles equally full (75 steps in tiles of 8 waves x 8 steps
+        // are one full tile and one of 11 steps; 5 waves make two tiles of 40 and 35).
+        if (l->kind == 0) {
+            const int64_t tile = l->waves * wave_steps, tiles_now = (T + tile - 1) / tile;
+            if (tiles_now <= 2) {
+                const int64_t even = (segments + tiles_now - 1) / tiles_now;
+                // (Lanes of 8 bytes or more: 4 waves, three tiles for such a row -- bf16 [506, 75, 943] 63 / 117 us with 8 waves,
+                // 55 / 106 us with 5, 50 / 86 us with 4; single channels do best with the even split: fp32 [4526, 65, 432]
+                // 405 / 714 -> 289 / 503 us with 5 and 9 waves, [1704, 67, 85] 49 / 81 -> 32 / 72 us.)
+                if (even < l->waves) l->waves = (l->vec * esize >= 8 && l->group == kWave && even > 4) ? 4 : (int)even;
+            }
+        }
     }
     if (l->waves < 1 || l->waves > max_waves) return SCANSCAM_EPLAN;
 

@@ -358,6 +358,21 @@ MANY_WORKGROUPS = [
     (torch.float16, (300, 1, 1000), None),      # a single time step
     (torch.float32, (20, 300, 2048), None),     # fp32, 2048 or more channels: 16 steps per wave forwards, 16-byte lanes backwards
     (torch.float32, (10, 200, 4096), None),
+    (torch.float32, (600, 65, 432), None),      # rows of one or two tiles: waves that fill the tiles evenly (5 and 9 of them)
+    (torch.bfloat16, (520, 67, 85), None),      # ... single channels of 16-bit storage, 9 waves
+    (torch.float32, (700, 99, 64), None),       # ... 7 and 13 waves
+    (torch.bfloat16, (300, 75, 943), None),     # ... lanes of 8 bytes: three tiles of 4 waves
+    (torch.float32, (1200, 330, 21), None),     # ... two time steps per instruction, 6 and 11 waves
+    (torch.float32, (600, 500, 40), None),      # 33 to 63 channels: single channels forwards, 16-byte lanes backwards
+    (torch.bfloat16, (600, 520, 40), None),     # ... four-channel lanes backwards
+    (torch.float32, (520, 300, 8), None),       # up to 32 channels of fp32: 16-byte lanes, 4 steps, 4 waves
+    (torch.float32, (100, 1300, 24), None),     # ... the walk from 80 workgroups on
+    (torch.bfloat16, (64, 2100, 16), None),     # ... tiles of single 16-bit channels below that
+    (torch.float32, (260, 600, 113), None),     # fp32 off whole lines: tiles backwards from 384 steps on
+    (torch.float32, (60, 2000, 113), None),     # ... and forwards from 1900
+    (torch.float32, (14, 1100, 2539), None),    # element-aligned fp32 lanes, a few workgroups too many: tiles of single channels
+    (torch.bfloat16, (71, 600, 257), None),     # 16-bit backwards: 213 workgroups of element-aligned pairs
+    (torch.bfloat16, (39, 125, 4806), None),    # short rows, element-aligned: four-channel lanes
 ]
 
 
