@@ -788,7 +788,7 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // 47 / 59 -> 60 / 59 %, [512, 2048, 96] 54 / 61 -> 64 / 64 %, [256, 4096, 64] 60 / 68 -> 73 / 67 %; against single
     // channels with 4 steps: [4096, 1024, 8] 63 / 65 -> 73 / 72 %.
     // (From the `enough` workgroups of above on, not only from 256: [234, 1315, 72] forward 84 -> 64 us.)
-    if (!u.vec && esize == 4 && C < 2 * kWave && batch >= enough && u.mode != kModeLookback) {
+    if (!u.vec && esize == 4 && C < 2 * kWave && batch >= (C > 32 ? enough : 256) && u.mode != kModeLookback) {
         if (C == kWave) l->vec = 1;
         else if (half_possible) l->vec = 2;
     }
@@ -804,12 +804,12 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         if (C <= 32 ? (vec_possible && batch >= (rev ? 256 : 512)) : (vec_possible && rev && batch >= 512)) {
             l->vec = full;
             small_fours = true;
-        } else if (C > 32 && !rev && batch >= 512) {
+        } else if (C > 32 && !rev && batch >= enough) {  // (forwards from 176 workgroups on: [231, 773, 56] 37 -> 29 us, bf16 30 -> 20 us)
             l->vec = 1;
             small_singles = true;
         }
     }
-    if (!u.vec && u.mode != kModeLookback && C < kWave && C > 32 && esize == 2 && batch >= 512) {
+    if (!u.vec && u.mode != kModeLookback && C < kWave && C > 32 && esize == 2 && batch >= (rev ? 512 : enough)) {
         if (!rev) {
             l->vec = 1;
         } else if (half_possible && T >= 512) {  // (shorter rows keep pairs: [5159, 257, 40] 194 against 224 us, [827, 388, 40] 55 against 59 us)
@@ -835,7 +835,13 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // into a wave, is ahead from 80 workgroups on: fp32 [128, 8192, 16] 99 / 168 -> 68 / 94 us, [200, 4000, 24] backward
     // 138 -> 98 us, [95, 8181, 16] 82 / 132 -> 72 / 96 us, bf16 [128, 8192, 16] 125 / 273 -> 65 / 90 us; at 64 workgroups the
     // tiles are ahead forwards and level backwards.)
-    const int64_t walk_from = C <= 32 ? 80 : (wide_enough ? enough : 256);
+    // (17 to 32 channels fill a quarter to a half of a tile's wave, and there the tiles hold out up to 192 workgroups: fp32
+    // [139, 11578, 23] 237 / 352 us walked, 173 / 290 us in tiles, [123, 5560, 28] forward 102 against 76 us, [176, 9879, 19]
+    // 198 against 174 us; [200, 4000, 24] is level forwards and 40 % faster backwards in the walk.)
+    // (16-bit storage backwards keeps the walk: bf16 [123, 5560, 28] 115-133 us walked, [64, 16384, 16] 159 against 187 us.)
+    const bool one_wave_singles = l->vec == 1 && C > 32 && C < kWave;  // (33 to 63 channels forwards, above)
+    const int64_t walk_from = (C <= 16 || (C <= 32 && esize == 2 && rev)) ? 80
+                              : (C <= 32 ? 192 : ((wide_enough || one_wave_singles) ? enough : 256));
     if (u.mode == kModeLookback || (u.mode == SCANSCAM_MODE_AUTO && rowgroups < walk_from)) l->kind = 2;
     // (Those tiles of 16-bit storage in single channels, 16 lanes of a wave rather than 8: bf16 [64, 16384, 16] forward
     // 135 -> 103 us, backward 283 -> 187 us.)
@@ -843,6 +849,10 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // 149 / 296 -> 114 / 211 us, [84, 7773, 56] 96 / 183 -> 76 / 146 us, [92, 1781, 56] 30 / 55 -> 25 / 42 us.)
     if (l->kind == 2 && !u.vec && esize == 2 && l->vec == 2 &&
         (C <= 32 || (groups(2) * kWave * 2 * 7 > C * 10 && groups(2) * 2 > groups(1)))) {
+        l->vec = 1;
+        rowgroups = batch * groups(1);
+    }
+    if (l->kind == 2 && !u.vec && C <= 32 && l->vec != 1) {  // (fp32 likewise: [123, 5560, 28] forward 76 us)
         l->vec = 1;
         rowgroups = batch * groups(1);
     }
@@ -922,6 +932,14 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         l->vec = half;
         rowgroups = batch * groups(half);
     }
+    // Forwards, pairs in place of single channels wherever they fill their waves as well (half as many waves for the
+    // same channels): fp32 [51, 9920, 82] 163 -> 120 us, [160, 1995, 68] 84 -> 70 us, [42, 4018, 112] 64 -> 56 us, bf16
+    // [160, 1995, 68] 64 -> 50 us.
+    if (l->kind == 2 && !u.vec && !rev && l->vec == 1 && C > kWave && (esize == 2 ? pair_possible : half_possible) &&
+        esize <= 4 && groups(2) * 2 <= groups(1)) {
+        l->vec = 2;
+        rowgroups = batch * groups(2);
+    }
     // fp32 backwards on time steps that are no whole 128-byte lines: pairs of channels with 8 steps, where they
     // fill their waves as well as single channels do ([20, 8192, 250] 265 -> 214 us, [48, 2048, 1500] 860 -> 706 us,
     // [8, 4096, 1000] 178 -> 155 us, [260, 2000, 66] 305 -> 244 us; with whole lines single channels are level or ahead).
@@ -968,9 +986,11 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
                             small_singles ||
                             // (fp32 forwards in single channels from two workgroups per CU on, with 8 waves: [3237, 206, 192] 295 ->
                             // 255 us, [1704, 67, 85] 49 -> 38 us, [2106, 99, 64] 37 -> 29 us, [5005, 328, 21] 185 -> 149 us; on rows of
-                            // fewer than 512 steps -- [1024, 1024, 64] and [700, 512, 192] are level, [986, 969, 157] loses 26 %.
+                            // fewer than 512 steps -- [1024, 1024, 64] and [700, 512, 192] are level, [986, 969, 157] loses 26 % -- and
+                            // not on an odd number of channels above 64: [3964, 290, 89] 342 -> 413 us, though [1704, 67, 85] gains.
                             // Backwards 16 waves of 8 steps stay ahead with few channels.)
-                            (esize == 4 && !rev && l->vec == 1 && l->kind == 0 && rowgroups >= 2 * kComputeUnits && T < 512) ||
+                            (esize == 4 && !rev && l->vec == 1 && l->kind == 0 && rowgroups >= 2 * kComputeUnits && T < 512 &&
+                             (C % 2 == 0 || groups(1) == 1)) ||
                             (esize == 4 && l->ragged && l->vec == 2) ||
                             // (with loads issued a tile ahead, every walk in narrow 16-bit lanes whose time step fills its
                             // waves' lanes: bf16 [512, 1024, 256] 148 / 257 -> 145 / 238 us, [2048, 512, 128] backward 256 ->
