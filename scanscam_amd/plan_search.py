@@ -6,6 +6,7 @@ Time the library's automatic launch plan for a shape against a set of forced pla
     python -m scanscam_amd.plan_search --suite cl-a | cl-b | cl-odd | rows-23 | rows-25 | rows-26
     python -m scanscam_amd.plan_search --random 40 --seed 3      (channels-last shapes drawn at random, and the
                                                                   distribution of automatic / best over them)
+    python -m scanscam_amd.plan_search rows --random 30 --seed 1 (the same for the row layout)
 
 ``rows`` shapes are contiguous ``[rows, T]`` tensors scanned along ``T`` (the layout of
 ``simple_linear_scan`` and its siblings, ``scanscam/cuda.py:28-64`` in the reference), ``cl`` shapes are
@@ -114,6 +115,20 @@ def random_cl_shapes(n, seed):
     return out
 
 
+def random_row_shapes(n, seed):
+    """n shapes [rows, T]: T from 4 to 2^20 log-uniform, four in ten rounded to multiples of 8; 8 M to 190 M elements."""
+    rng = random.Random(seed)
+    out = []
+    while len(out) < n:
+        T = int(round(2 ** rng.uniform(2, 20)))
+        if rng.random() < 0.4:
+            T = max(4, (T + 4) // 8 * 8)
+        rows = int(2 ** rng.uniform(23, 27.5) / T)
+        if 1 <= rows <= 1 << 22:
+            out.append((rows, T))
+    return out
+
+
 def _time(calls, reps, warm):
     n = len(calls)
     for i in range(max(warm, 1)):
@@ -189,7 +204,8 @@ def main(argv=None):
     ap.add_argument("layout", nargs="?", choices=("rows", "cl"))
     ap.add_argument("shapes", nargs="*", metavar="SHAPE[:dtype]")
     ap.add_argument("--suite", choices=sorted(SUITES), help="a fixed list of shapes, each in f32 and bf16")
-    ap.add_argument("--random", type=int, metavar="N", help="N channels-last shapes drawn at random, each in f32 and bf16")
+    ap.add_argument("--random", type=int, metavar="N",
+                    help="N shapes drawn at random (channels-last, or rows when that layout is named), each in f32 and bf16")
     ap.add_argument("--seed", type=int, default=0, help="seed of --random")
     ap.add_argument("--reps", type=int, default=24)
     ap.add_argument("--every", action="store_true", help="also print every plan's timings")
@@ -203,7 +219,9 @@ def main(argv=None):
         layout, shapes = SUITES[args.suite]
         jobs = [(layout, s, dt) for s in shapes for dt in (torch.float32, torch.bfloat16)]
     elif args.random:
-        jobs = [("cl", s, dt) for s in random_cl_shapes(args.random, args.seed) for dt in (torch.float32, torch.bfloat16)]
+        layout = args.layout or "cl"
+        shapes = (random_row_shapes if layout == "rows" else random_cl_shapes)(args.random, args.seed)
+        jobs = [(layout, s, dt) for s in shapes for dt in (torch.float32, torch.bfloat16)]
     elif args.layout is None:
         ap.error("give a layout and shapes, --suite or --random")
     for spec in args.shapes:

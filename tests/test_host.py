@@ -212,6 +212,8 @@ def test_plan_search_sets_hold_plans_the_library_knows():
     # The random audit: the same shapes for the same seed, inside the stated bounds, and resolvable by the library.
     shapes = plan_search.random_cl_shapes(30, 3)
     assert shapes == plan_search.random_cl_shapes(30, 3) and shapes != plan_search.random_cl_shapes(30, 4)
+    rows = plan_search.random_row_shapes(20, 1)
+    assert rows == plan_search.random_row_shapes(20, 1) and all(1 <= r <= 1 << 22 and 4 <= T <= 1 << 20 for r, T in rows)
     for batch, T, C in shapes:
         assert 1 <= batch <= 8192 and 64 <= T <= 16384 and 8 <= C <= 5100 and batch * T * C <= 1 << 28
         for dtype in (torch.float32, torch.bfloat16):
