@@ -692,6 +692,17 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
                 l->vec = half;
                 l->ragged = !half_possible;
             }
+            // 65 to 127 channels that allow no whole pairs (an odd count, or tensors on odd elements): single channels are
+            // two waves per time step, the second mostly empty, and element-aligned pairs one. With a workgroup per
+            // batch element or more -- fp32 [2000, 1000, 65] 497 / 918 -> 367 / 624 us, [476, 1998, 113] 342 / 588 -> 277 / 480 us,
+            // [3964, 290, 89] 338 / 685 -> 266 / 466 us, bf16 [476, 1998, 113] 224 / 570 -> 150 / 262 us, [2000, 1000, 65] 260 / 660
+            // -> 227 / 412 us, [438, 1181, 93] 104 / 232 -> 84 / 139 us; 8 steps in 8 waves (16 steps lose 10 to 25 % backwards).
+            // (From 340 workgroups on: 300 are a round and a sixth, and there bf16 [300, 1000, 77] is 23 % slower forwards.)
+            if (esize <= 4 && l->vec == 1 && !l->ragged && C > kWave && C < 2 * kWave && batch >= 340 &&
+                u.mode == SCANSCAM_MODE_AUTO) {
+                l->vec = 2;
+                l->ragged = true;
+            }
             // 16-bit storage backwards, too few workgroups for the rule above but enough for a walk in pairs (168):
             // element-aligned pairs rather than single channels, walked or in tiles over time -- bf16 [71, 1910, 257]
             // 159 -> 124 us, [101, 1576, 219] 155 -> 124 us, [14, 1439, 1473] 121 -> 104 us, [64, 2048, 257] 141 -> 129 us.
@@ -821,7 +832,8 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // A forced wide lane that the alignment or C does not allow as it stands: element-aligned, where that kernel applies.
     if (u.vec && ((l->vec == full && full > 1 && !vec_possible) || (l->vec == 2 && esize == 2 && full != 2 && !pair_possible) ||
                   (half > 1 && l->vec == half && !half_possible))) {
-        if (C < (int64_t)kWave * l->vec || u.mode == kModeLookback) return SCANSCAM_EPLAN;
+        // (more than half a wave of such lanes per time step: below that several steps share a wave, in a kernel of whole lanes)
+        if (C <= (int64_t)(kWave / 2) * l->vec || u.mode == kModeLookback) return SCANSCAM_EPLAN;
         l->ragged = true;
     }
     // Too few (batch element, channel group) pairs to fill the GPU: cut time into tiles over
@@ -916,7 +928,8 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // [476, 1998, 113] 379 -> 344 us, [551, 3705, 59] 359 -> 319 us, [107, 2371, 206] 159 -> 130 us, [90, 2048, 514] 298 ->
     // 256 us; [986, 969, 157] and [438, 1181, 93] are level, and element-aligned pairs keep their walk.)
     if (l->kind == 0 && !u.vec && u.mode == SCANSCAM_MODE_AUTO && esize == 4 && l->vec <= 2 && C > 32 &&
-        (rev ? T >= (l->ragged ? 2048 : 384) : (T >= 1900 && !l->ragged)) && (C * esize) % 128 != 0) {
+        (rev ? T >= (l->ragged ? 2048 : 384) : (T >= 1900 && !l->ragged)) && (C * esize) % 128 != 0 &&
+        !(l->ragged && groups(2) == 1)) {  // (one wave of element-aligned pairs walks at 50-57 % of peak: above)
         l->kind = 2;
         // ([90, 2048, 514]: 436 us in pairs, 462 us in single channels; [100, 3000, 300], 0.83 of the fill: 265 / 439 against 288 / 476 us)
         l->vec = (half_possible && groups(2) * 2 * 8 <= groups(1) * 10) ? 2 : 1;
@@ -980,9 +993,10 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     // (and of fp32 channels: [512, 512, 333] backward 502 -> 390 us, [256, 1024, 777] 1246 -> 962 us, [128, 1024, 1003] 747 -> 664 us)
     // (Several time steps per wave, the packed kernel: only up to one workgroup per CU -- bf16 [306, 6590, 16] 117 / 163 us
     // with 16 steps, 84 / 107 us with 8; [128, 8192, 16] 65 / 90 against 70 / 89 us.)
+    const bool one_wave_ragged_pairs = l->ragged && l->vec == 2 && groups(2) == 1;  // (65 to 127 channels, above: 8 steps)
     const bool long_steps = l->kind != 0 ||
                             (esize == 2 && l->vec <= 2 && T >= 1024 && (rowgroups < 512 || (l->ragged && l->vec == 2)) &&
-                             (l->group == kWave || rowgroups <= kComputeUnits)) ||
+                             (l->group == kWave || rowgroups <= kComputeUnits) && !one_wave_ragged_pairs) ||
                             small_singles ||
                             // (fp32 forwards in single channels from two workgroups per CU on, with 8 waves: [3237, 206, 192] 295 ->
                             // 255 us, [1704, 67, 85] 49 -> 38 us, [2106, 99, 64] 37 -> 29 us, [5005, 328, 21] 185 -> 149 us; on rows of
@@ -991,7 +1005,7 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
                             // Backwards 16 waves of 8 steps stay ahead with few channels.)
                             (esize == 4 && !rev && l->vec == 1 && l->kind == 0 && rowgroups >= 2 * kComputeUnits && T < 512 &&
                              (C % 2 == 0 || groups(1) == 1)) ||
-                            (esize == 4 && l->ragged && l->vec == 2) ||
+                            (esize == 4 && l->ragged && l->vec == 2 && !one_wave_ragged_pairs) ||
                             // (with loads issued a tile ahead, every walk in narrow 16-bit lanes whose time step fills its
                             // waves' lanes: bf16 [512, 1024, 256] 148 / 257 -> 145 / 238 us, [2048, 512, 128] backward 256 ->
                             // 237 us, [512, 1024, 320] 184 / 331 -> 179 / 309 us, [1024, 1024, 64] backward 142 -> 124 us)

@@ -93,7 +93,7 @@ def cl_plans(dtype, C):
     if C % full != 0:  # lanes wider than the channel count divides: taken where a time step fills a wave of them
         out += [P(vec=v, unroll=s, waves=w, mode=walk)
                 for v, s, w in ((full, 4, most), (full, 4, 4), (half, 8, 8), (half, 8, 4), (2, 16, 8), (2, 8, 8))
-                if C % v != 0 and C >= 64 * v]
+                if C % v != 0 and C > 32 * v]
     out += [P(vec=v, unroll=s, waves=w, mode=split)
             for v, s, w in ((narrow, 16, 8), (half, 16, 8), (half, 8, 8), (1, 16, 8)) if C % v == 0]
     return out

@@ -227,12 +227,14 @@ WALK, TILES = hip.MODE_ROW, hip.MODE_LOOKBACK
         ((128, 8192, 16), torch.bfloat16, (WALK, 2, 16, 8), (WALK, 2, 16, 8)),    # ... walked from 100 workgroups on
         ((64, 16384, 16), torch.bfloat16, (TILES, 1, 16, 8), (TILES, 1, 16, 8)),
         ((209, 221, 1370), torch.bfloat16, (WALK, 4, 8, 8), (WALK, 4, 8, 8)),     # short rows, element-aligned: 8-byte lanes
-        ((476, 1998, 113), torch.float32, (TILES, 1, 16, 8), (TILES, 1, 16, 8)),  # fp32 off whole lines: tiles (forwards from 1900 steps)
+        ((476, 1998, 157), torch.float32, (TILES, 1, 16, 8), (TILES, 1, 16, 8)),  # fp32 off whole lines: tiles (forwards from 1900 steps)
         ((90, 2048, 514), torch.float32, (TILES, 2, 16, 8), (TILES, 2, 8, 8)),
         ((986, 969, 157), torch.float32, (WALK, 1, 8, 16), (TILES, 1, 16, 8)),
         ((4526, 65, 432), torch.float32, (WALK, 1, 16, 5), (WALK, 1, 8, 9)),       # rows of one or two tiles: evenly filled tiles
         ((506, 75, 943), torch.bfloat16, (WALK, 4, 8, 4), (WALK, 4, 8, 4)),        # ... three tiles of 4 waves for lanes of 8 bytes
         ((512, 512, 333), torch.float32, (WALK, 2, 16, 8), (WALK, 2, 16, 8)),     # ... element-aligned pairs only from 2048 steps
+        ((476, 1998, 113), torch.bfloat16, (WALK, 2, 8, 8), (WALK, 2, 8, 8)),      # 65-127 channels, an odd count: one wave of element-aligned pairs
+        ((2000, 1000, 65), torch.float32, (WALK, 2, 8, 8), (WALK, 2, 8, 8)),
         ((71, 1910, 257), torch.bfloat16, (TILES, 1, 16, 8), (WALK, 2, 16, 8)),   # 213 workgroups of element-aligned pairs backwards
         ((128, 512, 2048), torch.float32, (WALK, 2, 16, 8), (WALK, 4, 4, 4)),     # 2048 or more fp32 channels
         ((256, 1024, 256), torch.float64, (WALK, 1, 8, 8), (WALK, 1, 8, 8)),      # float64: its 8-byte lane is one channel

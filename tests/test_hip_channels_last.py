@@ -113,7 +113,8 @@ def test_element_aligned_lanes(gpu, dtype):
     bar = {torch.float32: 1e-5, torch.float64: 1e-13}.get(dtype, 1e-2)
     g = torch.Generator().manual_seed(23)
     n = 0
-    for shape in [(3, 107, 64 * full + 1), (2, 70, 64 * full + full - 1), (5, 33, 130 * full + 3), (2, 50, 401)]:
+    for shape in [(3, 107, 64 * full + 1), (2, 70, 64 * full + full - 1), (5, 33, 130 * full + 3), (2, 50, 401),
+                  (3, 85, 67), (2, 60, 127), (4, 40, 32 * full + 1)]:  # (more than half a wave of lanes per time step is enough)
         a = torch.rand(shape, generator=g, dtype=torch.float64).to(dtype)
         b = torch.randn(shape, generator=g, dtype=torch.float64).to(dtype)
         gh = torch.randn(shape, generator=g, dtype=torch.float64).to(dtype)
@@ -130,7 +131,7 @@ def test_element_aligned_lanes(gpu, dtype):
                 return v
             da, db, dgh, dhs = view_of(a), view_of(b), view_of(gh), view_of(hs)
             for vec in {8: (8, 4, 2), 4: (4, 2), 2: (2,)}[full]:
-                if shape[-1] < 64 * vec:
+                if shape[-1] <= 32 * vec:
                     continue
                 for steps in ((2, 4, 8) if vec == full else (4, 8, 16)):
                     plan = hip.Plan(vec=vec, unroll=steps, waves=3, mode=hip.MODE_ROW)
@@ -148,8 +149,8 @@ def test_element_aligned_lanes(gpu, dtype):
     b = torch.randn(shape, generator=g, dtype=torch.float64).to(dtype)
     want = oracle.fwd(as_rows(a), as_rows(b))
     assert rel_err(as_rows(hip.transposed_linear_scan_forward(a.to(gpu), b.to(gpu))), want) <= bar
-    # ... and a forced wide lane is refused where a time step does not fill a wave of them.
-    small = torch.rand(2, 8, 64 * full - 3, device=gpu).to(dtype)
+    # ... and a forced wide lane is refused where a time step fills no more than half a wave of them.
+    small = torch.rand(2, 8, 32 * full - 3, device=gpu).to(dtype)
     with pytest.raises(RuntimeError, match="plan"):
         hip.transposed_linear_scan_forward(small, small, plan=hip.Plan(vec=full, mode=hip.MODE_ROW))
 
@@ -373,6 +374,10 @@ MANY_WORKGROUPS = [
     (torch.float32, (14, 1100, 2539), None),    # element-aligned fp32 lanes, a few workgroups too many: tiles of single channels
     (torch.bfloat16, (71, 600, 257), None),     # 16-bit backwards: 213 workgroups of element-aligned pairs
     (torch.bfloat16, (39, 125, 4806), None),    # short rows, element-aligned: four-channel lanes
+    (torch.float32, (350, 300, 65), None),      # 65 to 127 channels, an odd count: one wave of element-aligned pairs
+    (torch.bfloat16, (350, 300, 113), None),
+    (torch.float16, (400, 67, 127), None),      # ... on a row of two tiles
+    (torch.float32, (345, 520, 93), None),
 ]
 
 
