@@ -235,6 +235,7 @@ WALK, TILES = hip.MODE_ROW, hip.MODE_LOOKBACK
         ((512, 512, 333), torch.float32, (WALK, 2, 16, 8), (WALK, 2, 16, 8)),     # ... element-aligned pairs only from 2048 steps
         ((476, 1998, 113), torch.bfloat16, (WALK, 2, 8, 8), (WALK, 2, 8, 8)),      # 65-127 channels, an odd count: one wave of element-aligned pairs
         ((2000, 1000, 65), torch.float32, (WALK, 2, 8, 8), (WALK, 2, 8, 8)),
+        ((15, 6680, 188), torch.bfloat16, (TILES, 2, 16, 8), (TILES, 4, 16, 8)),   # 16-bit backward tiles: four-channel lanes from 53 % fill
         ((71, 1910, 257), torch.bfloat16, (TILES, 1, 16, 8), (WALK, 2, 16, 8)),   # 213 workgroups of element-aligned pairs backwards
         ((128, 512, 2048), torch.float32, (WALK, 2, 16, 8), (WALK, 4, 4, 4)),     # 2048 or more fp32 channels
         ((256, 1024, 256), torch.float64, (WALK, 1, 8, 8), (WALK, 1, 8, 8)),      # float64: its 8-byte lane is one channel

@@ -378,6 +378,8 @@ MANY_WORKGROUPS = [
     (torch.bfloat16, (350, 300, 113), None),
     (torch.float16, (400, 67, 127), None),      # ... on a row of two tiles
     (torch.float32, (345, 520, 93), None),
+    (torch.bfloat16, (15, 1100, 188), None),    # 16-bit backward tiles in four-channel lanes that fill 47 of a wave's 64 lanes
+    (torch.float16, (13, 900, 400), None),
 ]
 
 
