@@ -338,7 +338,8 @@ def reference_grid(dev, args, hip, torch):
     Row layout: scanscam/cpu_test.py:51-77 and scanscam/cuda_test.py:166-247
     ((8,256,4096), (8,256,32), (256,4096), (16384,4096)); channels-last:
     cuda_test.py:250-308 ((8,4096,512) stored [B, T, C]). Mean microseconds per
-    launch over back-to-back launches on rotated buffer sets.
+    launch over back-to-back launches on rotated buffer sets; beside them the
+    reference's CPU loop on the same tensors (the CPU half of the same grid).
     """
     out = {}
     for shape in ((8, 256, 4096), (8, 256, 32), (256, 4096), (16384, 4096)):
@@ -359,6 +360,14 @@ def reference_grid(dev, args, hip, torch):
                 fwd_graph_us=round(gf_ms * 1e3, 2), bwd_graph_us=round(gb_ms * 1e3, 2),
                 fwd_graph_GBps=round(12 * n / (gf_ms * 1e-3) / 1e9, 1),
                 bwd_graph_GBps=round(20 * n / (gb_ms * 1e-3) / 1e9, 1))
+        if not args.no_cpu:
+            # The CPU half of the reference's grid (cpu_test.py:51-77): its single-threaded loop on the same
+            # shapes and N(0,1) tensors, called as its tests call it (contiguous inputs, outputs allocated by the
+            # caller), 1 warm-up + 3 repetitions per direction, median.
+            c = cpu_baseline(x, y, z, reps=3)
+            out["x".join(map(str, shape))].update(
+                cpu_fwd_us=round(c["fwd_s"] * 1e6, 1), cpu_bwd_us=round(c["bwd_s"] * 1e6, 1),
+                cpu_fwd_GBps=c["fwd_GBps"], cpu_bwd_GBps=c["bwd_GBps"], cpu_kind=c["kind"], cpu_cores=c["cores"])
         del sets, first
         torch.cuda.empty_cache()
     # Channels-last: logical [8, 512, 4096] stored [8, 4096, 512].
@@ -578,7 +587,7 @@ def channels_last_workload(spec, args, hip, torch):
 
 def channels_last_table(args, hip, torch):
     """Contiguous [B, T, C] tensors scanned along T (the layout of the reference's transposed kernels,
-    scanscam/cuda.py:100-148): its timing shape, many-channel and many-batch shapes in fp32 and bf16, channel
+    scanscam/cuda.py:69-95): its timing shape, many-channel and many-batch shapes in fp32 and bf16, channel
     counts that are no whole 128-byte lines or fewer than a wave. Rotated buffer sets, prepared calls."""
     shapes = [(8, 4096, 512, torch.float32), (8, 4096, 2048, torch.float32), (64, 2048, 1024, torch.float32),
               (256, 1024, 1024, torch.float32), (8, 4096, 512, torch.bfloat16), (8, 4096, 2048, torch.bfloat16),
@@ -649,8 +658,8 @@ def cpu_baseline(a, b, gh, reps):
         "sample": f"the full workload ({n} elements), 1 warm-up + {reps} repetitions per direction, median",
         "fwd_GBps": round(12 * n / tf / 1e9, 3),
         "bwd_GBps": round(20 * n / tb / 1e9, 3),
-        "fwd_s": round(tf, 4),
-        "bwd_s": round(tb, 4),
+        "fwd_s": round(tf, 7),
+        "bwd_s": round(tb, 7),
         "elements_per_s": round(n / (tf + tb)),
         "host_cpus": os.cpu_count(),
     }
@@ -688,8 +697,8 @@ def host_library(a, b, gh, reps):
         "value": round(32 * n / (tf + tb) / 1e9, 3),
         "unit": "GB/s",
         "threads": len(cpu._slabs(rows, T)),
-        "fwd_s": round(tf, 4),
-        "bwd_s": round(tb, 4),
+        "fwd_s": round(tf, 7),
+        "bwd_s": round(tb, 7),
     }
 
 

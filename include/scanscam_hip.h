@@ -12,7 +12,9 @@
  *   - every tensor is a dense row-major [rows, T] array on the current HIP
  *     device, scanned along T, all of one storage type;
  *   - the caller allocates every output and the workspace; the library
- *     allocates nothing, keeps no state and is re-entrant;
+ *     allocates nothing and is re-entrant. It keeps no state between calls,
+ *     with one exception: scanscam_scan_fwd_noalloc works in a fixed array of
+ *     the library's own in each GPU's memory (see there);
  *   - calls are asynchronous: kernels are enqueued on `stream` (0 = the null
  *     stream) and the call returns at once;
  *   - the return value is 0 on success or a SCANSCAM_E* code; nothing is
@@ -86,6 +88,10 @@ typedef struct scanscam_plan {
  * Forward scan: h[r,t] = a[r,t]*h[r,t-1] + b[r,t], h[r,-1] = 0.
  * Replaces blocked_linear_scan(gate, value, output), src/scanscam_cuda.cu:260-307
  * (arithmetic of simple_linear_scan_cpu, src/scanscam_cpu.hpp:30-52).
+ * h may be the very buffer of a or of b (an in-place call, as the reference's kernel allows,
+ * src/scanscam_cuda.cu:205-257); any other overlap of an output with an input is not allowed, and
+ * the outputs of the backward call must not share bytes with any of its inputs (a[t+1] and h[t-1] are
+ * read across the borders of what a workgroup writes).
  */
 int scanscam_scan_fwd(const void *a, const void *b, void *h, int64_t rows, int64_t T, int dtype,
                       void *workspace, size_t workspace_bytes, void *stream);
@@ -102,8 +108,8 @@ int scanscam_scan_bwd(const void *a, const void *h, const void *gh, void *ga, vo
 
 /*
  * scanscam_scan_fwd for callers that cannot allocate device memory: code under HIP graph capture,
- * tight serving loops, harnesses that forbid hipMalloc. It has no counterpart in the reference (whose
- * kernels need no workspace, src/scanscam_cuda.cu:260-307). Same arguments, results (bit for bit) and
+ * tight serving loops, harnesses that forbid hipMalloc. It has no counterpart in the reference, whose
+ * kernels need no workspace. Same arguments, results (bit for bit) and
  * errors as scanscam_scan_fwd, without the workspace: where rows are split over workgroups, the
  * look-back descriptors live in a fixed array of SCANSCAM_NOALLOC_SCRATCH_BYTES in the GPU's memory
  * that belongs to the library (one per GPU it runs on, held until the process ends), found once per
@@ -113,10 +119,16 @@ int scanscam_scan_bwd(const void *a, const void *h, const void *gh, void *ga, vo
  * Every call clears the part of the array it uses, with a kernel on `stream`. All calls on one GPU
  * share that GPU's array: calls that may overlap in time on one GPU (two streams, two threads) race
  * and must use scanscam_scan_fwd with separate workspaces instead.
+ * The first call on a device asks the runtime for the array's address there (not a stream operation, and
+ * it may load the library's code onto the device): make one call per device -- any shape, also rows == 0 --
+ * outside of any stream capture before capturing calls into a HIP graph. The device that `stream` belongs
+ * to must be the current device, as for every call of this library.
+ * scanscam_noalloc_timed_out is scanscam_workspace_timed_out (below) for the current device's array.
  */
 #define SCANSCAM_NOALLOC_SCRATCH_BYTES (1 << 20)
 int scanscam_scan_fwd_noalloc(const void *a, const void *b, void *h, int64_t rows, int64_t T, int dtype,
                               void *stream);
+int scanscam_noalloc_timed_out(void *stream, int *timed_out);
 
 /*
  * Bytes of device workspace the call above of that direction needs for this
@@ -244,7 +256,7 @@ int scanscam_resolve_plan(int64_t rows, int64_t T, int dtype, int direction, con
  * aligned: mode SCANSCAM_MODE_ROW where a workgroup walks all of T, SCANSCAM_MODE_LOOKBACK where
  * tiles of time steps chain through the workspace; vec channels per lane, unroll time steps per
  * wave and tile, waves per workgroup. No counterpart in the reference, whose kernel has one launch
- * shape (scanscam/cuda.py:100-148 passes channels_per_block only).
+ * shape (scanscam/cuda.py:69-95 passes channels_per_block only).
  */
 int scanscam_resolve_plan_cl(int64_t batch, int64_t T, int64_t C, int dtype, int direction,
                              const scanscam_plan *plan, scanscam_plan *out);

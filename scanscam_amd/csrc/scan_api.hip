@@ -173,7 +173,8 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
     const bool small_problem = rows * T * esize <= (int64_t(1) << 25) && T >= 4 * full &&
                                row_vectors * 10 >= (int64_t)pow2_ceil((int)row_vectors) * 9;
     if (u.mode == kModeFlat ||
-        (u.mode == SCANSCAM_MODE_AUTO && flat_possible && !u.vec && !small_problem && prefer_flat(T, full, esize))) {
+        (u.mode == SCANSCAM_MODE_AUTO && flat_possible && !u.vec && (u.unroll == 0 || u.unroll == 2 || u.unroll == 4) &&
+         !small_problem && prefer_flat(T, full, esize))) {
         if (!flat_possible) return SCANSCAM_EPLAN;
         if (u.vec && u.vec != full) return SCANSCAM_EPLAN;
         l.mode = kModeFlat;
@@ -467,6 +468,19 @@ int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y
     // The flat kernel takes dense [rows, T] tensors on 16-byte aligned bases (rows of any length).
     bool flat_ok = allow_flat && n0 == 1;
     for (int k = 0; k < 5; k++) flat_ok = flat_ok && (!used[k] || (aligned_to(ptrs[k], 16) && (n1 == 1 || s1[k] == T)));
+    // The flat kernel's workgroups read a halo of their neighbours' spans (and a[e+1] / h[e-1] across span
+    // borders backwards), so an output that shares bytes with an input -- an in-place call, which every other
+    // kernel family allows because it reads only what it is about to write -- would race there.
+    if (flat_ok) {
+        const int64_t bytes = rows * T * esize;
+        auto overlaps = [&](const void *p, const void *q) {
+            const char *pc = static_cast<const char *>(p), *qc = static_cast<const char *>(q);
+            return pc < qc + bytes && qc < pc + bytes;
+        };
+        for (int o = 3; o < 5; o++)
+            for (int i = 0; i < 3; i++)
+                if (used[o] && used[i] && overlaps(ptrs[o], ptrs[i])) flat_ok = false;
+    }
     // One pair of events cannot bracket the flat launch and the launch for the rows it leaves over.
     if ((start_event || stop_event) && flat_rows(rows, T, full) != rows) flat_ok = false;
 
@@ -1384,6 +1398,15 @@ int scanscam_workspace_timed_out(const void *workspace, void *stream, int *timed
     return SCANSCAM_OK;
 }
 
+int scanscam_noalloc_timed_out(void *stream, int *timed_out)
+{
+    if (!timed_out) return SCANSCAM_EINVAL;
+    void *ws = nullptr;
+    const int rc = noalloc_scratch(&ws);
+    if (rc != SCANSCAM_OK) return rc;
+    return scanscam_workspace_timed_out(ws, stream, timed_out);
+}
+
 int scanscam_resolve_plan(int64_t rows, int64_t T, int dtype, int direction, const scanscam_plan *plan,
                           scanscam_plan *out)
 {
@@ -1442,6 +1465,6 @@ const char *scanscam_strerror(int code)
     }
 }
 
-int scanscam_abi_version(void) { return 2; }
+int scanscam_abi_version(void) { return 3; }
 
 }  // extern "C"

@@ -29,7 +29,7 @@ LIB_PATH = os.environ.get("SCANSCAM_HIP_LIB") or os.path.join(_HERE, "libscansca
 
 MODE_AUTO, MODE_SMALL, MODE_ROW, MODE_LOOKBACK, MODE_FLAT = 0, 1, 2, 3, 4
 FORWARD, BACKWARD = 0, 1
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _DTYPES = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2, torch.float64: 3}
 
@@ -103,6 +103,8 @@ def _bind(path: str) -> ctypes.CDLL:
     lib.scanscam_workspace_bytes_cl.restype = sz
     lib.scanscam_workspace_timed_out.argtypes = [p, p, ctypes.POINTER(ctypes.c_int)]
     lib.scanscam_workspace_timed_out.restype = i32
+    lib.scanscam_noalloc_timed_out.argtypes = [p, ctypes.POINTER(ctypes.c_int)]
+    lib.scanscam_noalloc_timed_out.restype = i32
     lib.scanscam_resolve_plan.argtypes = [i64, i64, i32, i32, plan_p, plan_p]
     lib.scanscam_resolve_plan.restype = i32
     lib.scanscam_resolve_plan_cl.argtypes = [i64, i64, i64, i32, i32, plan_p, plan_p]
@@ -186,6 +188,32 @@ def _check_rows(*tensors: torch.Tensor) -> None:
             raise RuntimeError("scanscam_amd.hip: tensors must be contiguous")
 
 
+# Kernels that wait for another workgroup's carry give up after a bounded number of polls and then
+# write NaN (see ``scanscam_plan.spin_limit``); a correct launch never gets there. With checking on --
+# ``SCANSCAM_DEBUG=1`` in the environment, or ``check_waits(True)`` -- every wrapper below that handed
+# the library a workspace waits for its launch and raises if a wait expired, instead of returning NaN.
+# ``SCANSCAM_SPIN_LIMIT`` / ``check_waits(..., spin_limit=n)`` set the poll limit of calls without a plan.
+_check = os.environ.get("SCANSCAM_DEBUG", "") not in ("", "0")
+_spin_limit = int(os.environ.get("SCANSCAM_SPIN_LIMIT", "0") or 0)
+
+
+def check_waits(on: bool, spin_limit: int = 0) -> None:
+    """Turn the check for expired carry waits on or off (it blocks the host after every such launch)."""
+    global _check, _spin_limit
+    _check, _spin_limit = bool(on), int(spin_limit)
+
+
+def _raise_if_wait_expired(ws: Optional[torch.Tensor], what: str) -> None:
+    if not _check or ws is None:
+        return
+    flag = ctypes.c_int(0)
+    rc = lib().scanscam_workspace_timed_out(ws.data_ptr(), torch.cuda.current_stream().cuda_stream, ctypes.byref(flag))
+    if rc != 0:
+        raise RuntimeError(f"scanscam_workspace_timed_out: {strerror(rc)}")
+    if flag.value:
+        raise RuntimeError(f"{what}: a wait for another workgroup's carry expired; the affected outputs hold NaN")
+
+
 def _workspace(rows: int, T: int, dtype: torch.dtype, direction: int, plan: Optional[Plan],
                device: torch.device) -> Tuple[Optional[torch.Tensor], int, int]:
     n = workspace_bytes(rows, T, dtype, direction, plan)
@@ -213,7 +241,9 @@ def scan_forward_out(gate: torch.Tensor, value: torch.Tensor, out: torch.Tensor,
         ws, ws_ptr, ws_n = _workspace(rows, T, gate.dtype, FORWARD, plan, gate.device)
         stream = torch.cuda.current_stream().cuda_stream
         rc = L.scanscam_scan_fwd_plan(gate.data_ptr(), value.data_ptr(), out.data_ptr(), rows, T, code,
-                                      ws_ptr, ws_n, stream, ctypes.byref(plan) if plan is not None else None)
+                                      ws_ptr, ws_n, stream, _plan_ref(plan))
+        if rc == 0:
+            _raise_if_wait_expired(ws, "scanscam_scan_fwd")
     if rc != 0:
         raise RuntimeError(f"scanscam_scan_fwd: {strerror(rc)}")
 
@@ -233,7 +263,9 @@ def scan_backward_out(gate: torch.Tensor, output: torch.Tensor, out_grad: torch.
         stream = torch.cuda.current_stream().cuda_stream
         rc = L.scanscam_scan_bwd_plan(gate.data_ptr(), output.data_ptr(), out_grad.data_ptr(),
                                       gate_grad.data_ptr(), value_grad.data_ptr(), rows, T, code,
-                                      ws_ptr, ws_n, stream, ctypes.byref(plan) if plan is not None else None)
+                                      ws_ptr, ws_n, stream, _plan_ref(plan))
+        if rc == 0:
+            _raise_if_wait_expired(ws, "scanscam_scan_bwd")
     if rc != 0:
         raise RuntimeError(f"scanscam_scan_bwd: {strerror(rc)}")
 
@@ -312,6 +344,8 @@ def prepare_forward(gate: torch.Tensor, value: torch.Tensor, out: torch.Tensor,
     fixed buffers (benchmarks, a captured step). The tensors and the workspace
     are kept alive by the callable; launches go to the stream that is current
     when it is called, on the device that was current when it was prepared.
+    The callable owns ONE workspace: launches of it that may overlap in time (two
+    streams) race on it -- prepare one callable per stream.
     With ``events`` every launch records the scan kernel's own start and end
     on the GPU into them (``scanscam_scan_fwd_timed``).
     """
@@ -340,7 +374,7 @@ def prepare_forward(gate: torch.Tensor, value: torch.Tensor, out: torch.Tensor,
 def prepare_backward(gate: torch.Tensor, output: torch.Tensor, out_grad: torch.Tensor,
                      gate_grad: torch.Tensor, value_grad: torch.Tensor, plan: Optional[Plan] = None,
                      events: Optional["KernelEvents"] = None):
-    """The backward counterpart of ``prepare_forward``."""
+    """The backward counterpart of ``prepare_forward`` (one workspace: one stream at a time)."""
     L = lib()
     _check_rows(gate, output, out_grad, gate_grad, value_grad)
     rows, T = gate.shape
@@ -475,11 +509,13 @@ def transposed_linear_scan_forward(x: torch.Tensor, y: torch.Tensor, channels_pe
     batch, T, C = x.shape
     if x.numel() == 0:
         return out
-    plan_ref = ctypes.byref(plan) if plan is not None else None
+    plan_ref = _plan_ref(plan)
     with _on(x.device):
         ws, ws_ptr, ws_n = _workspace_cl(L, batch, T, C, x.dtype, FORWARD, plan, x.device)
         rc = L.scanscam_scan_fwd_cl(x.data_ptr(), y.data_ptr(), out.data_ptr(), batch, T, C, _dtype_code(x.dtype),
                                     ws_ptr, ws_n, torch.cuda.current_stream().cuda_stream, plan_ref)
+        if rc == 0:
+            _raise_if_wait_expired(ws, "scanscam_scan_fwd_cl")
     if rc != 0:
         raise RuntimeError(f"scanscam_scan_fwd_cl: {strerror(rc)}")
     return out
@@ -497,19 +533,22 @@ def transposed_linear_scan_backward(x: torch.Tensor, y: torch.Tensor, z: torch.T
     batch, T, C = x.shape
     if x.numel() == 0:
         return out_a, out_b
-    plan_ref = ctypes.byref(plan) if plan is not None else None
+    plan_ref = _plan_ref(plan)
     with _on(x.device):
         ws, ws_ptr, ws_n = _workspace_cl(L, batch, T, C, x.dtype, BACKWARD, plan, x.device)
         rc = L.scanscam_scan_bwd_cl(x.data_ptr(), y.data_ptr(), z.data_ptr(), out_a.data_ptr(), out_b.data_ptr(),
                                     batch, T, C, _dtype_code(x.dtype), ws_ptr, ws_n,
                                     torch.cuda.current_stream().cuda_stream, plan_ref)
+        if rc == 0:
+            _raise_if_wait_expired(ws, "scanscam_scan_bwd_cl")
     if rc != 0:
         raise RuntimeError(f"scanscam_scan_bwd_cl: {strerror(rc)}")
     return out_a, out_b
 
 
 def prepare_forward_cl(x: torch.Tensor, y: torch.Tensor, out: torch.Tensor, plan: Optional[Plan] = None):
-    """``prepare_forward`` for contiguous ``[batch, T, C]`` tensors: a callable that launches this scan again."""
+    """``prepare_forward`` for contiguous ``[batch, T, C]`` tensors: a callable that launches this scan again
+    (it owns one workspace: launches that may overlap on two streams need a callable each)."""
     L = lib()
     _check_channels_last(x, y, out)
     batch, T, C = x.shape
@@ -529,7 +568,7 @@ def prepare_forward_cl(x: torch.Tensor, y: torch.Tensor, out: torch.Tensor, plan
 
 def prepare_backward_cl(x: torch.Tensor, y: torch.Tensor, z: torch.Tensor, out_a: torch.Tensor, out_b: torch.Tensor,
                         plan: Optional[Plan] = None):
-    """The backward counterpart of ``prepare_forward_cl`` (gate ``x``, output ``y``, output grad ``z``)."""
+    """The backward counterpart of ``prepare_forward_cl`` (gate ``x``, output ``y``, output grad ``z``); one stream at a time."""
     L = lib()
     _check_channels_last(x, y, z, out_a, out_b)
     batch, T, C = x.shape
@@ -612,6 +651,8 @@ def _check_same(*tensors: torch.Tensor) -> None:
 
 
 def _plan_ref(plan: Optional[Plan]):
+    if plan is None and _spin_limit > 0:
+        plan = Plan(spin_limit=_spin_limit)
     return ctypes.byref(plan) if plan is not None else None
 
 
@@ -666,9 +707,17 @@ def _run_rows(inputs, n_out: int, direction: int, plan: Optional[Plan]):
         ptrs = [t.data_ptr() for t in tensors]
         fn = L.scanscam_scan_fwd_strided if direction == FORWARD else L.scanscam_scan_bwd_strided
         rc = fn(*ptrs, *refs, n0, n1, T, code, ws_ptr, ws_n, stream, _plan_ref(plan))
+        if rc == 0:
+            _raise_if_wait_expired(ws, "scanscam_scan_fwd_strided" if direction == FORWARD else "scanscam_scan_bwd_strided")
     if rc != 0:
         raise RuntimeError(f"scanscam_scan_{'fwd' if direction == FORWARD else 'bwd'}_strided: {strerror(rc)}")
     return outs
+
+
+def _cl_step_too_far(time_stride: int, C: int, esize: int) -> bool:
+    """The channels-last kernels address a wave's time steps with 32-bit byte offsets from its first one (18 steps
+    and the lane's channel): the library refuses time strides beyond that, and such views are copied first."""
+    return time_stride * esize * 18 + C * esize >= 2 ** 32
 
 
 def _run_cl(inputs, n_out: int, direction: int, plan: Optional[Plan]):
@@ -682,7 +731,7 @@ def _run_cl(inputs, n_out: int, direction: int, plan: Optional[Plan]):
         return outs
     tensors = list(inputs) + outs
     levels = _joint_levels(shape[:-2], [t.stride()[:-2] for t in tensors])
-    if len(levels) > 1 or any(t.stride(-1) >= 2 ** 31 for t in tensors):
+    if len(levels) > 1 or any(_cl_step_too_far(t.stride(-1), C, first.element_size()) for t in tensors):
         tensors = [t.mT.contiguous().mT for t in inputs] + outs
         levels = _joint_levels(shape[:-2], [t.stride()[:-2] for t in tensors])
     batch, sb = levels[0] if levels else (1, [0] * len(tensors))
@@ -695,6 +744,8 @@ def _run_cl(inputs, n_out: int, direction: int, plan: Optional[Plan]):
         refs = [ctypes.byref(x) for x in st]
         fn = L.scanscam_scan_fwd_cl_strided if direction == FORWARD else L.scanscam_scan_bwd_cl_strided
         rc = fn(*ptrs, *refs, batch, T, C, _dtype_code(first.dtype), ws_ptr, ws_n, stream, plan_ref)
+        if rc == 0:
+            _raise_if_wait_expired(ws, "scanscam_scan_fwd_cl_strided" if direction == FORWARD else "scanscam_scan_bwd_cl_strided")
     if rc != 0:
         raise RuntimeError(f"scanscam_scan_{'fwd' if direction == FORWARD else 'bwd'}_cl_strided: {strerror(rc)}")
     return outs

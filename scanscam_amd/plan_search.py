@@ -9,8 +9,8 @@ Time the library's automatic launch plan for a shape against a set of forced pla
     python -m scanscam_amd.plan_search rows --random 30 --seed 1 (the same for the row layout)
 
 ``rows`` shapes are contiguous ``[rows, T]`` tensors scanned along ``T`` (the layout of
-``simple_linear_scan`` and its siblings, ``scanscam/cuda.py:28-64`` in the reference), ``cl`` shapes are
-contiguous ``[batch, T, C]`` tensors scanned along ``T`` (``transposed_linear_scan``, ``cuda.py:100-148``).
+``simple_linear_scan`` and its siblings, ``scanscam/cuda.py:16-66`` in the reference), ``cl`` shapes are
+contiguous ``[batch, T, C]`` tensors scanned along ``T`` (``transposed_linear_scan``, ``cuda.py:69-95``).
 dtype is f32 (default), bf16, f16 or f64.
 
 One line per shape and dtype: the automatic plan's forward / backward microseconds and fraction of the 8 TB/s

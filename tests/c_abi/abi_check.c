@@ -170,6 +170,11 @@ static int check_case(const char *name, long rows, long T, long C, int channels_
         HIP_OK(hipStreamSynchronize(stream));
         HIP_OK(hipMemcpy(got, o0, n * 4, hipMemcpyDeviceToHost));
         if (memcmp(got, again, n * 4) != 0) failures++;
+        {
+            int expired = -1;
+            if (scanscam_noalloc_timed_out(stream, &expired) != SCANSCAM_OK || expired != 0) failures++;
+            if (scanscam_noalloc_timed_out(stream, NULL) != SCANSCAM_EINVAL) failures++;
+        }
         if (scanscam_scan_bwd_plan(da, dh, dgh, o1, o0, rows, T, SCANSCAM_F32, ws, ws_bytes, stream, NULL) != SCANSCAM_OK)
             failures++;
         HIP_OK(hipStreamSynchronize(stream));
@@ -275,7 +280,7 @@ static int check_strided(const char *name, long B, long C, long T, int channels_
 
 int main(void)
 {
-    if (scanscam_abi_version() != 2) {
+    if (scanscam_abi_version() != 3) {
         fprintf(stderr, "abi_check: unexpected ABI version %d\n", scanscam_abi_version());
         return 1;
     }

@@ -32,7 +32,7 @@ def test_library_is_built_and_loads():
 
 def test_every_declared_symbol_is_exported():
     names = declared_functions()
-    assert "scanscam_scan_fwd" in names and "scanscam_scan_bwd" in names and len(names) == 21
+    assert "scanscam_scan_fwd" in names and "scanscam_scan_bwd" in names and len(names) == 22
     raw = ctypes.CDLL(hip.LIB_PATH)
     for name in names:
         assert hasattr(raw, name), f"{name} declared in scanscam_hip.h but not exported"
@@ -194,6 +194,16 @@ def test_every_automatic_plan_is_a_valid_plan():
                             assert out.waves_per_row >= 1 and out.waves % out.waves_per_row == 0
                         checked += 1
     assert checked > 10000
+    # Hints without a mode: the automatic choice may only pick a family that accepts them (dense short rows
+    # prefer the flat kernel, which has 2 or 4 chunks per wave; the small kernel takes the other counts).
+    for dtype, T in ((torch.float32, 68), (torch.float64, 34), (torch.bfloat16, 136)):
+        for plan in (hip.Plan(unroll=1), hip.Plan(unroll=8), hip.Plan(unroll=8, waves=8), hip.Plan(unroll=2),
+                     hip.Plan(waves=3), hip.Plan(unroll=4, waves=16)):
+            for direction in (hip.FORWARD, hip.BACKWARD):
+                out = hip.Plan()
+                rc = L.scanscam_resolve_plan(200000, T, hip._dtype_code(dtype), direction, ctypes.byref(plan), ctypes.byref(out))
+                assert rc == 0, (dtype, T, plan, hip.strerror(rc))
+                assert out.mode == (hip.MODE_FLAT if plan.unroll in (0, 2, 4) else hip.MODE_SMALL), (dtype, T, plan, out)
 
 
 WALK, TILES = hip.MODE_ROW, hip.MODE_LOOKBACK

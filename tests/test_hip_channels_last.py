@@ -12,6 +12,7 @@ import pytest
 import torch
 
 import oracle
+from criteria import assert_reference_allclose
 from scanscam_amd import hip
 
 pytestmark = pytest.mark.gpu
@@ -60,11 +61,16 @@ def test_reference_shapes(gpu, shape, channels_per_block):
     assert out.shape == x.shape and out.is_contiguous()
     want = oracle.fwd(as_rows(x), as_rows(y))
     assert row_norm_err(as_rows(out), want) <= 1e-4
+    # The reference tests' own criterion, element by element (scanscam/cuda_test.py:141, 163).
+    assert_reference_allclose(as_rows(out), want, lambda: oracle.fwd_acc64(as_rows(x), as_rows(y)), f"h {shape}")
     hs = torch.from_numpy(want).mT.contiguous()  # the oracle's output, stored [batch, T, C]
     ga, gb = hip.transposed_linear_scan_backward(x.to(gpu), hs.to(gpu), gh.to(gpu), channels_per_block)
     wga, wgb = oracle.bwd(as_rows(x), want, as_rows(gh))
     assert row_norm_err(as_rows(gb), wgb) <= 1e-4
     assert row_norm_err(as_rows(ga), wga) <= 1e-4
+    exact = lambda: oracle.bwd_acc64(as_rows(x), want, as_rows(gh))  # noqa: E731
+    assert_reference_allclose(as_rows(gb), wgb, lambda: exact()[1], f"grad_b {shape}")
+    assert_reference_allclose(as_rows(ga), wga, lambda: exact()[0], f"grad_a {shape}")
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16, torch.float16])

@@ -119,3 +119,40 @@ def test_flat_is_bit_reproducible_run_to_run(gpu):
     b = torch.randn(5000, 101, generator=g).to(gpu)
     outs = [hip.linear_scan_forward(a, b, hip.Plan(mode=hip.MODE_FLAT)) for _ in range(3)]
     assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+
+
+def test_forward_in_place_on_a_shape_the_flat_kernel_prefers(gpu):
+    """h may share its buffer with a or b (every kernel that is chosen for such a call reads only what it is about
+    to write); the flat kernel, which reads a halo of its neighbours' spans, must then not be the one chosen."""
+    rows, T = 120003, 70
+    assert hip.resolve_plan(rows, T, torch.float32, hip.FORWARD).mode == hip.MODE_FLAT
+    g = seeded(70)
+    a = torch.rand(rows, T, generator=g)
+    b = torch.randn(rows, T, generator=g)
+    want = oracle.fwd(a.numpy(), b.numpy())
+    for alias in ("value", "gate"):
+        da, db = a.to(gpu), b.to(gpu)
+        out = db if alias == "value" else da
+        print(f"case flat in place over {alias}", flush=True)
+        hip.scan_forward_out(da, db, out)
+        assert rel_err(to_np(out), want) <= 1e-5, alias
+    # Forced, the flat kernel refuses an in-place call instead of racing.
+    da, db = a.to(gpu), b.to(gpu)
+    with pytest.raises(RuntimeError, match="plan"):
+        hip.scan_forward_out(da, db, db, hip.Plan(mode=hip.MODE_FLAT))
+
+
+def test_automatic_flat_choice_respects_plan_hints(gpu):
+    """A plan that only names unroll or waves (mode automatic) must resolve to a kernel that accepts them:
+    17 vectors per row are what the flat kernel is preferred for, and it takes 2 or 4 chunks per wave only."""
+    rows, T = 120003, 68
+    assert hip.resolve_plan(rows, T, torch.float32, hip.FORWARD).mode == hip.MODE_FLAT
+    assert hip.resolve_plan(rows, T, torch.float32, hip.FORWARD, hip.Plan(unroll=8)).mode == hip.MODE_SMALL
+    g = seeded(71)
+    a = torch.rand(rows, T, generator=g)
+    b = torch.randn(rows, T, generator=g)
+    want = oracle.fwd(a.numpy(), b.numpy())
+    for plan in (hip.Plan(unroll=1), hip.Plan(unroll=8), hip.Plan(unroll=8, waves=8), hip.Plan(unroll=2), hip.Plan(waves=2)):
+        print(f"case flat hints {plan}", flush=True)
+        h = hip.linear_scan_forward(a.to(gpu), b.to(gpu), plan)
+        assert rel_err(to_np(h), want) <= 1e-5, plan

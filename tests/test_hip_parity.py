@@ -21,6 +21,7 @@ import pytest
 import torch
 
 import oracle
+from criteria import assert_reference_allclose
 from scanscam_amd import hip
 
 pytestmark = pytest.mark.gpu
@@ -119,7 +120,7 @@ def test_reference_grid(gpu, shape, permute):
     want = oracle.fwd(a.numpy(), b.numpy())
     assert row_norm_err(to_np(h), want) <= 1e-4
     # The reference tests' own criterion, element by element (scanscam/cuda_test.py:80).
-    assert np.allclose(to_np(h), want, atol=1e-4, rtol=1e-5)
+    assert_reference_allclose(to_np(h), want, lambda: oracle.fwd_acc64(a.numpy(), b.numpy()), f"h {shape}")
     # Backward as a pure function of (gate, output, out_grad), as the reference tests it.
     hs = torch.from_numpy(want)
     if permute:
@@ -128,7 +129,11 @@ def test_reference_grid(gpu, shape, permute):
     wga, wgb = oracle.bwd(a.numpy(), hs.numpy(), gh.numpy())
     assert row_norm_err(to_np(gb), wgb) <= 1e-4
     assert row_norm_err(to_np(ga), wga) <= 1e-4
-    assert np.allclose(to_np(gb), wgb, atol=1e-4, rtol=1e-5)  # scanscam/cuda_test.py:125-126
+    # The reference tests' own criterion, element by element, on both gradients
+    # (scanscam/cuda_test.py:100-103, 123-126).
+    exact = lambda: oracle.bwd_acc64(a.numpy(), hs.numpy(), gh.numpy())  # noqa: E731
+    assert_reference_allclose(to_np(gb), wgb, lambda: exact()[1], f"grad_b {shape}")
+    assert_reference_allclose(to_np(ga), wga, lambda: exact()[0], f"grad_a {shape}")
 
 
 # ---------------------------------------------------------------------------

@@ -231,3 +231,17 @@ def test_bench_refuses_more_than_one_gpu():
                           timeout=120)
     assert done.returncode != 0
     assert "one GPU" in done.stderr and done.stdout.strip() == ""
+
+
+def test_channels_last_views_with_a_far_time_stride_are_copied_first():
+    """The channels-last kernels refuse time strides beyond 32-bit step offsets (4 GiB / 18); the wrapper's
+    decision to copy such a view first uses the library's own bound."""
+    from scanscam_amd import hip
+
+    assert not hip._cl_step_too_far(512, 512, 4)
+    assert not hip._cl_step_too_far(59_000_000, 1024, 4)        # 225 MiB steps: still addressable
+    assert hip._cl_step_too_far(59_700_000, 1024, 4)            # about 227.7 MiB: beyond
+    assert hip._cl_step_too_far(2 ** 31, 8, 2)
+    # Exactly the library's inequality (time stride * size * 18 + C * size < 2^32).
+    for stride, C, esize in ((59_652_323, 4, 4), (59_652_324, 4, 4), (119_304_646, 8, 2), (119_304_647, 2, 2)):
+        assert hip._cl_step_too_far(stride, C, esize) == (stride * esize * 18 + C * esize >= 2 ** 32)

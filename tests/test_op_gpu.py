@@ -240,3 +240,43 @@ def test_concurrent_launches_on_two_streams(gpu):
             s.synchronize()
         for w, x in zip(want, got):
             assert torch.equal(w, x)
+
+
+def test_expired_wait_raises_through_the_op_when_checking_is_on(gpu):
+    """With checking on (SCANSCAM_DEBUG=1 or hip.check_waits) a carry wait that gives up is an exception from
+    scan(), not NaNs in its result. One poll per wait makes expiry all but certain on 4 rows of 256 tiles; every
+    kernel still runs to its end. Should every tile have found its predecessors in that one poll, the result is
+    simply right."""
+    g = torch.Generator(device=gpu).manual_seed(8)
+    a = torch.rand((4, 1 << 22), generator=g, device=gpu)
+    b = torch.randn((4, 1 << 22), generator=g, device=gpu)
+    good = scanscam_amd.scan(a, b)
+    hip.check_waits(True, spin_limit=1)
+    try:
+        print("case expired wait through scan()", flush=True)
+        try:
+            out = scanscam_amd.scan(a, b)
+            raised = False
+        except RuntimeError as exc:
+            raised = True
+            assert "wait" in str(exc) and "expired" in str(exc)
+        torch.cuda.synchronize()  # returns: no wave is left spinning
+        if not raised:
+            assert not bool(torch.isnan(out).any()) and torch.equal(out, good)
+        # Checking on, default limit: nothing expires, nothing raises.
+        hip.check_waits(True)
+        assert torch.equal(scanscam_amd.scan(a, b), good)
+        # A channels-last shape whose time is split over workgroups goes through the same check.
+        x = torch.rand((2, 8192, 256), generator=g, device=gpu)
+        y = torch.randn((2, 8192, 256), generator=g, device=gpu)
+        assert hip.resolve_plan_cl(2, 8192, 256, torch.float32).mode == hip.MODE_LOOKBACK
+        good_cl = scanscam_amd.scan(x.mT, y.mT)
+        hip.check_waits(True, spin_limit=1)
+        try:
+            out = scanscam_amd.scan(x.mT, y.mT)
+            assert not bool(torch.isnan(out).any()) and torch.equal(out, good_cl)
+        except RuntimeError as exc:
+            assert "expired" in str(exc)
+        torch.cuda.synchronize()
+    finally:
+        hip.check_waits(False)

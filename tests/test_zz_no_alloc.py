@@ -81,6 +81,12 @@ def test_noalloc_matches_the_workspace_entry_point_call_after_call(gpu):
         want, _ = _fwd_with_workspace(a, b)
     s.synchronize()
     assert torch.equal(first, want) and torch.equal(second, want)
+    # No wait expired in any of these calls, says the query of the array's flag word.
+    import ctypes
+
+    flag = ctypes.c_int(-1)
+    assert hip.lib().scanscam_noalloc_timed_out(s.cuda_stream, ctypes.byref(flag)) == 0 and flag.value == 0
+    assert hip.lib().scanscam_noalloc_timed_out(None, None) == 1
 
 
 def test_noalloc_refuses_shapes_beyond_its_array_and_launches_nothing(gpu):
