@@ -25,17 +25,18 @@ using scanscam::kWave;
 using scanscam::Launch;
 using scanscam::ScanArgs;
 
-// Clears the look-back workspace (a kernel, not a memset, so that a caller may
-// capture the launch sequence in a HIP graph).
-__global__ __launch_bounds__(256) void scan_ws_clear_kernel(uint64_t *ws, int64_t words)
+// Prepares the look-back workspace (a kernel, not a memset, so that a caller may capture the launch
+// sequence in a HIP graph): the ticket counters and the time-out flag (the first `zero_words` words) are
+// zeroed, every descriptor word after them is set to all ones, the kernels' "not yet".
+__global__ __launch_bounds__(256) void scan_ws_clear_kernel(uint64_t *ws, int64_t words, int64_t zero_words)
 {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < words) ws[i] = 0;
+    if (i < words) ws[i] = i < zero_words ? 0ull : ~0ull;
 }
 
-hipError_t clear_workspace(uint64_t *ws, int64_t words, hipStream_t stream)
+hipError_t clear_workspace(uint64_t *ws, int64_t words, int64_t zero_words, hipStream_t stream)
 {
-    void *params[] = {&ws, &words};
+    void *params[] = {&ws, &words, &zero_words};
     return hipLaunchKernel(reinterpret_cast<const void *>(scan_ws_clear_kernel), dim3((unsigned)((words + 255) / 256)),
                            dim3(256), params, 0, stream);
 }
@@ -53,8 +54,12 @@ int elem_size(int dtype)
     }
 }
 
-// 64-bit words per value published in the look-back workspace (one per 32-bit half).
+// 64-bit words per value published in the look-back workspace (one per 32-bit half), and per tile (its
+// aggregate pair) and super-tile (its pair and its end value) of the row layout's look-back kernel, whose
+// fp32 pairs are one word (scanscam::kTileWords, kSuperWords).
 int value_words(int dtype) { return dtype == SCANSCAM_F64 ? 2 : 1; }
+int tile_words(int dtype) { return dtype == SCANSCAM_F64 ? scanscam::kTileWords<double> : scanscam::kTileWords<float>; }
+int super_words(int dtype) { return dtype == SCANSCAM_F64 ? scanscam::kSuperWords<double> : scanscam::kSuperWords<float>; }
 
 // Bytes of the arithmetic type behind a storage type.
 int compute_size(int dtype) { return dtype == SCANSCAM_F64 ? 8 : 4; }
@@ -359,9 +364,8 @@ int resolve(const scanscam_plan *user, int64_t rows, int64_t T, int dtype, bool 
         l.grid = (int64_t)out->counters * rows_per_counter * out->tiles_per_row;
         if (l.grid >= (int64_t(1) << 31)) return SCANSCAM_EINVAL;
         const int64_t supers = rows * (int64_t)((out->tiles_per_row + kSuper - 1) / kSuper);
-        const int vw = value_words(dtype);
-        out->super_base = (int64_t)out->counters * kCounterStride + tiles * 2 * vw;
-        out->ws_bytes = (size_t)(out->super_base + supers * 4 * vw) * sizeof(uint64_t);
+        out->super_base = (int64_t)out->counters * kCounterStride + tiles * tile_words(dtype);
+        out->ws_bytes = (size_t)(out->super_base + supers * super_words(dtype)) * sizeof(uint64_t);
     } else {
         return SCANSCAM_EPLAN;
     }
@@ -569,7 +573,7 @@ int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y
         if (!aligned_to(workspace, 8)) return SCANSCAM_EALIGN;
         args.ws = static_cast<uint64_t *>(workspace);
         const int64_t words = (int64_t)(r.ws_bytes / sizeof(uint64_t));
-        if (clear_workspace(args.ws, words, s) != hipSuccess) return SCANSCAM_ELAUNCH;
+        if (clear_workspace(args.ws, words, args.desc_base, s) != hipSuccess) return SCANSCAM_ELAUNCH;
         // One launch over all rows; the kernel splits a row index into (group, row). Its grid is far
         // below every launch limit by construction.
         return launch(args, r.l) == hipSuccess ? SCANSCAM_OK : SCANSCAM_ELAUNCH;
@@ -1136,7 +1140,8 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         if (tiles >= (int64_t(1) << 31)) return SCANSCAM_EINVAL;
         l->segments = (int)tiles;  // the kernel's tiles per row-group
         const int64_t supers = (tiles + l->waves - 1) / l->waves;
-        l->ws_bytes = (size_t)(rowgroups * kCounterStride + rowgroups * tiles * 2 * vals + rowgroups * supers * 4 * vals) *
+        const int64_t pairs = (int64_t)l->vec * kWave * tile_words(dtype);  // words of one [vec][64] array of pairs
+        l->ws_bytes = (size_t)(rowgroups * kCounterStride + rowgroups * tiles * pairs + rowgroups * supers * (pairs + vals)) *
                       sizeof(uint64_t);
     }
     if (l->segments <= 1) {  // nothing to split after all
@@ -1231,7 +1236,8 @@ int run_cl(bool rev, const void *a, const void *x, const void *h, void *y0, void
         if (!aligned_to(workspace, 8)) return SCANSCAM_EALIGN;
         args.ws = static_cast<uint64_t *>(workspace);
         const int64_t words = (int64_t)(l.ws_bytes / sizeof(uint64_t));
-        if (clear_workspace(args.ws, words, s) != hipSuccess) return SCANSCAM_ELAUNCH;
+        const int64_t rowgroups = batch * ((C + (int64_t)kWave * l.vec - 1) / ((int64_t)kWave * l.vec));
+        if (clear_workspace(args.ws, words, rowgroups * kCounterStride, s) != hipSuccess) return SCANSCAM_ELAUNCH;
     }
     hipError_t e = hipErrorInvalidValue;
     switch (dtype) {

@@ -659,8 +659,8 @@ __global__ __launch_bounds__(MAXT) void scan_cl_packed_kernel(const ClArgs p)
 //
 // Workspace, in 64-bit words: ticket counter of row-group r at word
 // r * kCounterStride, word 1 raised on a timed-out wait; then per (row-group,
-// tile) its pair, A then B, each [VEC][64] published values; then per
-// (row-group, super-tile) SA, SB, SI likewise (4 slots, one unused).
+// tile) its [VEC][64] published pairs; then per (row-group, super-tile) its
+// [VEC][64] pairs (SA, SB) and its [VEC][64] end values SI (encodings: Desc).
 // LDS: [W][7][VEC][64] values (per wave slot: wave pairs A, B; tile aggregates A, B;
 // super-tile SI, SA, SB).
 // ---------------------------------------------------------------------------
@@ -680,6 +680,25 @@ __device__ __forceinline__ void cl_publish(uint64_t *dst, int lane, const CT (&v
     using D = Desc<CT>;
 #pragma unroll
     for (int k = 0; k < VEC; k++) D::store(dst + (k * kWave + lane) * D::W, val[k]);
+}
+
+// The same for an affine pair per channel: [VEC][64] pairs (fp32: one word per pair, one load per poll).
+template <typename CT, int VEC>
+__device__ __forceinline__ bool cl_fetch_pair(const uint64_t *src, int lane, CT (&a)[VEC], CT (&b)[VEC])
+{
+    using D = Desc<CT>;
+    bool ready = true;
+#pragma unroll
+    for (int k = 0; k < VEC; k++) ready = D::load_pair(src + (k * kWave + lane) * D::PAIR, a[k], b[k]) && ready;
+    return __ballot(ready) == ~0ull;
+}
+
+template <typename CT, int VEC>
+__device__ __forceinline__ void cl_publish_pair(uint64_t *dst, int lane, const CT (&a)[VEC], const CT (&b)[VEC])
+{
+    using D = Desc<CT>;
+#pragma unroll
+    for (int k = 0; k < VEC; k++) D::store_pair(dst + (k * kWave + lane) * D::PAIR, a[k], b[k]);
 }
 
 template <typename ST, int VEC, int S, bool REV, int MAXT>
@@ -705,7 +724,9 @@ __global__ __launch_bounds__(MAXT) void scan_cl_lookback_kernel(const ClArgs p)
            tA, tB,     // aggregates of tiles 0..j-1 of the super-tile
            sI, sA, sB  // super-tiles m-1, m-2, ...
     };
-    constexpr int kVals = VEC * kWave * D::W;  // words of one [VEC][64] array of published values
+    constexpr int kVals = VEC * kWave * D::W;      // words of one [VEC][64] array of published values
+    constexpr int kPairs = VEC * kWave * D::PAIR;  // ... of published pairs
+    constexpr int kSup = kPairs + kVals;           // a super-tile: its pair (SA, SB), then its end value SI
 #define AT(arr, w, k) lds[((w) * 7 + (arr)) * (VEC * kWave) + (k) * kWave + lane]
 
     // Row-groups of a workgroup's XCD: with p.xcd_order (time steps that are not whole 128-byte lines) a
@@ -731,9 +752,9 @@ __global__ __launch_bounds__(MAXT) void scan_cl_lookback_kernel(const ClArgs p)
     __syncthreads();
     const int tile = (int)__builtin_amdgcn_readfirstlane((int)lds_ticket);
     const ClLane<ST> ln = cl_lane<ST, VEC>(p, rg / groups, (int)(rg % groups), lane);
-    uint64_t *tiles = p.ws + rowgroups * kCounterStride + rg * (int64_t)tpr * 2 * kVals;
-    uint64_t *supers = p.ws + rowgroups * kCounterStride + rowgroups * (int64_t)tpr * 2 * kVals +
-                       rg * (int64_t)spr * 4 * kVals;
+    uint64_t *tiles = p.ws + rowgroups * kCounterStride + rg * (int64_t)tpr * kPairs;
+    uint64_t *supers = p.ws + rowgroups * kCounterStride + rowgroups * (int64_t)tpr * kPairs +
+                       rg * (int64_t)spr * kSup;
     const int j = tile % W, m = tile / W;
 
     ClSteps<ST, VEC, S, REV, true, CT, true> cur;
@@ -766,10 +787,7 @@ __global__ __launch_bounds__(MAXT) void scan_cl_lookback_kernel(const ClArgs p)
 
     if (tpr > 1) {
         const bool closes = (j == W - 1) && (m + 1 < spr);
-        if (wave == 0 && j < W - 1 && tile + 1 < tpr) {
-            cl_publish<CT, VEC>(tiles + (int64_t)tile * 2 * kVals, lane, TA);
-            cl_publish<CT, VEC>(tiles + (int64_t)tile * 2 * kVals + kVals, lane, TB);
-        }
+        if (wave == 0 && j < W - 1 && tile + 1 < tpr) cl_publish_pair<CT, VEC>(tiles + (int64_t)tile * kPairs, lane, TA, TB);
         // Wave w is responsible for tile w of this super-tile (if w < j) and for super-tile m-1-w.
         bool have_t = wave >= j;
         const int sidx = m - 1 - wave;
@@ -787,9 +805,7 @@ __global__ __launch_bounds__(MAXT) void scan_cl_lookback_kernel(const ClArgs p)
         for (int spin = 0; spin < p.spin_limit; spin++) {
             CT val[VEC], val2[VEC];
             if (!have_t) {
-                const uint64_t *d = tiles + (int64_t)(m * W + wave) * 2 * kVals;
-                const bool ra = cl_fetch<CT, VEC>(d, lane, val), rb = cl_fetch<CT, VEC>(d + kVals, lane, val2);
-                if (ra && rb) {
+                if (cl_fetch_pair<CT, VEC>(tiles + (int64_t)(m * W + wave) * kPairs, lane, val, val2)) {
                     have_t = true;
 #pragma unroll
                     for (int k = 0; k < VEC; k++) {
@@ -799,16 +815,14 @@ __global__ __launch_bounds__(MAXT) void scan_cl_lookback_kernel(const ClArgs p)
                 }
             }
             if (!have_si) {
-                if (cl_fetch<CT, VEC>(supers + (int64_t)sidx * 4 * kVals + 2 * kVals, lane, val)) {
+                if (cl_fetch<CT, VEC>(supers + (int64_t)sidx * kSup + kPairs, lane, val)) {
                     have_si = true;
 #pragma unroll
                     for (int k = 0; k < VEC; k++) AT(sI, wave, k) = val[k];
                 }
             }
             if (!have_sa) {
-                const uint64_t *d = supers + (int64_t)sidx * 4 * kVals;
-                const bool ra = cl_fetch<CT, VEC>(d, lane, val), rb = cl_fetch<CT, VEC>(d + kVals, lane, val2);
-                if (ra && rb) {
+                if (cl_fetch_pair<CT, VEC>(supers + (int64_t)sidx * kSup, lane, val, val2)) {
                     have_sa = true;
 #pragma unroll
                     for (int k = 0; k < VEC; k++) {
@@ -857,8 +871,7 @@ __global__ __launch_bounds__(MAXT) void scan_cl_lookback_kernel(const ClArgs p)
                         SB[k] = fma_(TA[k], SB[k], TB[k]);
                         SA[k] = TA[k] * SA[k];
                     }
-                    cl_publish<CT, VEC>(supers + (int64_t)m * 4 * kVals, lane, SA);
-                    cl_publish<CT, VEC>(supers + (int64_t)m * 4 * kVals + kVals, lane, SB);
+                    cl_publish_pair<CT, VEC>(supers + (int64_t)m * kSup, lane, SA, SB);
                 }
             }
             if (tiles_done && supers_done) break;
@@ -905,7 +918,7 @@ __global__ __launch_bounds__(MAXT) void scan_cl_lookback_kernel(const ClArgs p)
                 SA[k] = TA[k] * SA[k];
                 SI[k] = fma_(SA[k], S_m[k], SB[k]);
             }
-            cl_publish<CT, VEC>(supers + (int64_t)m * 4 * kVals + 2 * kVals, lane, SI);
+            cl_publish<CT, VEC>(supers + (int64_t)m * kSup + kPairs, lane, SI);
         }
     }
 

@@ -82,12 +82,10 @@ struct ScanArgs {
 // Look-back workspace layout, in 64-bit words. Ticket counter c is word
 // c * kCounterStride (one counter per 128-byte line, so that counters do not
 // serialise on one another); word 1 is raised if a look-back wait ever expired
-// (results are then NaN). Then come 2 published values per tile (its aggregate)
-// and 4 slots per super-tile of 64 tiles (its aggregate and its end value). A
-// value is one word {1, bits(float)} for fp32 arithmetic and two words, one per
-// 32-bit half, for fp64: the upper half of every word is a ready flag and the
-// workspace is zeroed before each launch, so every word is self-validating and
-// no fence is needed around it.
+// (results are then NaN). Then come the descriptor words: per tile its aggregate
+// pair, per super-tile of 64 tiles its aggregate pair and its end value (see
+// Desc below for their encoding). Before each launch the counters are zeroed
+// and the descriptor words set to all ones ("not yet").
 constexpr int kCounterStride = 16;
 constexpr int kMaxCounters = 256;
 
@@ -738,13 +736,21 @@ __global__ __launch_bounds__(MAXT) void scan_small_kernel(const ScanArgs p)
 // ---------------------------------------------------------------------------
 constexpr int kSuper = 64;  // tiles per super-tile (one per lane)
 
-// A published value: each 32-bit half of it sits in the low half of its own
-// 64-bit word, whose high half is the ready flag (1). One word for fp32
-// arithmetic, two for fp64. A tile owns 2 values (A, B), a super-tile 4 slots
-// (SA, SB, SI, unused).
+// Published values. The workspace's descriptor words are set to all ones before each launch, and every
+// word that is written is distinguishable from that pattern on its own, so a word is self-validating and
+// no fence is needed around it (each is written with one relaxed agent-scope 64-bit store).
+//   fp32 pair (A, B) of an affine map: ONE word {bits(A), bits(B) << 32}. "Not yet" is the low half
+//     0xffffffff, a NaN pattern that no published A has: a NaN A is published as the canonical quiet
+//     NaN 0x7fc00000. A tile owns one such word; one poll of it is one 8-byte load.
+//   fp32 single value (a super-tile's end value): {bits(v), 1 << 32}.
+//   fp64: every 32-bit half of a value in the low half of its own word under the flag 1 (a pair is 4
+//     words, a single value 2).
+// A tile owns kTileWords<CT> words, a super-tile kSuperWords<CT>: its pair (SA, SB), then its end value SI.
 template <typename CT> struct Desc;
 template <> struct Desc<float> {
-    static constexpr int W = 1;
+    static constexpr int W = 1;        // words per single value
+    static constexpr int PAIR = 1;     // words per pair
+    static constexpr uint32_t kNotYet = 0xffffffffu;
     static __device__ __forceinline__ void store(uint64_t *p, float v)
     {
         const uint64_t w = (1ull << 32) | (uint64_t)__builtin_bit_cast(uint32_t, v);
@@ -754,11 +760,42 @@ template <> struct Desc<float> {
     {
         const uint64_t w = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         v = __builtin_bit_cast(float, (uint32_t)w);
-        return (w >> 32) != 0;
+        return (w >> 32) == 1;
+    }
+    static __device__ __forceinline__ uint64_t pack_pair(float a, float b)
+    {
+        uint32_t ua = __builtin_bit_cast(uint32_t, a);
+        ua = (a != a) ? 0x7fc00000u : ua;
+        return (uint64_t)ua | ((uint64_t)__builtin_bit_cast(uint32_t, b) << 32);
+    }
+    static __device__ __forceinline__ void store_pair(uint64_t *p, float a, float b)
+    {
+        __hip_atomic_store(p, pack_pair(a, b), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    // A raw word (fetched now, looked at later) and its interpretation as a pair or as a single value.
+    static __device__ __forceinline__ uint64_t fetch_raw(const uint64_t *p)
+    {
+        return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    static __device__ __forceinline__ bool unpack(uint64_t w, float &v)
+    {
+        v = __builtin_bit_cast(float, (uint32_t)w);
+        return (w >> 32) == 1;
+    }
+    static __device__ __forceinline__ bool unpack_pair(uint64_t w, float &a, float &b)
+    {
+        a = __builtin_bit_cast(float, (uint32_t)w);
+        b = __builtin_bit_cast(float, (uint32_t)(w >> 32));
+        return (uint32_t)w != kNotYet;
+    }
+    static __device__ __forceinline__ bool load_pair(const uint64_t *p, float &a, float &b)
+    {
+        return unpack_pair(fetch_raw(p), a, b);
     }
 };
 template <> struct Desc<double> {
     static constexpr int W = 2;
+    static constexpr int PAIR = 4;
     static __device__ __forceinline__ void store(uint64_t *p, double v)
     {
         const uint64_t b = __builtin_bit_cast(uint64_t, v);
@@ -770,9 +807,25 @@ template <> struct Desc<double> {
         const uint64_t lo = __hip_atomic_load(p + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         const uint64_t hi = __hip_atomic_load(p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         v = __builtin_bit_cast(double, (hi << 32) | (lo & 0xffffffffull));
-        return (lo >> 32) != 0 && (hi >> 32) != 0;
+        return (lo >> 32) == 1 && (hi >> 32) == 1;
     }
+    static __device__ __forceinline__ void store_pair(uint64_t *p, double a, double b)
+    {
+        store(p, a);
+        store(p + W, b);
+    }
+    static __device__ __forceinline__ bool load_pair(const uint64_t *p, double &a, double &b)
+    {
+        const bool ra = load(p, a), rb = load(p + W, b);
+        return ra && rb;
+    }
+    // (No raw form: a pair is four words. The look-back polls fp64 descriptors where it needs them.)
+    static __device__ __forceinline__ uint64_t fetch_raw(const uint64_t *) { return ~0ull; }
+    static __device__ __forceinline__ bool unpack(uint64_t, double &) { return false; }
+    static __device__ __forceinline__ bool unpack_pair(uint64_t, double &, double &) { return false; }
 };
+template <typename CT> constexpr int kTileWords = Desc<CT>::PAIR;
+template <typename CT> constexpr int kSuperWords = Desc<CT>::PAIR + Desc<CT>::W;
 
 // Default number of polls before a waiting wave gives up. Tickets make every
 // awaited tile belong to a workgroup that is already running, so the limit is
@@ -782,102 +835,151 @@ template <> struct Desc<double> {
 constexpr int kSpinLimit = 1 << 20;
 constexpr int kTimeoutWord = 1;
 
-// Returns the scan value entering tile `tile` of row `row`, whose own aggregate
-// is (TA, TB). Called by all 64 lanes of one wave; `tile` must be wave-uniform.
+// The look-back of one tile, run by all 64 lanes of one wave (`tile` is wave-uniform). Lane q < j
+// collects tile q of this tile's super-tile, lane j holds the tile itself, the rest the identity; lane k
+// also watches super-tile m-1-k (before the row starts the value is 0).
+//   begin()   where everything lies, what is already known;
+//   issue()   the loads of one poll of what is still missing (fp32: raw words kept in registers, not
+//             looked at -- so a poll can be in flight while the wave does other work);
+//   absorb()  looks at them;
+//   finish()  publishes the tile's own aggregate, then polls until the carry is known and returns the
+//             scan value entering the tile.
+// With EARLY the kernel issues one poll as soon as the wave's data has arrived and reduces the data
+// while it is in flight: a predecessor's aggregate that became visible in the meantime is then in hand
+// when the tile's own aggregate is, one memory round trip earlier than a poll issued after the reduce.
 template <typename CT>
-__device__ __forceinline__ CT lookback_carry(const ScanArgs &p, int64_t row, int tile, CT TA, CT TB, int lane)
-{
+struct Lookback {
     using D = Desc<CT>;
-    constexpr int TW = 2 * D::W, SW = 4 * D::W;  // words per tile / per super-tile
-    const int tpr = p.tiles_per_row;
-    const int spr = (tpr + kSuper - 1) / kSuper;
-    const int j = tile % kSuper, m = tile / kSuper;
-    uint64_t *trow = p.ws + p.desc_base + row * (int64_t)tpr * TW;
-    uint64_t *srow = p.ws + p.super_base + row * (int64_t)spr * SW;
-    const bool closes = (j == kSuper - 1) && (m + 1 < spr);  // a later super-tile needs (SA, SB, SI)
+    static constexpr int TW = kTileWords<CT>, SW = kSuperWords<CT>;
+    static constexpr bool RAW = sizeof(CT) == 4;  // polls may be issued ahead (one word per pair)
 
-    if (lane == 0 && j < kSuper - 1 && tile + 1 < tpr) {
-        D::store(trow + (int64_t)tile * TW, TA);
-        D::store(trow + (int64_t)tile * TW + D::W, TB);
+    uint64_t *trow, *srow;
+    int j, m, sidx, spr, tpr;
+    bool have_t, have_si, have_sa, pending;
+    CT A, B, SI, SA, SB;
+    uint64_t raw_t, raw_sa, raw_si;
+
+    __device__ __forceinline__ void begin(const ScanArgs &p, int64_t row, int tile, int lane)
+    {
+        tpr = p.tiles_per_row;
+        spr = (tpr + kSuper - 1) / kSuper;
+        j = tile % kSuper;
+        m = tile / kSuper;
+        trow = p.ws + p.desc_base + row * (int64_t)tpr * TW;
+        srow = p.ws + p.super_base + row * (int64_t)spr * SW;
+        have_t = lane >= j;
+        A = CT(1);
+        B = CT(0);
+        sidx = m - 1 - lane;
+        have_si = have_sa = sidx < 0;
+        SI = CT(0);
+        SA = CT(1);
+        SB = CT(0);
+        pending = false;
+        raw_t = raw_sa = raw_si = ~0ull;
     }
 
-    // Lane q < j collects tile q of this super-tile; lane j holds this tile; the rest the identity.
-    bool have_t = lane >= j;
-    CT A = (lane == j) ? TA : CT(1), B = (lane == j) ? TB : CT(0);
-    // Lane k watches super-tile m-1-k; before the row starts the value is 0.
-    const int sidx = m - 1 - lane;
-    bool have_si = sidx < 0, have_sa = sidx < 0;
-    CT SI = CT(0), SA = CT(1), SB = CT(0);
+    __device__ __forceinline__ void issue(int lane)
+    {
+        if (RAW) {
+            // Lanes with nothing to fetch keep "not yet" words, which absorb() skips.
+            if (!have_t) raw_t = D::fetch_raw(trow + (int64_t)(m * kSuper + lane) * TW);
+            if (!have_sa) raw_sa = D::fetch_raw(srow + (int64_t)sidx * SW);
+            if (!have_si) raw_si = D::fetch_raw(srow + (int64_t)sidx * SW + D::PAIR);
+            pending = true;
+        }
+    }
 
-    bool tiles_done = false, super_done = false;
-    CT PA = CT(1), PB = CT(0), S = CT(0);
-    for (int spin = 0; spin < p.spin_limit; spin++) {
-        if (!have_t) {
-            const uint64_t *d = trow + (int64_t)(m * kSuper + lane) * TW;
+    __device__ __forceinline__ void absorb(int lane)
+    {
+        if (RAW) {
+            if (!pending) issue(lane);
+            pending = false;
             CT va, vb;
-            const bool ra = D::load(d, va), rb = D::load(d + D::W, vb);
-            if (ra && rb) {
+            if (!have_t && D::unpack_pair(raw_t, va, vb)) {
                 have_t = true;
                 A = va;
                 B = vb;
             }
-        }
-        if (!have_si || !have_sa) {
-            const uint64_t *d = srow + (int64_t)sidx * SW;
-            if (!have_si) {
-                CT vi;
-                if (D::load(d + 2 * D::W, vi)) {
-                    have_si = true;
-                    SI = vi;
-                }
+            if (!have_sa && D::unpack_pair(raw_sa, va, vb)) {
+                have_sa = true;
+                SA = va;
+                SB = vb;
             }
-            if (!have_sa) {
-                CT va, vb;
-                const bool ra = D::load(d, va), rb = D::load(d + D::W, vb);
-                if (ra && rb) {
-                    have_sa = true;
-                    SA = va;
-                    SB = vb;
-                }
+            if (!have_si && D::unpack(raw_si, va)) {
+                have_si = true;
+                SI = va;
             }
-        }
-        if (!tiles_done && __ballot(have_t) == ~0ull) {
-            tiles_done = true;
-            PA = A;
-            PB = B;
-            wave_scan<false, CT>(PA, PB, lane);
-            if (closes) {
-                const CT sa = read_lane(PA, kSuper - 1), sb = read_lane(PB, kSuper - 1);
-                if (lane == 0) {
-                    D::store(srow + (int64_t)m * SW, sa);
-                    D::store(srow + (int64_t)m * SW + D::W, sb);
-                }
+        } else {
+            CT va, vb;
+            if (!have_t && D::load_pair(trow + (int64_t)(m * kSuper + lane) * TW, va, vb)) {
+                have_t = true;
+                A = va;
+                B = vb;
+            }
+            if (!have_sa && D::load_pair(srow + (int64_t)sidx * SW, va, vb)) {
+                have_sa = true;
+                SA = va;
+                SB = vb;
+            }
+            if (!have_si && D::load(srow + (int64_t)sidx * SW + D::PAIR, va)) {
+                have_si = true;
+                SI = va;
             }
         }
-        if (!super_done) {
-            const uint64_t mi = __ballot(have_si);
-            const uint64_t ma = __ballot(have_sa);
-            if (mi != 0) {
-                const int first = __builtin_ctzll(mi);  // nearest super-tile with a published end value
-                const uint64_t need = (first == 0) ? 0ull : ((~0ull) >> (64 - first));
-                if ((ma & need) == need) {
-                    S = read_lane(SI, first);
-                    for (int q = first - 1; q >= 0; q--) S = fma_(read_lane(SA, q), S, read_lane(SB, q));
-                    super_done = true;
-                }
-            }
-        }
-        if (tiles_done && super_done) break;
-        __builtin_amdgcn_s_sleep(1);
     }
-    if (!(tiles_done && super_done)) {
-        if (lane == 0) __hip_atomic_store(p.ws + kTimeoutWord, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        S = CT(__builtin_nanf(""));
+
+    __device__ __forceinline__ CT finish(const ScanArgs &p, int tile, CT TA, CT TB, int lane)
+    {
+        const bool closes = (j == kSuper - 1) && (m + 1 < spr);  // a later super-tile needs (SA, SB, SI)
+        if (lane == 0 && j < kSuper - 1 && tile + 1 < tpr) D::store_pair(trow + (int64_t)tile * TW, TA, TB);
+        if (lane == j) {
+            A = TA;
+            B = TB;
+        }
+        bool tiles_done = false, super_done = false;
+        CT PA = CT(1), PB = CT(0), S = CT(0);
+        for (int spin = 0; spin < p.spin_limit; spin++) {
+            absorb(lane);
+            if (!tiles_done && __ballot(have_t) == ~0ull) {
+                tiles_done = true;
+                PA = A;
+                PB = B;
+                wave_scan<false, CT>(PA, PB, lane);
+                if (closes) {
+                    const CT sa = read_lane(PA, kSuper - 1), sb = read_lane(PB, kSuper - 1);
+                    if (lane == 0) D::store_pair(srow + (int64_t)m * SW, sa, sb);
+                }
+            }
+            if (!super_done) {
+                const uint64_t mi = __ballot(have_si);
+                const uint64_t ma = __ballot(have_sa);
+                if (mi != 0) {
+                    const int first = __builtin_ctzll(mi);  // nearest super-tile with a published end value
+                    const uint64_t need = (first == 0) ? 0ull : ((~0ull) >> (64 - first));
+                    if ((ma & need) == need) {
+                        S = read_lane(SI, first);
+                        for (int q = first - 1; q >= 0; q--) S = fma_(read_lane(SA, q), S, read_lane(SB, q));
+                        super_done = true;
+                    }
+                }
+            }
+            if (tiles_done && super_done) break;
+            if (spin > 0) __builtin_amdgcn_s_sleep(1);
+        }
+        if (!(tiles_done && super_done)) {
+            if (lane == 0) __hip_atomic_store(p.ws + kTimeoutWord, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            S = CT(__builtin_nanf(""));
+        }
+        const CT end_a = read_lane(PA, kSuper - 1), end_b = read_lane(PB, kSuper - 1);
+        if (closes && lane == 0) D::store(srow + (int64_t)m * SW + D::PAIR, fma_(end_a, S, end_b));
+        return j > 0 ? fma_(read_lane(PA, j - 1), S, read_lane(PB, j - 1)) : S;
     }
-    const CT end_a = read_lane(PA, kSuper - 1), end_b = read_lane(PB, kSuper - 1);
-    if (closes && lane == 0) D::store(srow + (int64_t)m * SW + 2 * D::W, fma_(end_a, S, end_b));
-    return j > 0 ? fma_(read_lane(PA, j - 1), S, read_lane(PB, j - 1)) : S;
-}
+};
+
+#ifndef SCANSCAM_EARLY_POLL
+#define SCANSCAM_EARLY_POLL 0
+#endif
 
 template <typename ST, int VEC, int U, bool REV, int MAXT, bool RAGGED = false>
 __global__ __launch_bounds__(MAXT) void scan_lookback_kernel(const ScanArgs p)
@@ -926,6 +1028,16 @@ __global__ __launch_bounds__(MAXT) void scan_lookback_kernel(const ScanArgs p)
         w.place(u, REV ? nvp - 1 - s : s, shift, true, p.T);
     }
     w.load(p, lane, kWave - 1);
+    Lookback<CT> lb;
+    const bool chained = p.tiles_per_row > 1;
+    if (wave == 0 && chained) {
+        lb.begin(p, row, tile, lane);
+        if (SCANSCAM_EARLY_POLL && Lookback<CT>::RAW) {
+            // Once this wave's data is in, one poll goes out and is in flight during the reduce.
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            lb.issue(lane);
+        }
+    }
     w.reduce(lane, kWave - 1, hp);
 
     CT WA, WB;
@@ -944,7 +1056,7 @@ __global__ __launch_bounds__(MAXT) void scan_lookback_kernel(const ScanArgs p)
             TA = lds_A[q] * TA;
         }
         CT cin = CT(0);
-        if (p.tiles_per_row > 1) cin = lookback_carry<CT>(p, row, tile, TA, TB, lane);
+        if (chained) cin = lb.finish(p, tile, TA, TB, lane);
         if (lane == 0) lds_carry = cin;
     }
     __syncthreads();
