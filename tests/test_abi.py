@@ -165,8 +165,11 @@ def test_automatic_plan_per_regime(rows, T, dtype, mode, vec):
 def test_lookback_workspace_size_formula():
     plan = hip.Plan(mode=hip.MODE_LOOKBACK, vec=4, unroll=2, waves=2)
     # tile = 2 waves * 2 chunks * 256 elements = 1024 elements; 5 tiles per row of 4100;
-    # one ticket counter (a 16-word line) per row, 2 words per tile, 4 per super-tile of 64 tiles.
-    assert hip.workspace_bytes(3, 4100, torch.float32, hip.FORWARD, plan) == (3 * 16 + 3 * 5 * 2 + 3 * 1 * 4) * 8
+    # one ticket counter (a 16-word line) per row; fp32: 1 word per tile (its pair), 2 per super-tile of 64 tiles (its
+    # pair and its end value); fp64: 4 and 6 (a word per 32-bit half).
+    assert hip.workspace_bytes(3, 4100, torch.float32, hip.FORWARD, plan) == (3 * 16 + 3 * 5 * 1 + 3 * 1 * 2) * 8
+    plan64 = hip.Plan(mode=hip.MODE_LOOKBACK, vec=2, unroll=2, waves=2)  # tile = 512 float64 elements: 9 tiles
+    assert hip.workspace_bytes(3, 4100, torch.float64, hip.FORWARD, plan64) == (3 * 16 + 3 * 9 * 4 + 3 * 1 * 6) * 8
 
 
 def test_every_automatic_plan_is_a_valid_plan():
