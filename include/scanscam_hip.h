@@ -261,6 +261,16 @@ int scanscam_resolve_plan(int64_t rows, int64_t T, int dtype, int direction, con
 int scanscam_resolve_plan_cl(int64_t batch, int64_t T, int64_t C, int dtype, int direction,
                              const scanscam_plan *plan, scanscam_plan *out);
 
+/*
+ * The duration in microseconds that the library's cost model estimates for a channels-last call on dense
+ * [batch, T, C] tensors with this plan (NULL or zero fields: with what the model itself chooses for them, i.e.
+ * the estimate behind scanscam_resolve_plan_cl). The automatic plan is the candidate with the smallest such
+ * estimate; the constants of the model are fitted to timings on one MI355X (scanscam_amd/plan_fit.py), so the
+ * figure is a ranking aid with an error of about 10 %, not a promise. No counterpart in the reference.
+ */
+int scanscam_predict_cl(int64_t batch, int64_t T, int64_t C, int dtype, int direction, const scanscam_plan *plan,
+                        double *microseconds);
+
 /* Static, never-freed description of an error code. */
 const char *scanscam_strerror(int code);
 

@@ -3,11 +3,20 @@
 // ratio of the counter readings to the known sizes turns the same counters, read for a scan kernel,
 // into bytes of HBM traffic. Not part of the library: `make calib` builds build/copy_calib.
 //   copy_calib [MiB = 1024] [launches = 20]
+// Two further modes stream without scanning, in the scan kernels' access shapes, to show what the memory
+// system gives those shapes when no scan, no ticket and no carry chain is involved:
+//   copy_calib mix      each mix of read and write streams (1R0W ... 3R2W; forward scan = 2R1W, backward = 3R2W),
+//                       67 108 864 fp32 per stream, and each workgroup shape (W waves x U 16-byte accesses per lane
+//                       and stream, all loads issued before the first store), 4 rotated buffer sets;
+//   copy_calib order    the look-back tile (8 waves x 4 accesses) in the look-back kernel's tile-major order of
+//                       work: the stream is cut into R rows and workgroup k takes tile k / R of row k % R, so tiles
+//                       of all R rows are in flight together (R = 1 is one linear sweep).
 #include <hip/hip_runtime.h>
 #include <stdio.h>
 #include <stdlib.h>
 
 typedef unsigned u4 __attribute__((ext_vector_type(4)));
+typedef float f4 __attribute__((ext_vector_type(4)));
 
 #define CHECK(call)                                                        \
     do {                                                                   \
@@ -27,8 +36,102 @@ __global__ __launch_bounds__(256) void copy_calib_kernel(const u4 *__restrict__ 
         if (i < n) __builtin_nontemporal_store(__builtin_nontemporal_load(in + i), out + i);
 }
 
+// READS input and WRITES output streams in the scan kernels' shape: workgroup k covers W * U consecutive 1 KiB
+// spans of every stream (wave w its U spans), or, with R > 1, tile k / R of row k % R of a stream cut into R rows.
+template <int READS, int WRITES, int U, int W>
+__global__ __launch_bounds__(W * 64) void stream_kernel(const f4 *__restrict__ a, const f4 *__restrict__ b,
+                                                         const f4 *__restrict__ c, f4 *__restrict__ o0,
+                                                         f4 *__restrict__ o1, unsigned R, size_t row_vecs, float never)
+{
+    const size_t base = (size_t)(blockIdx.x % R) * row_vecs + (size_t)(blockIdx.x / R) * (W * U * 64) +
+                        (threadIdx.x / 64) * (U * 64) + (threadIdx.x % 64);
+    f4 va[U], vb[U], vc[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        va[u] = __builtin_nontemporal_load(a + base + u * 64);
+        if (READS > 1) vb[u] = __builtin_nontemporal_load(b + base + u * 64);
+        if (READS > 2) vc[u] = __builtin_nontemporal_load(c + base + u * 64);
+    }
+    if (WRITES == 0) {  // the sum of what was read is compared with a value it never takes, so the loads stay
+        f4 s = 0;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            s += va[u];
+            if (READS > 1) s += vb[u];
+            if (READS > 2) s += vc[u];
+        }
+        if (s.x + s.y + s.z + s.w == never) o0[base] = s;
+        return;
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        f4 r = va[u];
+        if (READS > 1) r += vb[u];
+        if (READS > 2) r *= vc[u];
+        __builtin_nontemporal_store(r, o0 + base + u * 64);
+        if (WRITES > 1) __builtin_nontemporal_store(r + 1.0f, o1 + base + u * 64);
+    }
+}
+
+static const size_t kStreamElems = (size_t)16384 * 4096;  // fp32 per stream
+static f4 *g_sets[4][5];
+
+template <int READS, int WRITES, int U, int W> static int stream_case(unsigned R)
+{
+    const size_t vecs = kStreamElems / 4, tile_vecs = (size_t)W * U * 64;
+    hipEvent_t e0, e1;
+    CHECK(hipEventCreate(&e0));
+    CHECK(hipEventCreate(&e1));
+    const int launches = 40;
+    for (int i = -4; i < launches; i++) {
+        f4 **s = g_sets[(i + 4) % 4];
+        if (i == 0) CHECK(hipEventRecord(e0, 0));
+        hipLaunchKernelGGL((stream_kernel<READS, WRITES, U, W>), dim3((unsigned)(vecs / tile_vecs)), dim3(W * 64), 0, 0,
+                           s[0], s[1], s[2], s[3], s[4], R, vecs / R, -12345.0f);
+    }
+    CHECK(hipEventRecord(e1, 0));
+    CHECK(hipEventSynchronize(e1));
+    float ms = 0;
+    CHECK(hipEventElapsedTime(&ms, e0, e1));
+    ms /= launches;
+    const double bytes = (double)(READS + WRITES) * kStreamElems * 4;
+    printf("  %dR%dW  %2d waves x %d accesses  %5u rows  %7.1f us  %7.1f GB/s  %4.1f %% of 8 TB/s\n", READS, WRITES, W, U, R,
+           ms * 1e3, bytes / (ms * 1e-3) / 1e9, bytes / (ms * 1e-3) / 8e12 * 100);
+    CHECK(hipEventDestroy(e0));
+    CHECK(hipEventDestroy(e1));
+    return 0;
+}
+
+static int run_streams(bool order)
+{
+    for (auto &set : g_sets)
+        for (auto &p : set) {
+            CHECK(hipMalloc(&p, kStreamElems * 4));
+            CHECK(hipMemset(p, 0, kStreamElems * 4));
+        }
+    int rc = 0;
+    if (!order) {
+        printf("stream mixes, 67 108 864 fp32 per stream, non-temporal 16-byte accesses, 4 rotated buffer sets:\n");
+        rc |= stream_case<1, 0, 4, 4>(1) | stream_case<2, 0, 4, 4>(1) | stream_case<3, 0, 4, 4>(1);
+        rc |= stream_case<0 + 1, 1, 4, 4>(1) | stream_case<2, 1, 4, 4>(1) | stream_case<3, 2, 4, 4>(1);
+        printf("forward mix (2 reads + 1 write) by workgroup shape:\n");
+        rc |= stream_case<2, 1, 2, 4>(1) | stream_case<2, 1, 8, 4>(1) | stream_case<2, 1, 2, 8>(1) | stream_case<2, 1, 4, 8>(1) |
+              stream_case<2, 1, 8, 8>(1) | stream_case<2, 1, 2, 16>(1) | stream_case<2, 1, 4, 16>(1);
+        printf("backward mix (3 reads + 2 writes) by workgroup shape:\n");
+        rc |= stream_case<3, 2, 2, 4>(1) | stream_case<3, 2, 2, 8>(1) | stream_case<3, 2, 4, 8>(1) | stream_case<3, 2, 2, 16>(1) |
+              stream_case<3, 2, 4, 16>(1);
+    } else {
+        printf("order of work, 8 waves x 4 accesses (8192-element tiles), workgroup k -> tile k / R of row k %% R:\n");
+        for (unsigned R : {1u, 8u, 32u, 64u, 128u, 256u, 1024u}) rc |= stream_case<2, 1, 4, 8>(R);
+        for (unsigned R : {1u, 8u, 32u, 64u, 128u, 256u, 1024u}) rc |= stream_case<3, 2, 4, 8>(R);
+    }
+    CHECK(hipDeviceSynchronize());
+    return rc;
+}
+
 int main(int argc, char **argv)
 {
+    if (argc > 1 && (argv[1][0] == 'm' || argv[1][0] == 'o')) return run_streams(argv[1][0] == 'o');
     const size_t mib = argc > 1 ? (size_t)atol(argv[1]) : 1024;
     const int launches = argc > 2 ? atoi(argv[2]) : 20;
     if (mib < 1 || mib > 65536 || launches < 1) {

@@ -3,6 +3,7 @@
 #include "scanscam_hip.h"
 
 #include "scan_launch.hpp"
+#include "scan_cl_plan.hpp"
 
 #include <mutex>
 
@@ -64,7 +65,6 @@ int super_words(int dtype) { return dtype == SCANSCAM_F64 ? scanscam::kSuperWord
 // Bytes of the arithmetic type behind a storage type.
 int compute_size(int dtype) { return dtype == SCANSCAM_F64 ? 8 : 4; }
 
-bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
 
 int pow2_ceil(int64_t v)
 {
@@ -617,523 +617,33 @@ int run(bool rev, const void *a, const void *x, const void *h, void *y0, void *y
     return SCANSCAM_OK;
 }
 
-// Channels-last: choice of vector width, steps per wave and waves per workgroup.
-// `align`: the largest of 16, 8, 4 and the element size that every tensor's base and strides are multiples of (bytes).
+// Channels-last: the launch plan. `align`: the largest of 16, 8, 4 and the element size that every tensor's base
+// and strides are multiples of (bytes). The choice itself is the cost model of scan_cl_plan.hpp: every field the
+// caller's plan leaves at zero is chosen by the smallest estimated duration; this function turns the chosen
+// candidate into launch parameters and sizes.
 int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, int dtype, int align, bool rev,
-               scanscam::ClLaunch *l)
+               scanscam::ClLaunch *l, double *predicted_us = nullptr)
 {
     const int esize = elem_size(dtype);
-    const int full = 16 / esize;
-    const bool aligned16 = align >= 16, aligned4 = align >= 4;
+    if (esize == 0) return SCANSCAM_EDTYPE;
     scanscam_plan u = {0, 0, 0, 0, 0, 0};
     if (user) u = *user;
-    const bool vec_possible = aligned16 && (C % full == 0);
-    // The narrow lane: one channel, or two for 16-bit storage (4 bytes, like one fp32 channel).
-    const bool pair_possible = esize == 2 && aligned4 && (C % 2 == 0);
-    // The 8-byte lane: two fp32 channels, four 16-bit ones.
-    const int half = esize <= 4 ? full / 2 : 0;
-    const bool half_possible = half > 0 && align >= 8 && (C % half == 0);
-    auto groups = [&](int vec) { return (C + (int64_t)kWave * vec - 1) / ((int64_t)kWave * vec); };
-    // Workgroups that lanes of 4 or 8 bytes need before a workgroup walks all of T with them: three quarters of
-    // the CUs (two thirds backwards), not all 256 -- at 176 to 255 workgroups they still beat twice as many
-    // workgroups of the next narrower lane (fp32 [28, 4096, 1024] 287 / 473 -> 261 / 388 us, [24, 4096, 1024] 261 / 442 ->
-    // 228 / 361 us, bf16 [28, 4096, 2048] 300 / 513 -> 278 / 430 us, [56, 2048, 512] forward 81 -> 70 us).
-    const int64_t enough = rev ? 168 : 176;  // (forwards 192 at first: bf16 [189, 4702, 82], 189 workgroups of pairs, 123 us against 190 us in single channels)
-    // Pairs halve the number of workgroups: not where single channels reach 256 of them and pairs fall short.
-    const int narrow = pair_possible && (batch * groups(2) >= enough || batch * groups(1) < 256) ? 2 : 1;
-    // Element-aligned lanes: where C is no multiple of the lane's channels, or the tensors are only element-aligned,
-    // wider lanes are still possible in the kernel in which a workgroup walks all of T -- vectors loaded and
-    // stored at element alignment, the last lane of a time step on the window of channels that ends with it.
-    // Worth it when the wider lanes still give at least 256 workgroups and a time step fills a wave (not the
-    // packed kernel's regime).
-    auto ragged_fits = [&](int vec) { return vec > 1 && C >= (int64_t)kWave * vec && batch * groups(vec) >= 256; };
-    l->ragged = false;
-    if (u.vec) {
-        l->vec = u.vec;
-    } else if (!vec_possible) {
-        l->vec = narrow;
-        if (u.mode != kModeLookback) {
-            // A lane's fill is C / (groups(vec) * 64 * vec): the wide lanes only where they fill their waves to 65 %,
-            // whole (aligned) 8-byte lanes ahead of element-aligned 16-byte ones where they fill theirs 1.15 times
-            // better, and no element-aligned lane that fills worse than aligned pairs would (fp32 [700, 300, 257]
-            // 221 / 351 -> 179 / 328 us, [90, 2048, 514] 323 / 642 -> 308 / 540 us, bf16 241 / 406 -> 180 / 349 us).
-            auto fills65 = [&](int vec) { return C * 20 >= groups(vec) * kWave * vec * 13; };
-            const bool full_fits = ragged_fits(full) && fills65(full);
-            const bool half_whole = half_possible && ragged_fits(half);
-            const bool half_ragged = half > 1 && !half_possible && ragged_fits(half) && fills65(half) &&
-                                     !(pair_possible && groups(half) * half > groups(2) * 2);
-            // 16-bit storage with 256 to 384 workgroups of 16-byte lanes (one to one and a half per CU): twice as many
-            // of 8-byte lanes, whole or element-aligned, where those fill their waves as well (bf16 [128, 1024, 1003]
-            // 224 / 408 -> 200 / 358 us, [160, 1024, 1003] backward 660 -> 508 us, [128, 1024, 1501] backward 817 -> 557 us,
-            // [128, 1024, 777] 202 / 332 -> 151 / 280 us, [160, 1024, 1004] 271 / 673 -> 251 / 447 us; from 400 workgroups
-            // on the 16-byte lanes are ahead again, and fp32 keeps them throughout).
-            // (And on rows of fewer than 384 steps whatever the count: bf16 [39, 125, 4806] 35 / 91 -> 29 / 49 us, [209, 221, 1370]
-            // forward 98 -> 77 us.)
-            const bool half_instead = esize == 2 && full_fits && (batch * groups(full) <= 384 || T < 384) &&
-                                      groups(half) * half <= groups(full) * full &&
-                                      (half_whole || (half > 1 && ragged_fits(half) && fills65(half)));
-            if (half_instead) {
-                l->vec = half;
-                l->ragged = !half_possible;
-            } else if (half_whole && (!full_fits || groups(full) * full * 20 >= groups(half) * half * 23)) {
-                l->vec = half;  // whole 8-byte lanes, nothing element-aligned about them
-            } else if (full_fits) {
-                l->vec = full;
-                l->ragged = true;
-            } else if (half_ragged) {
-                l->vec = half;
-                l->ragged = true;
-            } else if (esize == 2 && !pair_possible && ragged_fits(2)) {
-                l->vec = 2;
-                l->ragged = true;
-            }
-            // With their stores left to the caches (below, and in the kernel for element-aligned lanes) the narrower
-            // lanes are ahead wherever they fill their waves 1.1 times better: 8-byte lanes in place of element-aligned
-            // 16-byte ones (fp32 [512, 512, 333] 290 / 469 -> 248 / 390 us, [128, 1024, 601] 249 / 440 -> 230 / 395 us,
-            // [64, 1024, 777] 148 / 246 -> 122 / 238 us), pairs of 16-bit channels in place of four-channel lanes (bf16
-            // [512, 512, 333] 143 / 247 -> 121 / 254 us, [128, 1024, 601] 150 / 253 -> 122 / 235 us).
-            // (1.2 times where the 16-byte lanes give more than 256 workgroups: fp32 [256, 1024, 777], 1.14 times, is
-            // 13 % faster forwards in 16-byte lanes and level backwards.)
-            if (l->vec == full && l->ragged && half > 1 && ragged_fits(half) &&
-                groups(full) * full * 10 >= groups(half) * half * (batch * groups(full) <= 256 ? 11 : 12)) {
-                l->vec = half;
-                l->ragged = !half_possible;
-            }
-            if (esize == 2 && l->vec == half && half > 2 && (pair_possible || ragged_fits(2)) && batch * groups(2) >= 256 &&
-                groups(half) * half * 10 >= groups(2) * 2 * 11) {
-                l->vec = 2;
-                l->ragged = !pair_possible;
-            }
-            // fp32 forwards on rows of fewer than 384 steps: 8-byte lanes in place of element-aligned 16-byte ones
-            // ([209, 221, 1370] 179 -> 137 us, [90, 344, 1686] 148 -> 116 us, [39, 125, 4806] 63 -> 51 us; backwards level).
-            if (esize == 4 && !rev && T < 384 && l->vec == full && l->ragged && ragged_fits(half)) {
-                l->vec = half;
-                l->ragged = !half_possible;
-            }
-            // 65 to 127 channels that allow no whole pairs (an odd count, or tensors on odd elements): single channels are
-            // two waves per time step, the second mostly empty, and element-aligned pairs one. With a workgroup per
-            // batch element or more -- fp32 [2000, 1000, 65] 497 / 918 -> 367 / 624 us, [476, 1998, 113] 342 / 588 -> 277 / 480 us,
-            // [3964, 290, 89] 338 / 685 -> 266 / 466 us, bf16 [476, 1998, 113] 224 / 570 -> 150 / 262 us, [2000, 1000, 65] 260 / 660
-            // -> 227 / 412 us, [438, 1181, 93] 104 / 232 -> 84 / 139 us; 8 steps in 8 waves (16 steps lose 10 to 25 % backwards).
-            // (From 340 workgroups on: 300 are a round and a sixth, and there bf16 [300, 1000, 77] is 23 % slower forwards.)
-            if (esize <= 4 && l->vec == 1 && !l->ragged && C > kWave && C < 2 * kWave && batch >= 340 &&
-                u.mode == SCANSCAM_MODE_AUTO) {
-                l->vec = 2;
-                l->ragged = true;
-            }
-            // 16-bit storage backwards, too few workgroups for the rule above but enough for a walk in pairs (168):
-            // element-aligned pairs rather than single channels, walked or in tiles over time -- bf16 [71, 1910, 257]
-            // 159 -> 124 us, [101, 1576, 219] 155 -> 124 us, [14, 1439, 1473] 121 -> 104 us, [64, 2048, 257] 141 -> 129 us.
-            if (esize == 2 && rev && l->vec == 1 && !pair_possible && C >= 2 * kWave && u.mode == SCANSCAM_MODE_AUTO &&
-                batch * groups(2) >= enough && batch * groups(2) < 256) {
-                l->vec = 2;
-                l->ragged = true;
-            }
-        }
-    } else {
-        // A workgroup owns 64*vec channels of one batch element. Enough of them: 16-byte loads.
-        // Not enough: narrow lanes, which give full/narrow times as many workgroups; if even those
-        // are too few, time is split over workgroups as well (below), and there too the narrow lanes
-        // win: more, narrower carry chains (fp32 1.1-1.7 times faster than 16-byte lanes, measured from
-        // [1, 262144, 256] to [8, 4096, 512]; 16-bit storage 2.5-16 times, its 16-byte lanes leave
-        // 8 times fewer chains).
-        // A lane width whose last channel group is partly empty moves fewer bytes per workgroup in the same time
-        // (the kernels run at 1 / fill of their speed: fp32 C = 320, 83 % fill in pairs and 63 % in fours, 199 / 338 us
-        // and 225 / 375 us against 179 / 316 us with single channels), so a wider lane has to fill its groups
-        // within 5 % of the narrow one.
-        auto fills = [&](int vec) { return 21 * groups(narrow) * narrow >= 20 * groups(vec) * vec; };
-        // (Up to 32 channels several time steps share a wave whatever the lane, and the walk starts at 80 workgroups, below.)
-        l->vec = (C <= 32 ? batch >= 80 : (batch * groups(full) >= 256 && fills(full))) ? full : narrow;
-        // 8-byte lanes, where they still give 256 workgroups and fill their waves as well: they
-        // stream as fast as 16-byte lanes or faster at equal shapes (two or four times the waves per byte in
-        // flight: fp32 [256, 1024, 1024] 71 / 76 -> 80 / 74 % of peak, [128, 2048, 512] 72 / 70 -> 78 / 75 %, bf16
-        // [256, 1024, 1024] 69 / 68 -> 75 / 74 %, [160, 2048, 1024] 59 / 57 -> 70 / 69 %) and reach shapes where 16-byte
-        // lanes leave too few workgroups and narrow lanes were the only choice (fp32 [32, 2048, 1024] 67 / 65 ->
-        // 73 / 78 %, [64, 2048, 512] 67 / 66 -> 75 / 70 %, bf16 [32, 4096, 2048] 66 / 62 -> 69 / 72 %).
-        // (Time steps that are not whole 128-byte lines keep 16-byte lanes where those give 256 workgroups:
-        // fp32 [64, 2048, 1016] backward 57 % against 50 %. 16-bit storage in rows of fewer than 384 steps does not: bf16
-        // [256, 333, 1000] 125 / 207 -> 100 / 194 us, [512, 256, 1000] 184 / 324 -> 149 / 296 us; [300, 400, 1512] is 6 % faster
-        // in 16-byte lanes, [256, 1024, 1000] 18 %.)
-        // (16-bit storage keeps 256 for its four-channel lanes: bf16 [28, 4096, 2048] gains with 224 workgroups of
-        // them, [72, 2048, 768] loses 15 % with 216.)
-        // (And the backward pass of fp32 with 2048 or more channels: [32, 2048, 2048] 437 us against 505-530 us,
-        // [64, 1024, 2048] 466 against 508 us, [128, 1024, 2048] 911 against 1025 us, [40, 2048, 4096] 1219 against 1276 us;
-        // with 512 or fewer time steps in workgroups of 4 waves (below): [256, 512, 2048] 967 against 1088 us,
-        // [64, 512, 4096] 492 against 508 us, 516 us with 16 waves; rows of 128 steps keep the 8-byte lanes:
-        // [256, 128, 4096] 460 against 495 us.)
-        // (16-bit storage likewise from 4096 channels on: bf16 [16, 2048, 8192] backward 548 -> 465 us, [32, 2048, 4096]
-        // 486 -> 448 us, [64, 1024, 4096] 486 -> 462 us; with 2048 channels the four-channel lanes are 10 % ahead, and so
-        // they are with 512 time steps or where the 16-byte lanes' workgroups are no whole rounds of 256:
-        // [64, 512, 4096] 241 against 280 us, [40, 2048, 4096] 645 against 765 us.)
-        if (half_possible && C >= (int64_t)kWave * half && fills(half) &&
-            batch * groups(half) >= (esize == 2 ? 256 : enough) &&
-            (l->vec != full || (C * esize) % 128 == 0 || (esize == 2 && T < 384)) &&
-            !(l->vec == full && esize == 4 && rev && C >= 2048 && (batch * groups(full) < 512 || T >= 256)) &&
-            !(l->vec == full && esize == 2 && rev && C >= 4096 && T >= 1024 &&
-              batch * groups(full) * 10 >= ((batch * groups(full) + kComputeUnits - 1) / kComputeUnits) * kComputeUnits * 9))
-            l->vec = half;
-        // float64: its 8-byte lane is the single channel, and the same holds (fp64 [64, 2048, 512] 283 / 446 -> 258 / 429 us,
-        // [256, 1024, 256] 272 / 456 -> 251 / 434 us with 8 waves of 8 steps).
-        // (From 128 channels on; backwards only where the 16-byte lanes give 512 workgroups: at 256 of them,
-        // [32, 2048, 1024], the backward pass is 16 % faster in 16-byte lanes.)
-        if (esize == 8 && l->vec == full && C >= 2 * kWave && batch * groups(1) >= enough &&
-            groups(1) * 20 <= groups(full) * full * 21 && (!rev || batch * groups(full) >= 512))
-            l->vec = 1;
-        // Few channels (the packed kernel, below): a wide lane leaves more steps per instruction to scan
-        // across with lane shuffles, which costs more than the wider loads gain -- except where C is not a
-        // power of two and one channel per lane would leave a quarter of 32 lanes idle (fp32 [256, 8192, 24]:
-        // 177 / 235 us with 16-byte lanes, 209 / 320 with 4-byte lanes; [512, 4096, 8]: 66 / 80 against 44 / 67).
-        if (C <= 32 && (esize == 2 || pow2_ceil(C) <= 16 || is_pow2((int)C))) l->vec = narrow;
-        // 16-bit storage, 33 to 511 channels: with 8 channels per lane a time step fills only part of a wave, and
-        // the kernel that then packs several steps into a wave needs more registers than it has (bf16
-        // [256, 512, 256]: 28 / 29 % of peak; [256, 4096, 64]: 25 / 28 %). One channel per lane at exactly 64
-        // channels (a full wave: 61 / 62 %), two otherwise (66 / 68 % at 256 channels; 47 / 48 % at 96, where single
-        // channels would split a step into a full and a half-empty wave: 33 / 31 %; 46 / 46 % at 56, two steps per
-        // instruction, against 33 / 29 %).
-        if (esize == 2 && C > 32 && C < (int64_t)kWave * full) {
-            l->vec = (C == kWave || !pair_possible) ? 1 : 2;
-            // Measured later, over rotated buffers at 512 or more batch elements: 129 to 256 channels fill one wave
-            // of four-channel lanes, and a batch element is then one workgroup's contiguous block (C = 200: 201 / 376
-            // -> 121 / 248 us, C = 256: 147 / 261 -> 141 / 249 us); 320 or 448 channels are whole waves of single
-            // channels but leave the last wave of pairs half empty (C = 320: 215 / 358 -> 186 / 353 us, C = 448: 302 /
-            // 504 -> 264 / 494 us); at exactly 64 channels the backward pass is faster in pairs (98 -> 70 us).
-            // (pairs that fill their two waves keep them: C = 256 at 256 batch elements 73 / 128 us against 87 / 137 us)
-            // (With the next tile's loads issued ahead, from 256 batch elements on; at exactly 256 channels pairs with
-            // 16 steps, below, are level at 256 batch elements and 7 % ahead backwards at 512 and 2048.)
-            // (192 channels, three whole waves of single channels, with 16 steps: [512, 2048, 192] 245 / 402 -> 233 / 389 us.)
-            const bool odd_waves = C > 2 * kWave && C % kWave == 0 && C % (2 * kWave) != 0;
-            if (odd_waves && (C > 4 * kWave || T >= 512)) l->vec = 1;
-            else if (C > 2 * kWave && C <= 4 * kWave && C % (2 * kWave) != 0 && half_possible && batch >= 256) l->vec = half;
-            // (At exactly 64 channels, with loads issued a tile ahead: single channels in both directions, 8 waves of
-            // 16 steps -- [256, 4096, 64] 78 / 153 -> 76 / 131 us, [2048, 512, 64] 74 / 130 -> 69 / 124 us, [4096, 256, 64]
-            // forward 77 -> 65 us; pairs are 0 to 15 % behind backwards now and 5 to 25 % forwards. Rows of fewer than 256
-            // steps are shorter than two such tiles and keep pairs backwards.)
-            if (C == kWave && rev && pair_possible && batch >= 256 && T < 256) l->vec = 2;
-        }
-    }
-    // fp32 with fewer than 128 channels and a workgroup per batch element: pairs of channels (8-byte lanes) with 8
-    // steps per wave, whether a time step fills a wave or several steps share one; a single channel per lane
-    // at exactly 64. Against 16-byte lanes with 4 steps: [2048, 512, 40] 41 / 56 -> 56 / 56 % of peak, [1024, 1024, 48]
-    // 47 / 59 -> 60 / 59 %, [512, 2048, 96] 54 / 61 -> 64 / 64 %, [256, 4096, 64] 60 / 68 -> 73 / 67 %; against single
-    // channels with 4 steps: [4096, 1024, 8] 63 / 65 -> 73 / 72 %.
-    // (From the `enough` workgroups of above on, not only from 256: [234, 1315, 72] forward 84 -> 64 us.)
-    if (!u.vec && esize == 4 && C < 2 * kWave && batch >= (C > 32 ? enough : 256) && u.mode != kModeLookback) {
-        if (C == kWave) l->vec = 1;
-        else if (half_possible) l->vec = 2;
-    }
-    // Fewer than 64 channels and two or more workgroups per CU, measured again over every plan: fp32 up to 32
-    // channels in 16-byte lanes, 4 steps, 4 waves ([540, 4225, 8] 68 / 105 -> 53 / 96 us, [907, 3157, 24] 220 / 356 ->
-    // 201 / 325 us, [929, 1083, 16] 50 / 73 -> 46 / 69 us; backwards from one workgroup per CU on: [306, 6590, 16] 164 ->
-    // 135 us, forwards 97 -> 121 us). 33 to 63 channels: forwards a single channel per lane (fp32 16 steps in 8 waves:
-    // [2048, 512, 40] 114 -> 92 us, [1024, 1024, 48] 126 -> 104 us; bf16 [2048, 512, 40] 87 -> 74 us, [1024, 1024, 48]
-    // 88 -> 76 us), backwards 16-byte lanes of fp32 (190 -> 172 us, 214 -> 211 us) and four-channel lanes of 16-bit
-    // storage (135 -> 125 us, 137 -> 126 us), in 4 waves.
-    bool small_fours = false, small_singles = false;
-    if (!u.vec && u.mode != kModeLookback && C < kWave && esize == 4) {
-        if (C <= 32 ? (vec_possible && batch >= (rev ? 256 : 512)) : (vec_possible && rev && batch >= 512)) {
-            l->vec = full;
-            small_fours = true;
-        } else if (C > 32 && !rev && batch >= enough) {  // (forwards from 176 workgroups on: [231, 773, 56] 37 -> 29 us, bf16 30 -> 20 us)
-            l->vec = 1;
-            small_singles = true;
-        }
-    }
-    if (!u.vec && u.mode != kModeLookback && C < kWave && C > 32 && esize == 2 && batch >= (rev ? 512 : enough)) {
-        if (!rev) {
-            l->vec = 1;
-        } else if (half_possible && T >= 512) {  // (shorter rows keep pairs: [5159, 257, 40] 194 against 224 us, [827, 388, 40] 55 against 59 us)
-            l->vec = half;
-            small_fours = true;
-        }
-    }
-    if (l->vec != 1 && l->vec != full && !(l->vec == 2 && esize == 2) && !(half > 1 && l->vec == half)) return SCANSCAM_EPLAN;
-    // A forced wide lane that the alignment or C does not allow as it stands: element-aligned, where that kernel applies.
-    if (u.vec && ((l->vec == full && full > 1 && !vec_possible) || (l->vec == 2 && esize == 2 && full != 2 && !pair_possible) ||
-                  (half > 1 && l->vec == half && !half_possible))) {
-        // (more than half a wave of such lanes per time step: below that several steps share a wave, in a kernel of whole lanes)
-        if (C <= (int64_t)(kWave / 2) * l->vec || u.mode == kModeLookback) return SCANSCAM_EPLAN;
-        l->ragged = true;
-    }
-    // Too few (batch element, channel group) pairs to fill the GPU: cut time into tiles over
-    // workgroups as well. kind 0: one workgroup walks all of T. kind 2: tiles by ticket with a
-    // look-back chain of per-channel pairs (mode = SCANSCAM_MODE_LOOKBACK forces it,
-    // SCANSCAM_MODE_ROW forbids it).
-    int64_t rowgroups = batch * groups(l->vec);
-    l->kind = 0;
-    const bool wide_enough = esize == 2 ? l->vec == 2 : l->vec > 1;  // pairs of 16-bit channels, 8- or 16-byte fp32 lanes
-    // (Up to 32 channels a wave of the tiles' kernel is mostly empty lanes, and the walk, which packs several time steps
-    // into a wave, is ahead from 80 workgroups on: fp32 [128, 8192, 16] 99 / 168 -> 68 / 94 us, [200, 4000, 24] backward
-    // 138 -> 98 us, [95, 8181, 16] 82 / 132 -> 72 / 96 us, bf16 [128, 8192, 16] 125 / 273 -> 65 / 90 us; at 64 workgroups the
-    // tiles are ahead forwards and level backwards.)
-    // (17 to 32 channels fill a quarter to a half of a tile's wave, and there the tiles hold out up to 192 workgroups: fp32
-    // [139, 11578, 23] 237 / 352 us walked, 173 / 290 us in tiles, [123, 5560, 28] forward 102 against 76 us, [176, 9879, 19]
-    // 198 against 174 us; [200, 4000, 24] is level forwards and 40 % faster backwards in the walk.)
-    // (16-bit storage backwards keeps the walk: bf16 [123, 5560, 28] 115-133 us walked, [64, 16384, 16] 159 against 187 us.)
-    const bool one_wave_singles = l->vec == 1 && C > 32 && C < kWave;  // (33 to 63 channels forwards, above)
-    const int64_t walk_from = (C <= 16 || (C <= 32 && esize == 2 && rev)) ? 80
-                              : (C <= 32 ? 192 : ((wide_enough || one_wave_singles) ? enough : 256));
-    if (u.mode == kModeLookback || (u.mode == SCANSCAM_MODE_AUTO && rowgroups < walk_from)) l->kind = 2;
-    // (Those tiles of 16-bit storage in single channels, 16 lanes of a wave rather than 8: bf16 [64, 16384, 16] forward
-    // 135 -> 103 us, backward 283 -> 187 us.)
-    // (And wherever pairs would fill their waves to less than 70 % and single channels do better: [73, 14486, 40]
-    // 149 / 296 -> 114 / 211 us, [84, 7773, 56] 96 / 183 -> 76 / 146 us, [92, 1781, 56] 30 / 55 -> 25 / 42 us.)
-    if (l->kind == 2 && !u.vec && esize == 2 && l->vec == 2 &&
-        (C <= 32 || (groups(2) * kWave * 2 * 7 > C * 10 && groups(2) * 2 > groups(1)))) {
-        l->vec = 1;
-        rowgroups = batch * groups(1);
-    }
-    if (l->kind == 2 && !u.vec && C <= 32 && l->vec != 1) {  // (fp32 likewise: [123, 5560, 28] forward 76 us)
-        l->vec = 1;
-        rowgroups = batch * groups(1);
-    }
-    if (u.mode == kModeSmall) return SCANSCAM_EPLAN;
-    // A few more than 256 workgroups (up to 340) leave some CUs with twice the work of the others. Tiles over
-    // workgroups are taken instead, with the lanes that measure best there in each direction (below): fp32
-    // [20, 4096, 2048] forward 430 -> 354 us, [24, 2048, 1536] 194 / 360 -> 170 / 273 us, [68, 2048, 512] forward 183 ->
-    // 153 us, bf16 [24, 2048, 3072] backward 374 -> 305 us, [12, 4096, 3072] 231 / 399 -> 191 / 286 us. Exactly 256
-    // workgroups are one per CU, and from 350 on the walk is the faster one.
-    // (The same one round later: 520 workgroups are 2.03 rounds. And with few channels, where a batch element is a
-    // workgroup, from 40 channels on (below that several time steps share a wave): fp32 [260, 4000, 48]
-    // 207 / 348 -> 139 / 237 us, bf16 204 / 307 -> 108 / 201 us, fp32 [300, 1000, 77] 113 / 205 -> 93 / 168 us.)
-    const int64_t rounds_up = (rowgroups + kComputeUnits - 1) / kComputeUnits;
-    // (Up to 0.8 of the rounds they start, from 64 channels on, for the forward pass of fp32 and for lanes of a single
-    // channel -- of 16-bit storage backwards only: fp32 [300, 1024, 256] forward 192 -> 167 us, [400, 1024, 256] 247 ->
-    // 216 us, [150, 2048, 512] 351 -> 324 us, [300, 1000, 77] 112 / 206 -> 92 / 169 us, bf16 backward 147 -> 125 us.)
-    const bool to_08 = C >= 64 && (esize == 4 ? (!rev || l->vec == 1) : (rev && l->vec == 1));
-    // (fp32 in element-aligned lanes as well, which then gives way to tiles of single channels: [14, 3757, 2539], 280
-    // workgroups of pairs, 511 / 929 -> 392 / 668 us, [24, 3000, 1473] 385 / 703 -> 311 / 529 us, [48, 2000, 777] 238 / 436 ->
-    // 217 / 362 us; 16-bit storage gains nothing there.)
-    const bool few_too_many = l->kind == 0 && !u.vec && u.mode == SCANSCAM_MODE_AUTO && (!l->ragged || esize == 4) && rowgroups > 256 &&
-                              rowgroups * 10 < rounds_up * kComputeUnits * (to_08 && !l->ragged ? 8 : 7) && T >= 512 && C >= 40;
-    // (16-bit storage backwards only where four-channel lanes, the ones its tiles need, fill their waves.)
-    // (filling them to 85 %: bf16 C = 1600, 89 %, gains 11 % backwards in such tiles, C = 640, 83 %, loses 8 %)
-    const bool half_fits = half_possible && C >= (int64_t)kWave * half && C * 20 >= groups(half) * kWave * half * 17;
-    // Its pairs make poor tiles backwards, so without four-channel lanes it stays with the walk -- bf16 [300, 2048, 128]
-    // 189 us against 218 us in tiles -- unless the pairs leave most of a wave empty: [260, 4000, 48] 308 -> 201 us in
-    // tiles of single channels.)
-    const bool pairs_fill = groups(2) * kWave * 2 * 7 <= C * 10;
-    // (With many channel groups per batch element the tiles of pairs win all the same: bf16 [16, 4096, 2050] 572 -> 403 us.)
-    // (Forwards it needs pairs that fill their waves to 85 %, from 64 channels on: bf16 [520, 2000, 96], 75 %, 138 us in the
-    // walk and 156 us in tiles, [300, 1000, 200], 78 %, 93-98 against 105 us, [100, 3000, 300] 172 against 179 us; and the
-    // tiles are of pairs, not of the four-channel lanes the walk chose: [24, 2048, 3072] 220 -> 197 us, [130, 2048, 512]
-    // 200 -> 173 us.)
-    const bool pairs_fill_fwd = C < kWave || groups(2) * kWave * 2 * 17 <= C * 20;
-    // (Neither exception where the walk would be in single channels: bf16 [77, 11371, 212], 308 workgroups of them,
-    // 544 / 941 us.)
-    if (few_too_many && !(esize == 2 && rev && l->vec != 1 && !half_fits && pairs_fill && groups(2) < 8) &&
-        !(esize == 2 && !rev && l->vec != 1 && !pairs_fill_fwd)) {
-        l->kind = 2;
-        if (l->ragged) {
-            l->vec = 1;
-            l->ragged = false;
-        }
-        if (l->vec == full && full > 1) l->vec = narrow;
-        if (esize == 2 && !rev && l->vec == half) l->vec = narrow;
-        // single channels where the lane chosen so far leaves more than 30 % of its waves empty and they do better
-        if (groups(l->vec) * kWave * l->vec * 7 > C * 10 && groups(l->vec) * l->vec > groups(1)) l->vec = 1;
-        rowgroups = batch * groups(l->vec);
-    }
-    // fp32 backwards in single channels on time steps that are no whole 128-byte lines: the walk of all of T runs at
-    // 35-40 % of peak whatever the number of workgroups, tiles over time at 45-50 % -- [476, 1998, 113] 770 -> 587 us,
-    // [551, 3705, 59] 779 -> 557 us, [1000, 500, 130] 434 -> 358 us, [986, 969, 157] 931 -> 769 us, [438, 1181, 93] 327 ->
-    // 272 us, [100, 3000, 300] 553 -> 442 us. (Whole lines, [1024, 1024, 64], gain nothing.)
-    // (Pairs likewise, element-aligned ones giving way to single channels: [90, 2048, 514] 532 -> 442 us, [1429, 456, 202]
-    // 804 -> 677 us, [84, 1772, 216] 168 -> 137 us, [32, 4096, 999] 731 -> 652 us.)
-    // (From 384 steps on -- [1599, 379, 79] and [228, 402, 94] gain 11 and 22 % -- and element-aligned pairs from 2048:
-    // [512, 512, 333] is 13 % faster in their walk. Tiles of pairs where those fill their waves within 20 % of single
-    // channels: [1000, 500, 130] 425 us in pairs, 352 us in single channels.)
-    // (Forwards the walk holds up on rows of about 1000 steps and the tiles are 10 to 20 % ahead from about 2000 on:
-    // [476, 1998, 113] 379 -> 344 us, [551, 3705, 59] 359 -> 319 us, [107, 2371, 206] 159 -> 130 us, [90, 2048, 514] 298 ->
-    // 256 us; [986, 969, 157] and [438, 1181, 93] are level, and element-aligned pairs keep their walk.)
-    if (l->kind == 0 && !u.vec && u.mode == SCANSCAM_MODE_AUTO && esize == 4 && l->vec <= 2 && C > 32 &&
-        (rev ? T >= (l->ragged ? 2048 : 384) : (T >= 1900 && !l->ragged)) && (C * esize) % 128 != 0 &&
-        !(l->ragged && groups(2) == 1)) {  // (one wave of element-aligned pairs walks at 50-57 % of peak: above)
-        l->kind = 2;
-        // ([90, 2048, 514]: 436 us in pairs, 462 us in single channels; [100, 3000, 300], 0.83 of the fill: 265 / 439 against 288 / 476 us)
-        l->vec = (half_possible && groups(2) * 2 * 8 <= groups(1) * 10) ? 2 : 1;
-        l->ragged = false;
-        rowgroups = batch * groups(l->vec);
-    }
-    // Tiles over workgroups, lanes chosen here: 8-byte lanes where C fills whole waves of them, in the
-    // direction in which they measured faster than the narrow lane (16 steps per wave either way) -- the
-    // backward pass of 16-bit storage (bf16 [8, 4096, 512] 48 -> 38 us, [8, 4096, 2048] 166 -> 140 us,
-    // [1, 262144, 256] 198 -> 167 us; forward 3 to 10 % slower) and the forward pass of fp32
-    // ([8, 4096, 512] 47 -> 44 us, [1, 262144, 256] 203 -> 182 us; backward 15 to 25 % slower).
-    if (l->kind == 2 && !u.vec && half_fits && (esize == 2 ? rev : !rev)) {
-        l->vec = half;
-        rowgroups = batch * groups(half);
-    }
-    // (16-bit storage backwards from 53 % fill on, 128 channels or more: bf16 [79, 3383, 136] 178 -> 126 us, [148, 3569, 144]
-    // 317 -> 240 us, [53, 2498, 168] 96 -> 74 us, [15, 6680, 188] 81 -> 62 us, [60, 884, 208] 42 -> 32 us, [13, 2082, 400] 47 -> 37 us.)
-    if (l->kind == 2 && !u.vec && esize == 2 && rev && half_possible && l->vec != half && C >= 2 * kWave &&
-        groups(half) * kWave * half * 53 <= C * 100) {
-        l->vec = half;
-        rowgroups = batch * groups(half);
-    }
-    // Forwards, pairs in place of single channels wherever they fill their waves as well (half as many waves for the
-    // same channels): fp32 [51, 9920, 82] 163 -> 120 us, [160, 1995, 68] 84 -> 70 us, [42, 4018, 112] 64 -> 56 us, bf16
-    // [160, 1995, 68] 64 -> 50 us.
-    if (l->kind == 2 && !u.vec && !rev && l->vec == 1 && C > kWave && (esize == 2 ? pair_possible : half_possible) &&
-        esize <= 4 && groups(2) * 2 <= groups(1)) {
-        l->vec = 2;
-        rowgroups = batch * groups(2);
-    }
-    // fp32 backwards on time steps that are no whole 128-byte lines: pairs of channels with 8 steps, where they
-    // fill their waves as well as single channels do ([20, 8192, 250] 265 -> 214 us, [48, 2048, 1500] 860 -> 706 us,
-    // [8, 4096, 1000] 178 -> 155 us, [260, 2000, 66] 305 -> 244 us; with whole lines single channels are level or ahead).
-    if (l->kind == 2 && !u.vec && esize == 4 && rev && half_possible && (C * esize) % 128 != 0 &&
-        groups(2) * 2 <= groups(1)) {
-        l->vec = 2;
-        rowgroups = batch * groups(2);
-    }
-    // The backward pass of 16-bit storage takes the same tiles of four-channel lanes where the alternative is 256 to
-    // 511 workgroups of single-channel lanes walking all of T (a wave's access is 128 bytes there): bf16
-    // [4, 8192, 4096] 292 -> 265 us, [2, 16384, 8192] 584 -> 510 us, [16, 4096, 1024] 144 -> 140 us, [8, 4096, 2048]
-    // 148-185 -> 150 us over rotated buffers; forwards the single channels are 5 to 20 % faster.
-    if (l->kind == 0 && !u.vec && u.mode == SCANSCAM_MODE_AUTO && esize == 2 && rev && l->vec <= 2 && !l->ragged &&
-        (l->vec == 1 || rowgroups < 256) && half_fits && batch * groups(half) < 256 && T >= 1024) {
-        l->kind = 2;
-        l->vec = half;
-        rowgroups = batch * groups(half);
-    }
-    if (l->ragged && l->kind != 0) return SCANSCAM_EPLAN;  // (the automatic choice never gets here: it asked for 256 workgroups)
+    if (u.mode != SCANSCAM_MODE_AUTO && u.mode != kModeRow && u.mode != kModeLookback) return SCANSCAM_EPLAN;
+    const scanscam::ClShape shape = {batch, T, C, esize, compute_size(dtype), align, rev};
+    scanscam::ClCandidate c;
+    if (!scanscam::cl_choose(shape, u, &c, predicted_us)) return SCANSCAM_EPLAN;
 
-    // Steps per wave per tile: with one channel per lane and tiles over workgroups, 16 (8 measured 1.2-1.4
-    // times slower: twice as many tiles pay the carry wait).
-    // Few channels: a time step fills `group` lanes only, and a wave holds 64 / group consecutive steps
-    // per instruction (the packed kernel; a workgroup then owns a whole batch element).
-    l->group = kWave;
-    if (l->kind == 0 && groups(l->vec) == 1) {
-        const int g = pow2_ceil((C + l->vec - 1) / l->vec);
-        if (g < kWave) l->group = g;
-    }
-
-    // 16-bit storage moves half as many bytes per step of a narrow lane. Where there is only about one
-    // workgroup per CU (fewer than 512 of them) that leaves too little in flight, and a workgroup that walks
-    // all of T takes 16 steps per wave as well: forward +5 to +11 points of peak (bf16 [16, 4096, 1024]
-    // 48 -> 59 %, [128, 2048, 256] 56 -> 67 %), backward -2 to +4. With more workgroups, or rows too short to
-    // fill such tiles, it costs 2 to 10 points; fp32 gains nothing from it.
-    const bool narrow_lane = l->vec < full;
-    // (element-aligned pairs of 16-bit channels likewise: bf16 [64, 2048, 1001] 36 / 34 -> 39 / 38 % of peak)
-    // (and of fp32 channels: [512, 512, 333] backward 502 -> 390 us, [256, 1024, 777] 1246 -> 962 us, [128, 1024, 1003] 747 -> 664 us)
-    // (Several time steps per wave, the packed kernel: only up to one workgroup per CU -- bf16 [306, 6590, 16] 117 / 163 us
-    // with 16 steps, 84 / 107 us with 8; [128, 8192, 16] 65 / 90 against 70 / 89 us.)
-    const bool one_wave_ragged_pairs = l->ragged && l->vec == 2 && groups(2) == 1;  // (65 to 127 channels, above: 8 steps)
-    const bool long_steps = l->kind != 0 ||
-                            (esize == 2 && l->vec <= 2 && T >= 1024 && (rowgroups < 512 || (l->ragged && l->vec == 2)) &&
-                             (l->group == kWave || rowgroups <= kComputeUnits) && !one_wave_ragged_pairs) ||
-                            small_singles ||
-                            // (fp32 forwards in single channels from two workgroups per CU on, with 8 waves: [3237, 206, 192] 295 ->
-                            // 255 us, [1704, 67, 85] 49 -> 38 us, [2106, 99, 64] 37 -> 29 us, [5005, 328, 21] 185 -> 149 us; on rows of
-                            // fewer than 512 steps -- [1024, 1024, 64] and [700, 512, 192] are level, [986, 969, 157] loses 26 % -- and
-                            // not on an odd number of channels above 64: [3964, 290, 89] 342 -> 413 us, though [1704, 67, 85] gains.
-                            // Backwards 16 waves of 8 steps stay ahead with few channels.)
-                            (esize == 4 && !rev && l->vec == 1 && l->kind == 0 && rowgroups >= 2 * kComputeUnits && T < 512 &&
-                             (C % 2 == 0 || groups(1) == 1)) ||
-                            (esize == 4 && l->ragged && l->vec == 2 && !one_wave_ragged_pairs) ||
-                            // (with loads issued a tile ahead, every walk in narrow 16-bit lanes whose time step fills its
-                            // waves' lanes: bf16 [512, 1024, 256] 148 / 257 -> 145 / 238 us, [2048, 512, 128] backward 256 ->
-                            // 237 us, [512, 1024, 320] 184 / 331 -> 179 / 309 us, [1024, 1024, 64] backward 142 -> 124 us)
-                            // Rows shorter than a few such tiles lose: [4096, 128, 128] backward 114 -> 127 us, [1500, 100, 130]
-                            // 38 / 64 -> 45 / 84 us, element-aligned [700, 300, 257] 82 / 143 -> 94 / 188 us; the single channels of
-                            // 64 or fewer gain forwards from one tile on: [4096, 128, 64] 48 -> 35 us, [1024, 200, 64] 20.5 -> 18.2 us,
-                            // [5159, 257, 40] 134 -> 101 us.
-                            // (Nor do single channels backwards on an odd number of channels above 64, which stay with 16 waves of 8 steps:
-                            // [2000, 1000, 65] 664 against 810 us, [438, 1181, 93] 236 against 269 us, [1599, 379, 79] 215 us against
-                            // 256 us in 4 waves.)
-                            (esize == 2 && l->vec <= 2 && l->kind == 0 && l->group == kWave && !l->ragged &&
-                             !(rev && l->vec == 1 && !pair_possible && groups(1) >= 2) &&
-                             T >= (l->vec == 1 && C <= kWave ? (rev ? 256 : 64) : 512));
-    l->steps = u.unroll ? u.unroll : (narrow_lane ? (long_steps ? 16 : 8) : ((l->kind != 0 && full <= 4) ? 8 : 4));
-    // Tiles of 8-byte fp32 lanes backwards (kept from the choice above where there are a few workgroups too many):
-    // 8 steps, which fit 104 registers where 16 need 129 (fp32 [520, 2000, 96] 504 -> 438 us).
-    if (!u.unroll && l->kind == 2 && esize == 4 && l->vec == 2 && rev) l->steps = 8;
-    // (float64 in its 8-byte lanes likewise: [8, 4096, 512] backward 148 -> 130 us)
-    if (!u.unroll && l->kind == 2 && esize == 8 && l->vec == 1 && rev) l->steps = 8;
-    // A walk of all of T in 8-byte fp32 lanes forwards, 2048 or more channels: 16 steps per wave ([64, 1024, 2048]
-    // 292 -> 266 us, [256, 512, 2048] 589 -> 525 us, [512, 256, 2048] 561 -> 499 us, [128, 1024, 2048] 586 -> 535 us,
-    // [40, 2048, 4096] 712 -> 658 us, [12, 4096, 8192] 831 -> 774 us; with 1024 channels 16 steps lose as much).
-    const bool wide_rows_fwd = l->kind == 0 && esize == 4 && !rev && half > 1 && l->vec == half && !l->ragged && C >= 2048;
-    if (!u.unroll && wide_rows_fwd) l->steps = 16;
-    // Packed, 4 or more steps per instruction: 4 instructions per wave with one channel per lane; lanes of two
-    // channels keep 8 (bf16 [4096, 1024, 8] 41 / 41 -> 47 / 60 % of peak, [512, 4096, 24] 31 / 33 -> 37 / 44 %).
-    // (From one workgroup per CU on: fp32 [128, 8192, 16] 84 / 125 us with 4 steps, 67 / 94 us with 8.)
-    if (!u.unroll && l->group <= 16 && l->vec == 1 && rowgroups >= kComputeUnits) l->steps = 4;
-    const bool steps_ok = (l->vec == full) ? (l->steps == 2 || l->steps == 4 || l->steps == 8)
-                                           : (l->steps == 4 || l->steps == 8 || l->steps == 16);
-    if (!steps_ok) return SCANSCAM_EPLAN;
-
-    // LDS arrays of [waves][vec][64] values, kept within 64 KiB: 2 buffers x (A, B), or 7 for kind 2.
-    const int csize = compute_size(dtype);
-    const int planes = l->kind == 2 ? 7 : 4;
-    const int max_by_lds = (64 * 1024) / (planes * l->vec * kWave * csize);
-    const int max_by_threads = scanscam::cl_max_threads(l->vec, l->steps) / kWave;
-    int max_waves = scanscam::kMaxWaves;
-    if (max_waves > max_by_lds) max_waves = max_by_lds;
-    if (max_waves > max_by_threads) max_waves = max_by_threads;
-    if (u.waves) {
-        l->waves = u.waves;
-    } else {
-        const int64_t wave_steps = (int64_t)l->steps * (kWave / l->group);
-        const int64_t segments = (T + wave_steps - 1) / wave_steps;  // no more waves than segments of time
-        l->waves = segments < max_waves ? pow2_ceil(segments) : max_waves;
-        // Tiles over workgroups: 8 waves (shorter tiles, more of them to hand out), 16 when there are very
-        // few carry chains to spread the workgroups over.
-        if (l->kind != 0 && l->waves > 8 && rowgroups > 16) l->waves = 8;
-        // A workgroup walks all of T: 16-wave workgroups run one per CU, in rounds of 256. Where the last round
-        // would be mostly empty (320 workgroups = 1.25 rounds), 4-wave workgroups, several per CU, finish
-        // together instead: fp32 [80, 2048, 1024] 445 / 699 us -> 361 / 661 us, [64, 2048, 1032] 494 / 766 ->
-        // 413 / 734 us. (16-byte lanes only: narrow lanes need the waves to keep enough bytes in flight.)
-        // (Not element-aligned lanes with 16 steps per wave: fp32 [128, 1024, 601] backward 474 us with 4 waves, 395 us with 8.)
-        if (l->kind == 0 && l->group == kWave && l->vec * esize >= 8 && l->waves > 4 && rowgroups > kComputeUnits &&
-            !(l->ragged && l->steps == 16)) {
-            const int64_t rounds = (rowgroups + kComputeUnits - 1) / kComputeUnits;
-            if (rowgroups * 100 < rounds * kComputeUnits * 85) l->waves = 4;
-        }
-        // 16-bit storage, a workgroup per batch element or several: 4-wave workgroups for four-channel lanes that
-        // fill one wave per step and for pairs at 64 channels (above), and for the backward pass of single channels
-        // over two or more waves per step (C = 256: 374 -> 296 us, C = 320: 456 -> 353 us; forwards 16 waves are
-        // 5 to 10 % faster).
-        if (l->kind == 0 && esize == 2 && l->waves > 4 && !l->ragged) {
-            if (l->vec == half && l->group == kWave && groups(half) == 1) l->waves = 4;
-            if (l->vec == 2 && C == kWave && rowgroups >= 2 * kComputeUnits) l->waves = 4;  // ([256, 4096, 64] backward: 220 us with 4 waves, 154 us with 8)
-            if (l->vec == 1 && rev && groups(1) >= 2 && l->steps != 16 && pair_possible) l->waves = 4;
-            // Single channels with 16 steps: 8 waves from two workgroups per CU on ([4096, 256, 64] forward 90 us
-            // with 16 waves, 65 us with 8; [256, 4096, 64], one per CU, level).
-            if (l->vec == 1 && l->steps == 16 && rowgroups >= 2 * kComputeUnits && l->waves > 8) l->waves = 8;
-        }
-        // float64, single channels (8-byte lanes) walking all of T: 8 waves, as for the 8-byte lanes of fp32
-        // ([8, 4096, 2048] 282 / 484 us with 16 waves, 256-262 / 436-450 us with 4 or 8).
-        if (l->kind == 0 && esize == 8 && l->vec == 1 && l->group == kWave && l->waves > 8) l->waves = 8;
-        // fp32 with 2048 or more channels: the forward pass above in 4-wave workgroups from 4096 channels on
-        // ([24, 2048, 4096] 413 -> 391 us, [16, 2048, 8192] 554 -> 521 us), the backward pass in 16-byte lanes in
-        // 4-wave workgroups up to 512 time steps ([128, 512, 2048] 586 -> 478 us).
-        if (wide_rows_fwd && !u.unroll && C >= 4096 && l->waves > 4) l->waves = 4;
-        if (l->kind == 0 && esize == 4 && rev && l->vec == full && !l->ragged && C >= 2048 && T <= 512 && l->waves > 4)
-            l->waves = 4;
-        if (l->kind == 0 && small_fours && l->waves > 4) l->waves = 4;
-        if (l->kind == 0 && small_singles && l->waves > 8) l->waves = 8;
-        if (l->kind == 0 && esize == 4 && !rev && l->vec == 1 && l->steps == 16 && l->waves > 8) l->waves = 8;
-        while (l->waves > max_waves) l->waves >>= 1;
-        // Rows of one or two tiles: no more waves than make those tiles equally full (75 steps in tiles of 8 waves x 8 steps
-        // are one full tile and one of 11 steps; 5 waves make two tiles of 40 and 35).
-        if (l->kind == 0) {
-            const int64_t tile = l->waves * wave_steps, tiles_now = (T + tile - 1) / tile;
-            if (tiles_now <= 2) {
-                const int64_t even = (segments + tiles_now - 1) / tiles_now;
-                // (Lanes of 8 bytes or more: 4 waves, three tiles for such a row -- bf16 [506, 75, 943] 63 / 117 us with 8 waves,
-                // 55 / 106 us with 5, 50 / 86 us with 4; single channels do best with the even split: fp32 [4526, 65, 432]
-                // 405 / 714 -> 289 / 503 us with 5 and 9 waves, [1704, 67, 85] 49 / 81 -> 32 / 72 us.)
-                if (even < l->waves) l->waves = (l->vec * esize >= 8 && l->group == kWave && even > 4) ? 4 : (int)even;
-            }
-        }
-    }
-    if (l->waves < 1 || l->waves > max_waves) return SCANSCAM_EPLAN;
-
+    l->vec = c.vec;
+    l->steps = c.steps;
+    l->waves = c.waves;
+    l->kind = c.kind;
+    l->group = c.group;
+    l->ragged = c.ragged;
+    const int64_t rowgroups = batch * scanscam::cl_groups(C, c.vec);
     const int64_t tile_steps = (int64_t)l->waves * l->steps;
     const int64_t tiles = (T + tile_steps - 1) / tile_steps;
     const int64_t vals = (int64_t)l->vec * kWave * value_words(dtype);  // words of one [vec][64] array of values
-    l->lds_bytes = (size_t)planes * l->waves * l->vec * kWave * csize;
+    l->lds_bytes = (size_t)(l->kind == 2 ? 7 : 4) * l->waves * l->vec * kWave * compute_size(dtype);
     l->ws_bytes = 0;
     l->segments = 1;
     if (l->kind == 2) {
@@ -1144,7 +654,7 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
         l->ws_bytes = (size_t)(rowgroups * kCounterStride + rowgroups * tiles * pairs + rowgroups * supers * (pairs + vals)) *
                       sizeof(uint64_t);
     }
-    if (l->segments <= 1) {  // nothing to split after all
+    if (l->segments <= 1) {  // a forced time split of a single tile: nothing to split after all
         l->kind = 0;
         l->ws_bytes = 0;
     }
@@ -1452,6 +962,19 @@ int scanscam_resolve_plan_cl(int64_t batch, int64_t T, int64_t C, int dtype, int
     out->waves_per_row = 0;
     out->spin_limit = (plan && plan->spin_limit > 0) ? plan->spin_limit : scanscam::kSpinLimit;
     return SCANSCAM_OK;
+}
+
+int scanscam_predict_cl(int64_t batch, int64_t T, int64_t C, int dtype, int direction, const scanscam_plan *plan,
+                        double *microseconds)
+{
+    if (!microseconds) return SCANSCAM_EINVAL;
+    const int esize = elem_size(dtype);
+    if (esize == 0) return SCANSCAM_EDTYPE;
+    if (batch <= 0 || T <= 0 || C <= 0 || T >= kMaxT || C >= kMaxT) return SCANSCAM_EINVAL;
+    int align = 16;
+    while (align > esize && !(batch == 1 && T == 1) && (C * esize) % align != 0) align >>= 1;
+    scanscam::ClLaunch l;
+    return resolve_cl(plan, batch, T, C, dtype, align, direction == SCANSCAM_BACKWARD, &l, microseconds);
 }
 
 const char *scanscam_strerror(int code)

@@ -484,6 +484,44 @@ __global__ __launch_bounds__(MAXT) void scan_cl_kernel(const ClArgs p)
 // the wave. A workgroup owns one batch element.
 // LDS: two buffers (tiles alternate) of A and B, each [W][VEC][G] values.
 // ---------------------------------------------------------------------------
+// Inclusive scan of affine pairs over the lanes that hold one channel vector: lanes cl, cl + G, cl + 2G, ... of a
+// wave (G a power of two below 64; ascending lane = later in scan order). DPP moves inside each row of 16 lanes
+// at distances G ... 8 (lanes without a source in their row receive the identity), then two shuffles across
+// rows: rows 1 and 3 take the total of the row before (held by its last lanes of the same channel vector), then
+// rows 2 and 3 the total of rows 0-1.
+template <typename CT>
+__device__ __forceinline__ void packed_lane_scan(CT &A, CT &B, int G, int cl, int lane)
+{
+#define SCANSCAM_ROW_STEP(OFF)                                  \
+    if (G <= (OFF)) {                                           \
+        const CT A1 = dpp_move<0x110 + (OFF), 0xf>(CT(1), A);   \
+        const CT B1 = dpp_move<0x110 + (OFF), 0xf>(CT(0), B);   \
+        B = fma_(A, B1, B);                                     \
+        A = A * A1;                                             \
+    }
+    SCANSCAM_ROW_STEP(1)
+    SCANSCAM_ROW_STEP(2)
+    SCANSCAM_ROW_STEP(4)
+    SCANSCAM_ROW_STEP(8)
+#undef SCANSCAM_ROW_STEP
+    if (G <= 16) {
+        const int src = ((lane & ~15) - G + cl) & (kWave - 1);  // rows 0 and 2 discard what they read
+        const CT A1 = __shfl(A, src, kWave), B1 = __shfl(B, src, kWave);
+        if (lane & 16) {
+            B = fma_(A, B1, B);
+            A = A * A1;
+        }
+    }
+    {
+        const int src = 32 - G + cl;
+        const CT A1 = __shfl(A, src, kWave), B1 = __shfl(B, src, kWave);
+        if (lane & 32) {
+            B = fma_(A, B1, B);
+            A = A * A1;
+        }
+    }
+}
+
 template <typename ST, int VEC, int S, bool REV, int MAXT>
 __global__ __launch_bounds__(MAXT) void scan_cl_packed_kernel(const ClArgs p)
 {
@@ -557,38 +595,7 @@ __global__ __launch_bounds__(MAXT) void scan_cl_packed_kernel(const ClArgs p)
                         }
                     }
                 } else {
-                    // Inside each row of 16 lanes: DPP moves at distances G, 2G, ... 8 (lanes without a
-                    // source in their row receive the identity).
-#define SCANSCAM_ROW_STEP(OFF)                                  \
-    if (G <= (OFF)) {                                           \
-        const CT A1 = dpp_move<0x110 + (OFF), 0xf>(CT(1), A);   \
-        const CT B1 = dpp_move<0x110 + (OFF), 0xf>(CT(0), B);   \
-        B = fma_(A, B1, B);                                     \
-        A = A * A1;                                             \
-    }
-                    SCANSCAM_ROW_STEP(1)
-                    SCANSCAM_ROW_STEP(2)
-                    SCANSCAM_ROW_STEP(4)
-                    SCANSCAM_ROW_STEP(8)
-#undef SCANSCAM_ROW_STEP
-                    // Across rows: rows 1 and 3 take the total of the row before (held by its last lanes of
-                    // the same channel vector), then rows 2 and 3 the total of rows 0-1.
-                    if (G <= 16) {
-                        const int src = ((lane & ~15) - G + cl) & (kWave - 1);  // rows 0 and 2 discard what they read
-                        const CT A1 = __shfl(A, src, kWave), B1 = __shfl(B, src, kWave);
-                        if (lane & 16) {
-                            B = fma_(A, B1, B);
-                            A = A * A1;
-                        }
-                    }
-                    {
-                        const int src = 32 - G + cl;
-                        const CT A1 = __shfl(A, src, kWave), B1 = __shfl(B, src, kWave);
-                        if (lane & 32) {
-                            B = fma_(A, B1, B);
-                            A = A * A1;
-                        }
-                    }
+                    packed_lane_scan<CT>(A, B, G, cl, lane);
                 }
                 const CT TA = __shfl(A, kWave - G + cl, kWave), TB = __shfl(B, kWave - G + cl, kWave);
                 PB[s][k] = fma_(A, RB[k], B);

@@ -109,6 +109,8 @@ def _bind(path: str) -> ctypes.CDLL:
     lib.scanscam_resolve_plan.restype = i32
     lib.scanscam_resolve_plan_cl.argtypes = [i64, i64, i64, i32, i32, plan_p, plan_p]
     lib.scanscam_resolve_plan_cl.restype = i32
+    lib.scanscam_predict_cl.argtypes = [i64, i64, i64, i32, i32, plan_p, ctypes.POINTER(ctypes.c_double)]
+    lib.scanscam_predict_cl.restype = i32
     lib.scanscam_strerror.argtypes = [i32]
     lib.scanscam_strerror.restype = ctypes.c_char_p
     lib.scanscam_abi_version.argtypes = []
@@ -471,6 +473,20 @@ def resolve_plan_cl(batch: int, T: int, C: int, dtype: torch.dtype, direction: i
     if rc != 0:
         raise RuntimeError(f"scanscam_resolve_plan_cl: {strerror(rc)}")
     return out
+
+
+def predict_cl(batch: int, T: int, C: int, dtype: torch.dtype, direction: int = FORWARD,
+               plan: Optional[Plan] = None) -> float:
+    """Microseconds the library's cost model estimates for this channels-last call and plan (no GPU needed)."""
+    us = ctypes.c_double()
+    rc = lib().scanscam_predict_cl(batch, T, C, _dtype_code(dtype), direction, _plan_ref_plain(plan), ctypes.byref(us))
+    if rc != 0:
+        raise RuntimeError(f"scanscam_predict_cl: {strerror(rc)}")
+    return float(us.value)
+
+
+def _plan_ref_plain(plan: Optional[Plan]):
+    return ctypes.byref(plan) if plan is not None else None
 
 
 def _workspace_cl(L, batch: int, T: int, C: int, dtype: torch.dtype, direction: int, plan: Optional[Plan],

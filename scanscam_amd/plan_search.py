@@ -99,6 +99,25 @@ def cl_plans(dtype, C):
     return out
 
 
+def cl_plans_all(dtype, C):
+    """Every launch plan of the channels-last kernels worth timing on a shape: each lane width (whole or
+    element-aligned), a walk of all of T or tiles over time, every number of steps per wave, 2 to 16 waves.
+    The set that --dump records, from which the constants of the library's cost model are fitted."""
+    esize = torch.empty(0, dtype=dtype).element_size()
+    full = 16 // esize
+    widths = sorted({1, full, max(1, full // 2)} | ({2} if esize == 2 else set()))
+    out = []
+    for v in widths:
+        if C % v != 0 and C <= 32 * v:
+            continue  # element-aligned lanes need more than half a wave of them per time step
+        for s in ((2, 4, 8) if v == full else (4, 8, 16)):
+            for w in (2, 4, 8, 16):
+                out.append(P(vec=v, unroll=s, waves=w, mode=hip.MODE_ROW))
+                if C % v == 0:
+                    out.append(P(vec=v, unroll=s, waves=w, mode=hip.MODE_LOOKBACK))
+    return out
+
+
 def random_cl_shapes(n, seed):
     """n shapes [batch, T, C]: C from 8 to 5000 and T from 64 to 16384, both log-uniform, half of the channel counts
     rounded to multiples of 8; 8 M to 190 M elements; batch what that leaves, 1 to 8192."""
@@ -150,8 +169,10 @@ def _short(plan):
     return s + (f" r{plan.waves_per_row}" if plan.waves_per_row else "")
 
 
-def search(layout, shape, dtype, reps=24, warm=4, out=sys.stdout, every=False):
-    """Time every plan of the set on ``shape``; returns {direction: (auto_us, best_us, best_plan)}."""
+def search(layout, shape, dtype, reps=24, warm=4, out=sys.stdout, every=False, dump=None):
+    """Time every plan of the set on ``shape``; returns {direction: (auto_us, best_us, best_plan)}.
+    With ``dump`` (an open text file) the set is every plan of ``cl_plans_all`` and each timing is written there as
+    one line ``batch T C dtype direction mode vec unroll waves microseconds`` (mode 0 = the automatic plan)."""
     dev = torch.device("cuda:0")
     esize = torch.empty(0, dtype=dtype).element_size()
     n = 1
@@ -168,6 +189,8 @@ def search(layout, shape, dtype, reps=24, warm=4, out=sys.stdout, every=False):
         plans, fwd, bwd = row_plans(dtype, shape[-1]), hip.prepare_forward, hip.prepare_backward
     else:
         plans, fwd, bwd = cl_plans(dtype, shape[-1]), hip.prepare_forward_cl, hip.prepare_backward_cl
+        if dump is not None:
+            plans = cl_plans_all(dtype, shape[-1])
     times = {"fwd": [], "bwd": []}
     for plan in [None] + plans + [None]:
         try:
@@ -179,6 +202,11 @@ def search(layout, shape, dtype, reps=24, warm=4, out=sys.stdout, every=False):
             continue
         times["fwd"].append((_time(f, reps, warm), plan))
         times["bwd"].append((_time(r, reps, warm), plan))
+        if dump is not None:
+            for name in ("fwd", "bwd"):
+                q = plan if plan is not None else P()
+                print(*shape, str(dtype).replace("torch.", ""), name, q.mode, q.vec, q.unroll, q.waves,
+                      f"{times[name][-1][0]:.2f}", file=dump, flush=True)
     res, text = {}, []
     if layout == "rows":
         chosen = [hip.resolve_plan(*shape, dtype, d) for d in (hip.FORWARD, hip.BACKWARD)]
@@ -209,6 +237,8 @@ def main(argv=None):
     ap.add_argument("--seed", type=int, default=0, help="seed of --random")
     ap.add_argument("--reps", type=int, default=24)
     ap.add_argument("--every", action="store_true", help="also print every plan's timings")
+    ap.add_argument("--dump", metavar="FILE", help="channels-last: time every plan of the full set and append each "
+                    "timing to FILE (the data the cost model's constants are fitted to)")
     args = ap.parse_intermixed_args(argv)  # options may stand between the layout and the shapes
     if not hip.has_hip_ops:
         sys.exit("plan_search: libscanscam_hip.so does not load")
@@ -231,8 +261,9 @@ def main(argv=None):
             ap.error(f"{spec}: a {args.layout} shape has {2 if args.layout == 'rows' else 3} sizes")
         jobs.append((args.layout, shape, DTYPES[dtype_s]))
     ratios = []
+    dump = open(args.dump, "a") if args.dump else None
     for layout, shape, dtype in jobs:
-        res = search(layout, shape, dtype, reps=args.reps, every=args.every)
+        res = search(layout, shape, dtype, reps=args.reps, every=args.every, dump=dump if layout == "cl" else None)
         ratios += [auto / best for auto, best, _ in res.values()]
     behind = sum(r > 1.08 for r in ratios)
     print(f"{2 * len(jobs)} timings, automatic plan more than 8 % behind the set's best in {behind}", flush=True)
