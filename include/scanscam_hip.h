@@ -114,8 +114,8 @@ int scanscam_scan_bwd(const void *a, const void *h, const void *gh, void *ga, vo
  * look-back descriptors live in a fixed array of SCANSCAM_NOALLOC_SCRATCH_BYTES in the GPU's memory
  * that belongs to the library (one per GPU it runs on, held until the process ends), found once per
  * device on the first call there. The call itself allocates and frees nothing, on the device or
- * through any library. A shape whose descriptors do not fit (more than about 65 000 look-back tiles,
- * i.e. 0.5 G fp32 elements in long rows) is refused with SCANSCAM_ESCRATCH and nothing is launched.
+ * through any library. A shape whose descriptors do not fit (more than about 120 000 look-back tiles
+ * of fp32 arithmetic, i.e. 1 G elements in long rows) is refused with SCANSCAM_ESCRATCH and nothing is launched.
  * Every call clears the part of the array it uses, with a kernel on `stream`. All calls on one GPU
  * share that GPU's array: calls that may overlap in time on one GPU (two streams, two threads) race
  * and must use scanscam_scan_fwd with separate workspaces instead.

@@ -319,11 +319,12 @@ struct ClSteps {
             const Elems<ST, VEC> e = __builtin_bit_cast(Elems<ST, VEC>, r);
 #pragma unroll
             for (int k = 0; k < VEC; k++)
-                if (k < VEC - ln.shift)
+                if (k < VEC - ln.shift) {
                     if constexpr (sizeof(raw_t) <= 8)
                         One::store_cached_elem_aligned(__builtin_bit_cast(typename One::raw_t, e.e[k]), res, ln.c + (unsigned)((ln.shift + k) * sizeof(ST)), off);
                     else
                         One::store(__builtin_bit_cast(typename One::raw_t, e.e[k]), res, ln.c + (unsigned)((ln.shift + k) * sizeof(ST)), off);
+                }
         }
     }
 

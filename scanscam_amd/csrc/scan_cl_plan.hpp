@@ -10,7 +10,7 @@
 // The terms (microseconds):
 //   stream   algorithmic bytes / (rate of this kernel variant) x (lines touched / lines used) / fill^alpha
 //            `rate`: one measured streaming rate per kernel variant (kernel, lane bytes, storage size,
-//            direction), the table of scan_cl_model.inc; `lines touched`: every wave access that starts or ends
+//            direction, and whether a time step is whole 128-byte lines), the table of scan_cl_model.inc; `lines touched`: every wave access that starts or ends
 //            inside a 128-byte line moves the rest of that line as well; `fill`: the part of the lanes
 //            of a time step's waves that hold a channel.
 //   latency  rounds of workgroups x tiles per workgroup x time of one tile, where a tile takes the memory
@@ -20,8 +20,8 @@
 //            registers the kernels were compiled to) cover each other's latency but share its SIMDs.
 //   chain    time-split tiles per (batch element, channel group) / waves: the super-tile chain of a
 //            row-group advances one memory round trip at a time.
-// They are combined as (stream^3 + latency^3 + chain^3)^(1/3) plus the launch itself (and the launch that
-// prepares the workspace of a time split).
+// The estimate is their sum plus the launch itself (and the launch that prepares the workspace of a time split).
+// (Combined as a p-norm with p = 1.5 to 4, the fitted model chose worse plans on shapes it had not seen.)
 //
 // The constants are fitted, not hand-set: `python -m scanscam_amd.plan_search --dump FILE` times every
 // candidate on a set of shapes and `python -m scanscam_amd.plan_fit FILE...` fits them to those timings and
@@ -52,7 +52,8 @@ inline int cl_max_waves(int vec, int steps, int kind, int csize)
 struct ClModel {
     // Streaming rate in bytes per microsecond / 1e6 (= TB/s of algorithmic bytes at full lanes):
     // [kernel: 0 walk, 1 several steps per wave, 2 time split][storage: 2, 4, 8 bytes][lane: 2, 4, 8, 16 bytes][direction]
-    double rate[3][3][4][2];
+    // [a time step is a whole number of 128-byte lines]
+    double rate[3][3][4][2][2];
     double latency;      // memory latency of a tile's loads
     double latency_w8;   // ... more per 8 waves of the workgroup (the barrier waits for the slowest wave)
     double issue;        // issue time of one wave's instructions per element per lane (fp32, forward)
@@ -64,6 +65,7 @@ struct ClModel {
     double carry;        // ticket and carry wait of a time-split tile
     double fill_alpha;   // exponent of 1 / fill in the streaming term
     double chain;        // one hop of a row-group's super-tile chain
+    double issue_shared; // additional issue time per doubling of the time steps that share a wave (the lane scan per load)
     double line[4];      // weight of the lines touched beyond the bytes used, for lanes of 2, 4, 8, 16 bytes
 };
 
@@ -124,8 +126,8 @@ inline double cl_registers(const ClShape &s, const ClCandidate &c)
 {
     double per = s.esize == 2 ? (s.rev ? 3.8 : 2.8) : (s.rev ? 3.0 : 2.1), base = c.kind == 2 ? 34.0 : 24.0;
     if (c.group < kWave) {  // several time steps per wave
-        base = 35.0;
-        per = s.rev ? 5.0 : 4.0;
+        base = s.rev ? 36.0 : 32.0;
+        per = s.rev ? 5.7 : 4.6;
     }
     return base + c.steps * c.vec * per * (s.esize == 8 ? 2.0 : 1.0);
 }
@@ -141,9 +143,11 @@ inline double cl_predict_us(const ClShape &s, const ClCandidate &c, const ClMode
     const int64_t tiles = (s.T + tile_steps - 1) / tile_steps;
     const double bytes = (double)s.batch * (double)s.T * (double)s.C * s.esize * (s.rev ? 5.0 : 3.0);
 
+    // More than the launch bounds leave a lane (512 threads: 256 registers, 1024: 128) is spilled.
     double regs = cl_registers(s, c);
-    const bool spills = regs >= 256.0;
-    if (spills) regs = 256.0;
+    const double cap = cl_max_threads(c.vec, c.steps) == 512 ? 256.0 : 128.0;
+    const bool spills = regs > cap;
+    if (spills) regs = cap;
     int occupancy = (int)(512.0 / regs);
     occupancy = occupancy < 1 ? 1 : (occupancy > 8 ? 8 : occupancy);
     const int resident_max = (4 * occupancy) / c.waves < 1 ? 1 : (4 * occupancy) / c.waves;
@@ -151,7 +155,7 @@ inline double cl_predict_us(const ClShape &s, const ClCandidate &c, const ClMode
     double busy = m.issue * c.steps * c.vec * (c.waves > 4 ? c.waves / 4.0 : 1.0) * (s.rev ? m.issue_bwd : 1.0) *
                   (s.esize == 2 ? m.issue_16 : 1.0);
     if (spills) busy *= 2.0;
-    if (c.group < kWave) busy *= 1.0 + 0.25 * std::log2((double)sub);
+    if (c.group < kWave) busy *= 1.0 + m.issue_shared * std::log2((double)sub);
     if (c.ragged) busy *= 1.0 + m.issue_ragged;
     const double tile_us = m.latency + m.latency_w8 * c.waves / 8.0 + busy + (c.kind == 2 ? m.carry : 0.0);
     const int64_t workgroups = c.kind == 2 ? RG * tiles : RG;
@@ -164,8 +168,8 @@ inline double cl_predict_us(const ClShape &s, const ClCandidate &c, const ClMode
     const int kernel = c.group < kWave ? 1 : c.kind;
     const int es = s.esize == 2 ? 0 : (s.esize == 4 ? 1 : 2);
     const int ln = lane <= 2 ? 0 : (lane == 4 ? 1 : (lane == 8 ? 2 : 3));
-    const double rate = m.rate[kernel][es][ln][s.rev ? 1 : 0] * 1e6;
     const int64_t step_bytes = s.C * s.esize;
+    const double rate = m.rate[kernel][es][ln][s.rev ? 1 : 0][step_bytes % 128 == 0 ? 1 : 0] * 1e6;
     auto gcd = [](int64_t a, int64_t b) {
         while (b) {
             const int64_t t = a % b;
@@ -184,8 +188,7 @@ inline double cl_predict_us(const ClShape &s, const ClCandidate &c, const ClMode
     }
     const double stream_us = bytes / std::pow(fill, m.fill_alpha) / rate * lines;
     const double chain_us = c.kind == 2 ? m.chain * (double)tiles / c.waves : 0.0;
-    const double sum = stream_us * stream_us * stream_us + latency_us * latency_us * latency_us + chain_us * chain_us * chain_us;
-    return m.launch + (c.kind == 2 ? m.launch_split : 0.0) + std::cbrt(sum);
+    return m.launch + (c.kind == 2 ? m.launch_split : 0.0) + stream_us + latency_us + chain_us;
 }
 
 // The candidate with the smallest estimate among those that agree with the caller's plan `u` (zero fields are
@@ -205,8 +208,12 @@ inline bool cl_choose(const ClShape &s, const scanscam_plan &u, ClCandidate *bes
     }
     const int all_steps[4] = {2, 4, 8, 16};
     const int all_waves[2] = {4, 8};
-    bool found = false;
-    double least = 0.0;
+    // A walk keeps one workgroup per batch and channel group: with fewer of them than half the compute units it
+    // leaves most of the chip idle however well it streams, so it stands back ("thin") whenever the time can be
+    // split instead. Among 328 timed shapes of that kind a walk was the fastest plan once.
+    bool found = false, found_thin = false;
+    double least = 0.0, least_thin = 0.0;
+    ClCandidate thin{};
     for (int iv = 0; iv < nv; iv++) {
         for (int kind = 0; kind <= 2; kind += 2) {
             if ((kind == 2 && u.mode == kModeRow) || (kind == 0 && u.mode == kModeLookback)) continue;
@@ -232,6 +239,14 @@ inline bool cl_choose(const ClShape &s, const scanscam_plan &u, ClCandidate *bes
                     const int64_t tile_steps = (int64_t)c.waves * c.steps * (kWave / c.group);
                     if (kind == 2 && u.mode != kModeLookback && s.T <= tile_steps) continue;  // one tile: nothing to split
                     const double us = cl_predict_us(s, c);
+                    if (kind == 0 && u.mode == 0 && 2 * s.batch * cl_groups(s.C, c.vec) < kClComputeUnits) {
+                        if (!found_thin || us < least_thin) {
+                            found_thin = true;
+                            least_thin = us;
+                            thin = c;
+                        }
+                        continue;
+                    }
                     if (!found || us < least) {
                         found = true;
                         least = us;
@@ -240,6 +255,11 @@ inline bool cl_choose(const ClShape &s, const scanscam_plan &u, ClCandidate *bes
                 }
             }
         }
+    }
+    if (!found && found_thin) {
+        found = true;
+        least = least_thin;
+        *best = thin;
     }
     if (found && best_us) *best_us = least;
     return found;

@@ -26,16 +26,16 @@ import numpy as np
 ESIZE = {"float32": 4, "bfloat16": 2, "float16": 2, "float64": 8}
 KERNELS, STORAGE, LANES = (0, 1, 2), (2, 4, 8), (2, 4, 8, 16)
 SCALARS = ["latency", "latency_w8", "issue", "issue_bwd", "issue_16", "issue_ragged", "launch", "launch_split", "carry",
-           "fill_alpha", "chain", "line_2", "line_4", "line_8", "line_16"]
-START = [1.0, 0.5, 0.04, 1.4, 0.6, 0.6, 3.0, 0.5, 6.0, 0.2, 1.0, 0.5, 0.5, 0.5, 0.5]
-LOWER = [0.2, 0.0, 0.001, 0.8, 0.3, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0]
-UPPER = [10.0, 5.0, 0.3, 4.0, 4.0, 3.0, 15.0, 20.0, 20.0, 1.0, 10.0, 5.0, 5.0, 5.0, 5.0]
-N_RATE = len(KERNELS) * len(STORAGE) * len(LANES) * 2
+           "fill_alpha", "chain", "issue_shared", "line_2", "line_4", "line_8", "line_16"]
+START = [1.0, 0.5, 0.04, 1.4, 0.6, 0.6, 3.0, 0.5, 6.0, 0.2, 1.0, 0.5, 0.5, 0.5, 0.5, 0.5]
+LOWER = [0.2, 0.0, 0.001, 0.8, 0.3, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0]
+UPPER = [10.0, 5.0, 0.3, 4.0, 4.0, 3.0, 15.0, 20.0, 20.0, 1.0, 10.0, 10.0, 5.0, 5.0, 5.0, 5.0]
+N_RATE = len(KERNELS) * len(STORAGE) * len(LANES) * 2 * 2
 WAVE, CUS = 64, 256
 
 
-def rate_index(kernel, esize, lane, rev):
-    return ((kernel * len(STORAGE) + STORAGE.index(esize)) * len(LANES) + LANES.index(max(lane, 2))) * 2 + int(rev)
+def rate_index(kernel, esize, lane, rev, whole=False):
+    return (((kernel * len(STORAGE) + STORAGE.index(esize)) * len(LANES) + LANES.index(max(lane, 2))) * 2 + int(rev)) * 2 + int(whole)
 
 
 def pow2_ceil(v):
@@ -66,7 +66,7 @@ def registers(d):
     per = (3.8 if d["rev"] else 2.8) if d["esize"] == 2 else (3.0 if d["rev"] else 2.1)
     base = 34.0 if d["kind"] == 2 else 24.0
     if d["group"] < WAVE:
-        base, per = 35.0, (5.0 if d["rev"] else 4.0)
+        base, per = (36.0, 5.7) if d["rev"] else (32.0, 4.6)
     return base + d["steps"] * d["vec"] * per * (2.0 if d["esize"] == 8 else 1.0)
 
 
@@ -74,8 +74,9 @@ def predict(d, p):
     """cl_predict_us() of scan_cl_plan.hpp, term for term."""
     q = dict(zip(SCALARS, p[N_RATE:]))
     regs = registers(d)
-    spills = regs >= 256.0
-    regs = min(regs, 256.0)
+    cap = 256.0 if d["vec"] > 1 and d["steps"] >= 8 else 128.0  # the kernels' launch bounds: 512 or 1024 threads
+    spills = regs > cap
+    regs = min(regs, cap)
     occupancy = max(1, min(8, int(512.0 / regs)))
     resident_max = max(1, (4 * occupancy) // d["waves"])
     busy = (q["issue"] * d["steps"] * d["vec"] * (d["waves"] / 4.0 if d["waves"] > 4 else 1.0) *
@@ -83,16 +84,16 @@ def predict(d, p):
     if spills:
         busy *= 2.0
     if d["group"] < WAVE:
-        busy *= 1.0 + 0.25 * math.log2(d["sub"])
+        busy *= 1.0 + q["issue_shared"] * math.log2(d["sub"])
     if d["ragged"]:
         busy *= 1.0 + q["issue_ragged"]
-    tile_us = q["latency"] + q["latency_w8"] * d["waves"] / 8.0 + busy + (q["carry"] if d["kind"] == 2 else 0.0)
     workgroups = d["RG"] * d["tiles"] if d["kind"] == 2 else d["RG"]
     resident = min(math.ceil(workgroups / CUS), resident_max)
+    tile_us = q["latency"] + q["latency_w8"] * d["waves"] / 8.0 + busy + (q["carry"] if d["kind"] == 2 else 0.0)
     rounds = math.ceil(workgroups / (CUS * resident_max))
     latency_us = rounds * (1 if d["kind"] == 2 else d["tiles"]) * max(tile_us, resident * busy)
     kernel = 1 if d["group"] < WAVE else d["kind"]
-    rate = p[rate_index(kernel, d["esize"], d["lane"], d["rev"])] * 1e6
+    rate = p[rate_index(kernel, d["esize"], d["lane"], d["rev"], (d["C"] * d["esize"]) % 128 == 0)] * 1e6
     step_bytes = d["C"] * d["esize"]
     line = q["line_%d" % max(2, d["lane"])]
     if d["group"] < WAVE:
@@ -103,7 +104,7 @@ def predict(d, p):
         lines = 1.0 + line * d["G"] * (128 - a) / step_bytes
     stream_us = d["bytes"] / d["fill"] ** q["fill_alpha"] / rate * lines
     chain_us = q["chain"] * d["tiles"] / d["waves"] if d["kind"] == 2 else 0.0
-    return q["launch"] + (q["launch_split"] if d["kind"] == 2 else 0.0) + (stream_us ** 3 + latency_us ** 3 + chain_us ** 3) ** (1 / 3)
+    return q["launch"] + (q["launch_split"] if d["kind"] == 2 else 0.0) + stream_us + latency_us + chain_us
 
 
 FIELDS = ("steps", "vec", "waves", "rev", "esize", "group", "sub", "ragged", "kind", "RG", "tiles", "lane", "C", "G", "fill",
@@ -114,7 +115,9 @@ def columns(ds):
     """The descriptions of many (shape, plan) pairs as arrays, for predict_many()."""
     cols = {k: np.array([float(d[k]) for d in ds]) for k in FIELDS}
     cols["regs"] = np.array([registers(d) for d in ds])
-    cols["rate_index"] = np.array([rate_index(1 if d["group"] < WAVE else d["kind"], d["esize"], d["lane"], d["rev"]) for d in ds])
+    cols["cap"] = np.array([256.0 if d["vec"] > 1 and d["steps"] >= 8 else 128.0 for d in ds])
+    cols["rate_index"] = np.array([rate_index(1 if d["group"] < WAVE else d["kind"], d["esize"], d["lane"], d["rev"],
+                                              (d["C"] * d["esize"]) % 128 == 0) for d in ds])
     step_bytes = [d["C"] * d["esize"] for d in ds]
     cols["lines_extra"] = np.array([
         (128 - math.gcd(d["sub"] * sb, 128)) / (d["sub"] * sb) if d["group"] < WAVE
@@ -125,18 +128,18 @@ def columns(ds):
 def predict_many(c, p):
     """predict() over the arrays of columns(): the same arithmetic, vectorised (the fit calls it millions of times)."""
     q = dict(zip(SCALARS, p[N_RATE:]))
-    spills = c["regs"] >= 256.0
-    regs = np.minimum(c["regs"], 256.0)
+    spills = c["regs"] > c["cap"]
+    regs = np.minimum(c["regs"], c["cap"])
     occupancy = np.clip(np.floor(512.0 / regs), 1, 8)
     resident_max = np.maximum(1, np.floor(4 * occupancy / c["waves"]))
     packed, split, rev = c["group"] < WAVE, c["kind"] == 2, c["rev"] > 0
     busy = (q["issue"] * c["steps"] * c["vec"] * np.where(c["waves"] > 4, c["waves"] / 4.0, 1.0) *
             np.where(rev, q["issue_bwd"], 1.0) * np.where(c["esize"] == 2, q["issue_16"], 1.0))
-    busy = busy * np.where(spills, 2.0, 1.0) * np.where(packed, 1.0 + 0.25 * np.log2(c["sub"]), 1.0)
+    busy = busy * np.where(spills, 2.0, 1.0) * np.where(packed, 1.0 + q["issue_shared"] * np.log2(c["sub"]), 1.0)
     busy = busy * np.where(c["ragged"] > 0, 1.0 + q["issue_ragged"], 1.0)
-    tile_us = q["latency"] + q["latency_w8"] * c["waves"] / 8.0 + busy + np.where(split, q["carry"], 0.0)
     workgroups = np.where(split, c["RG"] * c["tiles"], c["RG"])
     resident = np.minimum(np.ceil(workgroups / CUS), resident_max)
+    tile_us = q["latency"] + q["latency_w8"] * c["waves"] / 8.0 + busy + np.where(split, q["carry"], 0.0)
     rounds = np.ceil(workgroups / (CUS * resident_max))
     latency_us = rounds * np.where(split, 1.0, c["tiles"]) * np.maximum(tile_us, resident * busy)
     rate = p[c["rate_index"]] * 1e6
@@ -144,7 +147,7 @@ def predict_many(c, p):
     lines = 1.0 + line * c["lines_extra"]
     stream_us = c["bytes"] / c["fill"] ** q["fill_alpha"] / rate * lines
     chain_us = np.where(split, q["chain"] * c["tiles"] / c["waves"], 0.0)
-    return q["launch"] + np.where(split, q["launch_split"], 0.0) + np.cbrt(stream_us ** 3 + latency_us ** 3 + chain_us ** 3)
+    return q["launch"] + np.where(split, q["launch_split"], 0.0) + stream_us + latency_us + chain_us
 
 
 def load(paths):
@@ -172,6 +175,9 @@ def regret(by, p, out, label):
     for key, timings in by.items():
         plans = [(d, us) for d, us in timings if d is not None]
         cands = [(d, us) for d, us in plans if candidate(d)]
+        # cl_choose passes over a walk with fewer workgroups than half the compute units when the time can be split
+        wide = [(d, us) for d, us in cands if not (d["kind"] == 0 and 2 * d["RG"] < CUS)]
+        cands = wide or cands
         if not cands:
             continue
         best = min(us for _, us in plans)
@@ -229,28 +235,33 @@ def emit(p, seen, note, out):
     print("// Constants of the channels-last cost model (ClModel, scan_cl_plan.hpp). Printed by", file=out)
     print(f"//   python -m scanscam_amd.plan_fit {note}", file=out)
     print("// from timings written by `python -m scanscam_amd.plan_search --dump` on one MI355X; do not edit by hand.", file=out)
-    print("// rate[kernel][storage][lane][direction]; a variant that no timing exercised (marked *) holds its neighbours' mean.", file=out)
+    print("// rate[kernel][storage][lane][direction][time steps are whole 128-byte lines]; a variant that no timing exercised", file=out)
+    print("// (marked *) holds the mean of the exercised ones of its kernel and storage size.", file=out)
     print("const ClModel kClModel = {", file=out)
     print("    {", file=out)
+    per = len(LANES) * 4
     for k in KERNELS:
         print("        {", file=out)
         for e in STORAGE:
             cells = []
             for lane in LANES:
-                vals = []
+                pairs = []
                 for rev in (0, 1):
-                    i = rate_index(k, e, lane, rev)
-                    v = p[i]
-                    if i not in seen:
-                        same = [p[j] for j in seen if j // (len(LANES) * 2) == i // (len(LANES) * 2)] or [p[j] for j in seen]
-                        v = float(np.mean(same))
-                    vals.append(f"{v:.3f}" + ("" if i in seen else " /* * */"))
-                cells.append("{" + ", ".join(vals) + "}")
-            print(f"            {{{', '.join(cells)}}},  // kernel {k}, {e}-byte storage: lanes of 2, 4, 8, 16 bytes x (forward, backward)", file=out)
+                    vals = []
+                    for whole in (0, 1):
+                        i = rate_index(k, e, lane, rev, whole)
+                        v = p[i]
+                        if i not in seen:
+                            same = [p[j] for j in seen if j // per == i // per] or [p[j] for j in seen]
+                            v = float(np.mean(same))
+                        vals.append(f"{v:.3f}" + ("" if i in seen else " /* * */"))
+                    pairs.append("{" + ", ".join(vals) + "}")
+                cells.append("{" + ", ".join(pairs) + "}")
+            print(f"            {{{', '.join(cells)}}},  // kernel {k}, {e}-byte storage: lanes of 2, 4, 8, 16 bytes x (forward, backward) x (part lines, whole lines)", file=out)
         print("        },", file=out)
     print("    },", file=out)
     q = dict(zip(SCALARS, p[N_RATE:]))
-    for name in SCALARS[:11]:
+    for name in SCALARS[:12]:
         print(f"    {q[name]:.4f},  // {name}", file=out)
     print("    {" + ", ".join(f"{q['line_%d' % b]:.4f}" for b in LANES) + "},  // line: lanes of 2, 4, 8, 16 bytes", file=out)
     print("};", file=out)
