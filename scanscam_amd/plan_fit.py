@@ -194,8 +194,8 @@ def regret(by, p, out, label):
 def fit(by, evaluations=200):
     from scipy.optimize import least_squares
 
-    rows, weights = [], []
-    for key, timings in by.items():
+    rows, weights, case = [], [], []
+    for number, (key, timings) in enumerate(by.items()):
         plans = [(d, us) for d, us in timings if d is not None and d["waves"] in (4, 8, 16)]
         if not plans:
             continue
@@ -204,8 +204,11 @@ def fit(by, evaluations=200):
             if us < 2.5 * best:
                 rows.append((d, math.log(us)))
                 weights.append(1.0 / (1.0 + 3.0 * math.log(us / best)))
+                case.append(number)
     weights = np.array(weights)
     target = np.array([y for _, y in rows])
+    case = np.array(case)
+    case_weight = np.maximum(np.bincount(case, weights=weights), 1e-9)
     cols = columns([d for d, _ in rows])
     # Only the rates that some timing exercises are free; the others stay at the start value (emit() says so).
     seen = sorted(set(int(i) for i in cols["rate_index"]))
@@ -219,8 +222,13 @@ def fit(by, evaluations=200):
         p[free] = x
         return p
 
+    # What the choice needs is the order of one shape's plans, not the level of its durations: 0.7 of a case's
+    # (weighted) mean error is taken out of each of its residuals, so an error common to all plans of a shape
+    # counts for little and the constants go where they tell plans apart.
     def residual(x):
-        return (np.log(np.maximum(predict_many(cols, expand(x)), 1e-3)) - target) * weights
+        r = np.log(np.maximum(predict_many(cols, expand(x)), 1e-3)) - target
+        common = np.bincount(case, weights=weights * r) / case_weight
+        return (r - 0.7 * common[case]) * weights
 
     sol = least_squares(residual, full0[free], bounds=(lo, hi), loss="soft_l1", f_scale=0.1, max_nfev=evaluations)
     p = expand(sol.x)
