@@ -207,7 +207,7 @@ inline bool cl_choose(const ClShape &s, const scanscam_plan &u, ClCandidate *bes
         if (full > 1) vecs[nv++] = full;
     }
     const int all_steps[4] = {2, 4, 8, 16};
-    const int all_waves[2] = {4, 8};
+    const int all_waves[3] = {4, 8, 16};  // 16 only for a walk: tiles of 16 waves measured behind 8 throughout
     // A walk keeps one workgroup per batch and channel group: with fewer of them than half the compute units it
     // leaves most of the chip idle however well it streams, so it stands back ("thin") whenever the time can be
     // split instead. Among 328 timed shapes of that kind a walk was the fastest plan once.
@@ -222,7 +222,7 @@ inline bool cl_choose(const ClShape &s, const scanscam_plan &u, ClCandidate *bes
             if (!u.vec && kind == 2 && s.esize == 2 && vecs[iv] == 8) continue;
             for (int is = 0; is < 4; is++) {
                 if (u.unroll && u.unroll != all_steps[is]) continue;
-                for (int iw = 0; iw < (u.waves ? 1 : 2); iw++) {
+                for (int iw = 0; iw < (u.waves ? 1 : (kind == 0 ? 3 : 2)); iw++) {
                     ClCandidate c{vecs[iv], all_steps[is], u.waves ? u.waves : all_waves[iw], kind, kWave, false};
                     if (!u.waves) {
                         // No more waves than the LDS arrays and the thread limit allow, nor than there are spans of time.

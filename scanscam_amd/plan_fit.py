@@ -166,8 +166,10 @@ def load(paths):
 
 
 def candidate(d):
-    """A plan the library's own choice considers (cl_choose): 4 or 8 waves, no 16-byte 16-bit lanes in a time split."""
-    return d["waves"] in (4, 8) and not (d["kind"] == 2 and d["esize"] == 2 and d["vec"] == 8)
+    """A plan the library's own choice considers (cl_choose): 4 or 8 waves (a walk also 16), no 16-byte 16-bit lanes in
+    a time split."""
+    waves = (4, 8, 16) if d["kind"] == 0 else (4, 8)
+    return d["waves"] in waves and not (d["kind"] == 2 and d["esize"] == 2 and d["vec"] == 8)
 
 
 def regret(by, p, out, label):

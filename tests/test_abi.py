@@ -224,7 +224,7 @@ def _forced_cl_plans(dtype):
     full = 16 // torch.empty(0, dtype=dtype).element_size()
     widths = sorted({1, full, max(1, full // 2)} | ({2} if full == 8 else set()))
     return [hip.Plan(mode=m, vec=v, unroll=s, waves=w) for v in widths for m in (WALK, TILES)
-            for s in ((2, 4, 8) if v == full else (4, 8, 16)) for w in (4, 8)]
+            for s in ((2, 4, 8) if v == full else (4, 8, 16)) for w in ((4, 8, 16) if m == WALK else (4, 8))]
 
 
 def test_the_automatic_channels_last_plan_is_the_cheapest_by_the_cost_model():
