@@ -245,3 +245,46 @@ def test_channels_last_views_with_a_far_time_stride_are_copied_first():
     # Exactly the library's inequality (time stride * size * 18 + C * size < 2^32).
     for stride, C, esize in ((59_652_323, 4, 4), (59_652_324, 4, 4), (119_304_646, 8, 2), (119_304_647, 2, 2)):
         assert hip._cl_step_too_far(stride, C, esize) == (stride * esize * 18 + C * esize >= 2 ** 32)
+
+
+def test_the_fitting_tool_recovers_a_table_from_timings_and_writes_it_back(tmp_path):
+    """plan_fit end to end on the CPU: timings generated from the shipped table (with 2 % noise), in the format
+    plan_search --dump writes, are read, fitted, printed as a .inc and read back; the fitted model then orders the
+    plans of each shape as the generating table does."""
+    import io
+    import os
+
+    from scanscam_amd import plan_fit
+
+    root = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..")
+    table = plan_fit.read_table(os.path.join(root, "scanscam_amd", "csrc", "scan_cl_model.inc"))
+    rng = np.random.default_rng(11)
+    dump = tmp_path / "dump.txt"
+    with open(dump, "w") as f:
+        for _ in range(60):
+            batch, T, C = int(2 ** rng.uniform(3, 10)), int(2 ** rng.uniform(8, 13)), 64 * int(rng.integers(1, 24))
+            for direction in ("fwd", "bwd"):
+                for mode in (2, 3):
+                    for vec, steps in ((1, 16), (2, 8), (4, 4), (4, 8)):
+                        for waves in (4, 8):
+                            d = plan_fit.describe(batch, T, C, 4, direction == "bwd", mode, vec, steps, waves)
+                            us = plan_fit.predict(d, table) * float(np.exp(rng.normal(0, 0.02)))
+                            f.write(f"{batch} {T} {C} float32 {direction} {mode} {vec} {steps} {waves} {us:.2f}\n")
+    by = plan_fit.load([str(dump)])
+    assert len(by) == 120
+    p, rms, seen, n = plan_fit.fit(by, evaluations=60)
+    assert n > 1000 and rms < 0.05, (n, rms)
+    text = io.StringIO()
+    plan_fit.emit(p, seen, "dump.txt", text)
+    inc = tmp_path / "model.inc"
+    inc.write_text(text.getvalue())
+    back = plan_fit.read_table(str(inc))
+    assert back.shape == table.shape
+    picked, ideal = [], []
+    for key, timings in by.items():
+        plans = [(d, us) for d, us in timings if d is not None and plan_fit.candidate(d)]
+        truth = [plan_fit.predict(d, table) for d, _ in plans]
+        choice = int(np.argmin([plan_fit.predict(d, back) for d, _ in plans]))
+        picked.append(truth[choice])
+        ideal.append(min(truth))
+    assert np.mean(np.array(picked) / np.array(ideal)) < 1.02
