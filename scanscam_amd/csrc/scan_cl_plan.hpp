@@ -2,17 +2,17 @@
 //
 // Every launch shape the kernels are instantiated for is a candidate: lanes of 1 channel up to 16 bytes
 // (whole, or element-aligned where C or the alignment does not allow whole ones), a workgroup that walks
-// all of T or tiles of time handed out over workgroups, 2 to 16 time steps per wave, 4 or 8 waves. For
-// each candidate cl_predict_us() estimates the launch's duration from a few terms, and the plan is the
+// all of T or tiles of time handed out over workgroups, 2 to 16 time steps per wave, 4 or 8 waves (a walk
+// also 16). For each candidate cl_predict_us() estimates the launch's duration from a few terms, and the plan is the
 // candidate with the smallest estimate. Fields that the caller's plan names are taken as given and only
 // the others are chosen.
 //
 // The terms (microseconds):
 //   stream   algorithmic bytes / (rate of this kernel variant) x (lines touched / lines used) / fill^alpha
 //            `rate`: one measured streaming rate per kernel variant (kernel, lane bytes, storage size,
-//            direction, and whether a time step is whole 128-byte lines), the table of scan_cl_model.inc; `lines touched`: every wave access that starts or ends
-//            inside a 128-byte line moves the rest of that line as well; `fill`: the part of the lanes
-//            of a time step's waves that hold a channel.
+//            direction, and whether a time step is whole 128-byte lines), the table of scan_cl_model.inc;
+//            `lines touched`: every wave access that starts or ends inside a 128-byte line moves the rest of
+//            that line as well; `fill`: the part of the lanes of a time step's waves that hold a channel.
 //   latency  rounds of workgroups x tiles per workgroup x time of one tile, where a tile takes the memory
 //            latency plus the issue time of its waves' instructions (proportional to elements per lane,
 //            more backwards, for 16-bit storage and for element-aligned lanes), a tile of the time split
@@ -25,7 +25,9 @@
 //
 // The constants are fitted, not hand-set: `python -m scanscam_amd.plan_search --dump FILE` times every
 // candidate on a set of shapes and `python -m scanscam_amd.plan_fit FILE...` fits them to those timings and
-// prints this file's table (scan_cl_model.inc). No shape has a rule of its own.
+// prints this file's table (scan_cl_model.inc). No shape has a rule of its own. Two facts about resources are
+// constraints on the candidates instead of terms (cl_choose): 16-byte lanes of 16-bit storage spill in the time
+// split, and a walk with fewer workgroups than half the compute units cannot keep the chip busy.
 #pragma once
 
 #include "scan_launch.hpp"
