@@ -11,6 +11,11 @@
 //   copy_calib order    the look-back tile (8 waves x 4 accesses) in the look-back kernel's tile-major order of
 //                       work: the stream is cut into R rows and workgroup k takes tile k / R of row k % R, so tiles
 //                       of all R rows are in flight together (R = 1 is one linear sweep).
+//   copy_calib cl       channels-last tensors [B, T, C]: a workgroup's waves are `side` channel spans side by side
+//                       (64 lanes x the lane's bytes each) times `spans` spans of S time steps, tiles of time handed
+//                       out over workgroups as in the time-split kernel. side = 1 is that kernel's shape (a wave
+//                       reads pieces of a time step, one row of C apart); side = all spans of a time step makes a
+//                       workgroup's tile one contiguous block of memory.
 #include <hip/hip_runtime.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -73,6 +78,41 @@ __global__ __launch_bounds__(W * 64) void stream_kernel(const f4 *__restrict__ a
     }
 }
 
+// Channels-last shapes: lane vector V (4, 8 or 16 bytes), S time steps per wave. Workgroup k covers tile
+// k / (batch * blocks) of (batch element, channel block) k % (batch * blocks); wave w is channel span w % side of
+// the block and time span w / side of the tile.
+template <typename V, int S, int READS, int WRITES>
+__global__ __launch_bounds__(1024) void cl_stream_kernel(const char *__restrict__ a, const char *__restrict__ b,
+                                                         const char *__restrict__ c, char *__restrict__ o0,
+                                                         char *__restrict__ o1, int batch, int T, int row_bytes, int side)
+{
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, spans = blockDim.x / 64 / side;
+    const int span_bytes = 64 * (int)sizeof(V), blocks = (row_bytes + side * span_bytes - 1) / (side * span_bytes);
+    const int pairs = batch * blocks, pair = blockIdx.x % pairs, tile = blockIdx.x / pairs;
+    const int col = ((pair % blocks) * side + wave % side) * span_bytes + lane * (int)sizeof(V);
+    const int t0 = (tile * spans + wave / side) * S;
+    const size_t base = ((size_t)(pair / blocks) * T + t0) * row_bytes + col;
+    const bool live = col + (int)sizeof(V) <= row_bytes;
+    V va[S], vb[S], vc[S];
+#pragma unroll
+    for (int k = 0; k < S; k++) {
+        const bool ok = live && t0 + k < T;
+        const size_t at = ok ? base + (size_t)k * row_bytes : 0;
+        va[k] = __builtin_nontemporal_load(reinterpret_cast<const V *>(a + at));
+        if (READS > 1) vb[k] = __builtin_nontemporal_load(reinterpret_cast<const V *>(b + at));
+        if (READS > 2) vc[k] = __builtin_nontemporal_load(reinterpret_cast<const V *>(c + at));
+    }
+#pragma unroll
+    for (int k = 0; k < S; k++) {
+        if (!(live && t0 + k < T)) continue;
+        V r = va[k];
+        if (READS > 1) r += vb[k];
+        if (READS > 2) r *= vc[k];
+        __builtin_nontemporal_store(r, reinterpret_cast<V *>(o0 + base + (size_t)k * row_bytes));
+        if (WRITES > 1) __builtin_nontemporal_store(r + r, reinterpret_cast<V *>(o1 + base + (size_t)k * row_bytes));
+    }
+}
+
 static const size_t kStreamElems = (size_t)16384 * 4096;  // fp32 per stream
 static f4 *g_sets[4][5];
 
@@ -100,6 +140,76 @@ template <int READS, int WRITES, int U, int W> static int stream_case(unsigned R
     CHECK(hipEventDestroy(e0));
     CHECK(hipEventDestroy(e1));
     return 0;
+}
+
+template <typename V, int S, int READS, int WRITES> static int cl_case(int batch, int T, int row_bytes, int side, int spans)
+{
+    const int span_bytes = 64 * (int)sizeof(V), blocks = (row_bytes + side * span_bytes - 1) / (side * span_bytes);
+    const int tiles = (T + spans * S - 1) / (spans * S);
+    const size_t bytes_per_stream = (size_t)batch * T * row_bytes;
+    if (bytes_per_stream > kStreamElems * 4 || side * spans > 16) return 1;
+    hipEvent_t e0, e1;
+    CHECK(hipEventCreate(&e0));
+    CHECK(hipEventCreate(&e1));
+    const int launches = 40;
+    for (int i = -4; i < launches; i++) {
+        f4 **s = g_sets[(i + 4) % 4];
+        if (i == 0) CHECK(hipEventRecord(e0, 0));
+        hipLaunchKernelGGL((cl_stream_kernel<V, S, READS, WRITES>), dim3((unsigned)(batch * blocks * tiles)),
+                           dim3(side * spans * 64), 0, 0, (const char *)s[0], (const char *)s[1], (const char *)s[2],
+                           (char *)s[3], (char *)s[4], batch, T, row_bytes, side);
+    }
+    CHECK(hipEventRecord(e1, 0));
+    CHECK(hipEventSynchronize(e1));
+    float ms = 0;
+    CHECK(hipEventElapsedTime(&ms, e0, e1));
+    ms /= launches;
+    const double bytes = (double)(READS + WRITES) * bytes_per_stream;
+    printf("  %dR%dW  %2d-byte lanes  %2d side by side x %2d spans x %2d steps  %5d workgroups  %7.1f us  %4.1f %%\n", READS, WRITES,
+           (int)sizeof(V), side, spans, S, batch * blocks * tiles, ms * 1e3, bytes / (ms * 1e-3) / 8e12 * 100);
+    CHECK(hipEventDestroy(e0));
+    CHECK(hipEventDestroy(e1));
+    return 0;
+}
+
+typedef float f2 __attribute__((ext_vector_type(2)));
+
+template <typename V, int S> static int cl_both(int batch, int T, int row_bytes, int side, int spans)
+{
+    return cl_case<V, S, 2, 1>(batch, T, row_bytes, side, spans) | cl_case<V, S, 3, 2>(batch, T, row_bytes, side, spans);
+}
+
+static int run_cl()
+{
+    for (auto &set : g_sets)
+        for (auto &p : set) {
+            CHECK(hipMalloc(&p, kStreamElems * 4));
+            CHECK(hipMemset(p, 0, kStreamElems * 4));
+        }
+    int rc = 0;
+    printf("channels-last tile shapes, scan-free (forward mix 2R1W, backward mix 3R2W), 4 rotated buffer sets, %% of 8 TB/s:\n");
+    printf("fp32 [8, 4096, 512] (time steps of 2048 bytes):\n");
+    rc |= cl_both<f2, 16>(8, 4096, 2048, 1, 8) | cl_both<f2, 16>(8, 4096, 2048, 2, 4) | cl_both<f2, 16>(8, 4096, 2048, 4, 2) |
+          cl_both<f2, 16>(8, 4096, 2048, 4, 4) | cl_both<f4, 8>(8, 4096, 2048, 1, 8) | cl_both<f4, 8>(8, 4096, 2048, 2, 4) |
+          cl_both<f4, 8>(8, 4096, 2048, 2, 8) | cl_both<float, 16>(8, 4096, 2048, 1, 8) | cl_both<float, 16>(8, 4096, 2048, 8, 1) |
+          cl_both<float, 16>(8, 4096, 2048, 8, 2);
+    printf("16-bit [8, 4096, 512] (time steps of 1024 bytes):\n");
+    rc |= cl_both<float, 16>(8, 4096, 1024, 1, 8) | cl_both<float, 16>(8, 4096, 1024, 4, 2) | cl_both<float, 16>(8, 4096, 1024, 4, 4) |
+          cl_both<f2, 16>(8, 4096, 1024, 1, 8) | cl_both<f2, 16>(8, 4096, 1024, 2, 4) | cl_both<f2, 16>(8, 4096, 1024, 2, 8);
+    printf("fp32 [8, 4096, 2048] (time steps of 8192 bytes):\n");
+    rc |= cl_both<f2, 16>(8, 4096, 8192, 1, 8) | cl_both<f2, 16>(8, 4096, 8192, 4, 2) | cl_both<f2, 16>(8, 4096, 8192, 8, 1) |
+          cl_both<f2, 16>(8, 4096, 8192, 16, 1) | cl_both<f4, 8>(8, 4096, 8192, 8, 1) | cl_both<f4, 8>(8, 4096, 8192, 8, 2);
+    printf("fp32 [32, 2048, 1001] (time steps of 4004 bytes, no whole lines):\n");
+    rc |= cl_both<float, 16>(32, 2048, 4004, 1, 8) | cl_both<float, 16>(32, 2048, 4004, 1, 16) | cl_both<float, 16>(32, 2048, 4004, 16, 1) |
+          cl_both<float, 16>(32, 2048, 4004, 8, 2) | cl_both<float, 16>(32, 2048, 4004, 4, 4) | cl_both<float, 8>(32, 2048, 4004, 16, 1);
+    printf("16-bit [90, 2048, 514] (time steps of 1028 bytes, no whole lines):\n");
+    rc |= cl_both<float, 16>(90, 2048, 1028, 1, 8) | cl_both<float, 16>(90, 2048, 1028, 5, 1) | cl_both<float, 16>(90, 2048, 1028, 5, 2) |
+          cl_both<float, 16>(90, 2048, 1028, 5, 3);
+    printf("fp32 [32, 2048, 1024] (time steps of 4096 bytes; tiles only, a workgroup that walks all of T is not modelled):\n");
+    rc |= cl_both<f2, 8>(32, 2048, 4096, 1, 8) | cl_both<f2, 8>(32, 2048, 4096, 8, 1) | cl_both<f2, 8>(32, 2048, 4096, 8, 2) |
+          cl_both<f4, 8>(32, 2048, 4096, 4, 2) | cl_both<f4, 8>(32, 2048, 4096, 4, 4);
+    CHECK(hipDeviceSynchronize());
+    return rc;
 }
 
 static int run_streams(bool order)
@@ -131,6 +241,7 @@ static int run_streams(bool order)
 
 int main(int argc, char **argv)
 {
+    if (argc > 1 && argv[1][0] == 'c') return run_cl();
     if (argc > 1 && (argv[1][0] == 'm' || argv[1][0] == 'o')) return run_streams(argv[1][0] == 'o');
     const size_t mib = argc > 1 ? (size_t)atol(argv[1]) : 1024;
     const int launches = argc > 2 ? atoi(argv[2]) : 20;
