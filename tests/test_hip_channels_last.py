@@ -298,11 +298,13 @@ def test_few_channels_packed_kernel(gpu, dtype):
             assert rel_err(as_rows(got_ga), ga, prev_abs(as_rows(hs))) <= bar, (plan, shape)
 
 
-# (dtype, [batch, T, C], slice of C taken from a wider buffer or None). Automatic plans on grids of 64 and
-# more workgroups: time steps that are not whole 128-byte lines (every XCD then takes a contiguous run of
-# workgroups; numbers of workgroups that are and are not multiples of 8, dense tensors and views whose
-# rows are whole lines but start inside one; also with time split over workgroups), 320 workgroups of
-# 16-byte lanes (4-wave workgroups), and 16-bit single-channel lanes with 16 steps per wave.
+# (dtype, [batch, T, C], slice of C taken from a wider buffer or None). Shapes at the borders where the automatic
+# launch plan changes -- lane width, a walk of all of T or tiles of time over workgroups, steps per wave, waves,
+# several time steps per instruction -- and where the kernels' special cases sit: time steps that are not whole
+# 128-byte lines (dense, and views whose rows are whole lines but start inside one), numbers of (batch element,
+# channel group) pairs that are and are not multiples of 8, channel counts on and off every lane's multiple, rows of
+# one or two tiles, a single time step, very wide time steps. Whatever plan the cost model picks there, the result
+# has to agree with the oracle.
 MANY_WORKGROUPS = [
     (torch.float32, (37, 300, 1000), None),
     (torch.float32, (67, 90, 1000), None),
@@ -315,76 +317,76 @@ MANY_WORKGROUPS = [
     (torch.float64, (40, 100, 500), None),
     (torch.float32, (20, 150, 1000), (8, 1056)),
     (torch.bfloat16, (24, 140, 1024), (16, 1088)),
-    (torch.float32, (8, 2100, 500), None),      # time split over workgroups, 64 row-groups: XCD runs there too
+    (torch.float32, (8, 2100, 500), None),
     (torch.bfloat16, (8, 1500, 1000), None),
     (torch.float32, (80, 200, 1024), None),
-    (torch.bfloat16, (260, 130, 64), None),     # 16-bit, 33-511 channels: one channel per lane at 64 ...
-    (torch.bfloat16, (260, 130, 96), None),     # ... pairs otherwise (48 lanes of a wave)
-    (torch.float16, (300, 100, 40), None),      # (two time steps per instruction)
+    (torch.bfloat16, (260, 130, 64), None),
+    (torch.bfloat16, (260, 130, 96), None),
+    (torch.float16, (300, 100, 40), None),
     (torch.bfloat16, (257, 64, 256), None),
-    (torch.bfloat16, (9, 3000, 64), None),      # the same with time split over workgroups
+    (torch.bfloat16, (9, 3000, 64), None),
     (torch.bfloat16, (16, 1100, 1024), None),
-    (torch.float32, (260, 60, 256), None),      # 8-byte lanes: chosen ahead of 16-byte lanes ...
+    (torch.float32, (260, 60, 256), None),
     (torch.bfloat16, (130, 70, 1024), None),
-    (torch.float32, (130, 70, 512), None),      # ... and where only they and narrower ones give 256 workgroups
+    (torch.float32, (130, 70, 512), None),
     (torch.float16, (64, 100, 1016), None),
-    (torch.bfloat16, (64, 90, 1001), None),     # element-aligned 8-byte lanes (16-byte ones: 128 workgroups)
+    (torch.bfloat16, (64, 90, 1001), None),
     (torch.float32, (70, 50, 501), None),
-    (torch.float32, (300, 100, 40), None),      # fp32 below 128 channels: pairs of channels, 8 steps per wave ...
+    (torch.float32, (300, 100, 40), None),
     (torch.float32, (257, 64, 96), None),
     (torch.float32, (300, 200, 8), None),
-    (torch.float32, (260, 90, 64), None),       # ... one channel per lane at exactly 64
-    (torch.bfloat16, (300, 200, 8), None),      # 16-bit pairs, several time steps per instruction, 8 instructions
+    (torch.float32, (260, 90, 64), None),
+    (torch.bfloat16, (300, 200, 8), None),
     (torch.float16, (300, 100, 24), None),
-    (torch.float32, (8, 2100, 512), None),      # time split over workgroups: 8-byte lanes forwards (fp32) ...
-    (torch.bfloat16, (8, 1500, 1024), None),    # ... and backwards (16-bit storage)
-    (torch.float16, (8, 1100, 2048), None),     # 256 workgroups of single channels forwards, tiles of four-channel lanes backwards
-    (torch.float32, (36, 1100, 512), None),     # 288 workgroups of 8-byte lanes: tiles over workgroups instead
+    (torch.float32, (8, 2100, 512), None),
+    (torch.bfloat16, (8, 1500, 1024), None),
+    (torch.float16, (8, 1100, 2048), None),
+    (torch.float32, (36, 1100, 512), None),
     (torch.bfloat16, (36, 1100, 1024), None),
-    (torch.float32, (260, 50, 320), None),      # lanes that would leave their last group half empty: single channels
-    (torch.float32, (50, 1100, 512), None),     # 200 workgroups of 8-byte lanes are enough for a walk of all of T
-    (torch.float32, (260, 1100, 48), None),     # a workgroup per batch element, a few too many: tiles of single channels
+    (torch.float32, (260, 50, 320), None),
+    (torch.float32, (50, 1100, 512), None),
+    (torch.float32, (260, 1100, 48), None),
     (torch.bfloat16, (260, 1100, 48), None),
-    (torch.bfloat16, (400, 60, 200), None),     # 16-bit storage: 129-256 channels in four-channel lanes, 4-wave workgroups
-    (torch.float16, (300, 50, 320), None),      # 320 channels: whole waves of single channels
-    (torch.bfloat16, (130, 70, 1003), None),    # 16-bit, 260 workgroups of 16-byte lanes: element-aligned 8-byte lanes, 4 waves
-    (torch.float16, (96, 70, 1501), None),      # ... 8 waves (576 workgroups)
-    (torch.bfloat16, (130, 70, 1004), None),    # ... whole 8-byte lanes
-    (torch.float32, (300, 600, 256), None),     # 0.78 of the rounds started: fp32 forwards in tiles over workgroups
-    (torch.float32, (300, 600, 77), None),      # ... single channels in both directions
-    (torch.bfloat16, (300, 600, 77), None),     # ... 16-bit storage backwards only
-    (torch.float32, (260, 70, 333), None),      # lanes that fill their waves better: element-aligned pairs of fp32 channels, 16 steps
-    (torch.bfloat16, (260, 70, 333), None),     # ... element-aligned pairs of 16-bit channels
+    (torch.bfloat16, (400, 60, 200), None),
+    (torch.float16, (300, 50, 320), None),
+    (torch.bfloat16, (130, 70, 1003), None),
+    (torch.float16, (96, 70, 1501), None),
+    (torch.bfloat16, (130, 70, 1004), None),
+    (torch.float32, (300, 600, 256), None),
+    (torch.float32, (300, 600, 77), None),
+    (torch.bfloat16, (300, 600, 77), None),
+    (torch.float32, (260, 70, 333), None),
+    (torch.bfloat16, (260, 70, 333), None),
     (torch.float16, (130, 1030, 601), None),
-    (torch.bfloat16, (260, 130, 256), None),    # 16-bit, 129-256 channels: four-channel lanes, 4 waves
-    (torch.bfloat16, (32, 1100, 4096), None),   # 16-bit, 4096 or more channels: 16-byte lanes backwards
-    (torch.float64, (260, 70, 256), None),      # float64: single channels (8-byte lanes) ahead of 16-byte lanes
-    (torch.float64, (8, 1100, 256), None),      # ... 8 steps per tile backwards when time is split over workgroups
-    (torch.float32, (2, 40, 65536), None),      # very wide time steps
+    (torch.bfloat16, (260, 130, 256), None),
+    (torch.bfloat16, (32, 1100, 4096), None),
+    (torch.float64, (260, 70, 256), None),
+    (torch.float64, (8, 1100, 256), None),
+    (torch.float32, (2, 40, 65536), None),
     (torch.bfloat16, (1, 7, 100001), None),
-    (torch.float16, (300, 1, 1000), None),      # a single time step
-    (torch.float32, (20, 300, 2048), None),     # fp32, 2048 or more channels: 16 steps per wave forwards, 16-byte lanes backwards
+    (torch.float16, (300, 1, 1000), None),
+    (torch.float32, (20, 300, 2048), None),
     (torch.float32, (10, 200, 4096), None),
-    (torch.float32, (600, 65, 432), None),      # rows of one or two tiles: waves that fill the tiles evenly (5 and 9 of them)
-    (torch.bfloat16, (520, 67, 85), None),      # ... single channels of 16-bit storage, 9 waves
-    (torch.float32, (700, 99, 64), None),       # ... 7 and 13 waves
-    (torch.bfloat16, (300, 75, 943), None),     # ... lanes of 8 bytes: three tiles of 4 waves
-    (torch.float32, (1200, 330, 21), None),     # ... two time steps per instruction, 6 and 11 waves
-    (torch.float32, (600, 500, 40), None),      # 33 to 63 channels: single channels forwards, 16-byte lanes backwards
-    (torch.bfloat16, (600, 520, 40), None),     # ... four-channel lanes backwards
-    (torch.float32, (520, 300, 8), None),       # up to 32 channels of fp32: 16-byte lanes, 4 steps, 4 waves
-    (torch.float32, (100, 1300, 24), None),     # ... the walk from 80 workgroups on
-    (torch.bfloat16, (64, 2100, 16), None),     # ... tiles of single 16-bit channels below that
-    (torch.float32, (260, 600, 113), None),     # fp32 off whole lines: tiles backwards from 384 steps on
-    (torch.float32, (60, 2000, 113), None),     # ... and forwards from 1900
-    (torch.float32, (14, 1100, 2539), None),    # element-aligned fp32 lanes, a few workgroups too many: tiles of single channels
-    (torch.bfloat16, (71, 600, 257), None),     # 16-bit backwards: 213 workgroups of element-aligned pairs
-    (torch.bfloat16, (39, 125, 4806), None),    # short rows, element-aligned: four-channel lanes
-    (torch.float32, (350, 300, 65), None),      # 65 to 127 channels, an odd count: one wave of element-aligned pairs
+    (torch.float32, (600, 65, 432), None),
+    (torch.bfloat16, (520, 67, 85), None),
+    (torch.float32, (700, 99, 64), None),
+    (torch.bfloat16, (300, 75, 943), None),
+    (torch.float32, (1200, 330, 21), None),
+    (torch.float32, (600, 500, 40), None),
+    (torch.bfloat16, (600, 520, 40), None),
+    (torch.float32, (520, 300, 8), None),
+    (torch.float32, (100, 1300, 24), None),
+    (torch.bfloat16, (64, 2100, 16), None),
+    (torch.float32, (260, 600, 113), None),
+    (torch.float32, (60, 2000, 113), None),
+    (torch.float32, (14, 1100, 2539), None),
+    (torch.bfloat16, (71, 600, 257), None),
+    (torch.bfloat16, (39, 125, 4806), None),
+    (torch.float32, (350, 300, 65), None),
     (torch.bfloat16, (350, 300, 113), None),
-    (torch.float16, (400, 67, 127), None),      # ... on a row of two tiles
+    (torch.float16, (400, 67, 127), None),
     (torch.float32, (345, 520, 93), None),
-    (torch.bfloat16, (15, 1100, 188), None),    # 16-bit backward tiles in four-channel lanes that fill 47 of a wave's 64 lanes
+    (torch.bfloat16, (15, 1100, 188), None),
     (torch.float16, (13, 900, 400), None),
 ]
 
@@ -413,6 +415,36 @@ def test_automatic_plans_on_many_workgroups(gpu, dtype, shape, window):
     assert got_h.shape == a.mT.shape and got_h.mT.is_contiguous()
     assert rel_err(as_rows(got_h.mT), h) <= bar
     hs = place(torch.from_numpy(h).mT)
+    ga, gb = oracle.bwd(as_rows(a), as_rows(hs), as_rows(gh))
+    got_ga, got_gb = hip.scan_backward(a.mT, hs.mT, gh.mT)
+    assert rel_err(as_rows(got_gb.mT), gb) <= bar
+    assert rel_err(as_rows(got_ga.mT), ga, prev_abs(as_rows(hs))) <= bar
+
+
+def _large_shapes():
+    from scanscam_amd import plan_search
+
+    shapes = [s for s in plan_search.random_cl_shapes(60, 101) if s[0] * s[1] * s[2] <= 24 << 20][:8]
+    return [(dtype, s) for s in shapes for dtype in (torch.float32, torch.bfloat16)]
+
+
+@pytest.mark.parametrize("dtype,shape", _large_shapes())
+def test_automatic_plans_on_large_shapes(gpu, dtype, shape):
+    """The automatic plan of shapes of the size the plan search times (8 M to 24 M elements, drawn like its random
+    audit's): at that size the cost model picks plans (16-wave walks, tiles in wide lanes) that the small shapes of
+    the other tests never reach. Against the oracle, the bars of the other tests."""
+    bar = 1e-5 if dtype == torch.float32 else 1e-2
+    B, T, C = shape
+    g = torch.Generator().manual_seed(B + T + C)
+    a = torch.rand(shape, generator=g, dtype=torch.float32).to(dtype).to(gpu)
+    b = torch.randn(shape, generator=g, dtype=torch.float32).to(dtype).to(gpu)
+    gh = torch.randn(shape, generator=g, dtype=torch.float32).to(dtype).to(gpu)
+    plans = [hip.resolve_plan_cl(B, T, C, dtype, d) for d in (hip.FORWARD, hip.BACKWARD)]
+    print(f"case cl large {dtype} shape={shape} plans={plans}", flush=True)
+    h = oracle.fwd(as_rows(a), as_rows(b))
+    got_h = hip.scan_forward(a.mT, b.mT)
+    assert rel_err(as_rows(got_h.mT), h) <= bar
+    hs = torch.from_numpy(h).mT.to(dtype).to(gpu).contiguous()  # [B, T, C], rounded to the storage type
     ga, gb = oracle.bwd(as_rows(a), as_rows(hs), as_rows(gh))
     got_ga, got_gb = hip.scan_backward(a.mT, hs.mT, gh.mT)
     assert rel_err(as_rows(got_gb.mT), gb) <= bar
