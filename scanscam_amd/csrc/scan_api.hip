@@ -631,7 +631,34 @@ int resolve_cl(const scanscam_plan *user, int64_t batch, int64_t T, int64_t C, i
     if (u.mode != SCANSCAM_MODE_AUTO && u.mode != kModeRow && u.mode != kModeLookback) return SCANSCAM_EPLAN;
     const scanscam::ClShape shape = {batch, T, C, esize, compute_size(dtype), align, rev};
     scanscam::ClCandidate c;
-    if (!scanscam::cl_choose(shape, u, &c, predicted_us)) return SCANSCAM_EPLAN;
+    // The choice is a pure function of (shape, caller's plan) and costs about a hundred microseconds (some forty
+    // candidates through the cost model), so each thread remembers its last few dozen: a model calls the same shapes
+    // over and over. Nothing but speed depends on it.
+    struct Remembered {
+        bool valid;
+        int64_t batch, T, C;
+        int dtype, align;
+        bool rev;
+        int32_t mode, vec, unroll, waves;
+        scanscam::ClCandidate c;
+        double us;
+    };
+    constexpr int kRemembered = 64;
+    static thread_local Remembered remembered[kRemembered] = {};
+    const uint64_t key = (uint64_t)batch * 0x9E3779B97F4A7C15ull ^ (uint64_t)T * 0xC2B2AE3D27D4EB4Full ^ (uint64_t)C * 0x165667B19E3779F9ull ^
+                         (uint64_t)(dtype * 64 + align * 2 + (rev ? 1 : 0)) * 0x27D4EB2F165667C5ull ^
+                         (uint64_t)(u.mode * 4096 + u.vec * 256 + u.unroll * 16 + u.waves);
+    Remembered &slot = remembered[(key >> 32 ^ key) % kRemembered];
+    if (slot.valid && slot.batch == batch && slot.T == T && slot.C == C && slot.dtype == dtype && slot.align == align &&
+        slot.rev == rev && slot.mode == u.mode && slot.vec == u.vec && slot.unroll == u.unroll && slot.waves == u.waves) {
+        c = slot.c;
+        if (predicted_us) *predicted_us = slot.us;
+    } else {
+        double us = 0.0;
+        if (!scanscam::cl_choose(shape, u, &c, &us)) return SCANSCAM_EPLAN;
+        slot = Remembered{true, batch, T, C, dtype, align, rev, u.mode, u.vec, u.unroll, u.waves, c, us};
+        if (predicted_us) *predicted_us = us;
+    }
 
     l->vec = c.vec;
     l->steps = c.steps;

@@ -71,7 +71,21 @@ struct ClModel {
     double line[4];      // weight of the lines touched beyond the bytes used, for lanes of 2, 4, 8, 16 bytes
 };
 
-#include "scan_cl_model.inc"  // const ClModel kClModel = {...}: printed by scanscam_amd/plan_fit.py
+// What the formula leaves unexplained (about 7 % rms against 1 % of run-to-run noise) a small network has learned
+// from the same timings: ln(measured / estimate) as a function of cl_features(), two hidden layers of tanh units.
+// The library only evaluates it; scanscam_amd/plan_fit.py trains it and prints its weights.
+constexpr int kClInputs = 24, kClHidden1 = 64, kClHidden2 = 32;
+constexpr double kClResidualLimit = 0.7;  // the correction of ln(duration) stays within +-0.7
+
+struct ClResidual {
+    double lo[kClInputs], hi[kClInputs];      // range of each input in the training timings: inputs are clipped to it
+    double mean[kClInputs], scale[kClInputs]; // standardisation
+    double w1[kClInputs][kClHidden1], b1[kClHidden1];
+    double w2[kClHidden1][kClHidden2], b2[kClHidden2];
+    double w3[kClHidden2], b3;
+};
+
+#include "scan_cl_model.inc"  // const ClModel kClModel = {...}; const ClResidual kClResidual = {...}: printed by scanscam_amd/plan_fit.py
 
 struct ClShape {
     int64_t batch, T, C;
@@ -134,7 +148,8 @@ inline double cl_registers(const ClShape &s, const ClCandidate &c)
     return base + c.steps * c.vec * per * (s.esize == 8 ? 2.0 : 1.0);
 }
 
-inline double cl_predict_us(const ClShape &s, const ClCandidate &c, const ClModel &m = kClModel)
+// The formula: launch + stream + latency + chain (see the head of this file). `x`, if given, receives cl_features().
+inline double cl_physical_us(const ClShape &s, const ClCandidate &c, const ClModel &m = kClModel, double *x = nullptr)
 {
     const int sub = kWave / c.group;  // time steps per wave instruction
     const int64_t G = cl_groups(s.C, c.vec);
@@ -190,7 +205,63 @@ inline double cl_predict_us(const ClShape &s, const ClCandidate &c, const ClMode
     }
     const double stream_us = bytes / std::pow(fill, m.fill_alpha) / rate * lines;
     const double chain_us = c.kind == 2 ? m.chain * (double)tiles / c.waves : 0.0;
-    return m.launch + (c.kind == 2 ? m.launch_split : 0.0) + stream_us + latency_us + chain_us;
+    const double us = m.launch + (c.kind == 2 ? m.launch_split : 0.0) + stream_us + latency_us + chain_us;
+    if (x) {  // cl_features: what the learned correction sees of (shape, plan)
+        x[0] = std::log2((double)RG);
+        x[1] = std::log2((double)tiles);
+        x[2] = std::log2((double)s.T);
+        x[3] = std::log2((double)s.C);
+        x[4] = std::log2((double)s.batch);
+        x[5] = fill;
+        x[6] = c.steps;
+        x[7] = c.vec;
+        x[8] = c.waves;
+        x[9] = c.kind;
+        x[10] = s.esize;
+        x[11] = s.rev ? 1.0 : 0.0;
+        x[12] = c.group < kWave ? 1.0 : 0.0;
+        x[13] = std::log2((double)sub);
+        x[14] = c.ragged ? 1.0 : 0.0;
+        x[15] = cl_registers(s, c);
+        x[16] = std::log2((double)workgroups);
+        x[17] = (double)((workgroups - 1) % kClComputeUnits + 1) / kClComputeUnits;  // how full the last round of workgroups is
+        x[18] = step_bytes % 128 == 0 ? 1.0 : 0.0;
+        x[19] = step_bytes % 16 == 0 ? 1.0 : 0.0;
+        x[20] = std::log2(bytes);
+        x[21] = std::log(us);
+        x[22] = std::log2((double)lane);
+        x[23] = (double)workgroups / kClComputeUnits < 8.0 ? (double)workgroups / kClComputeUnits : 8.0;
+    }
+    return us;
+}
+
+// The learned correction of ln(duration) for one candidate's features.
+inline double cl_residual(const double (&x)[kClInputs], const ClResidual &r = kClResidual)
+{
+    double z[kClInputs], h1[kClHidden1], h2[kClHidden2];
+    for (int i = 0; i < kClInputs; i++) {
+        const double v = x[i] < r.lo[i] ? r.lo[i] : (x[i] > r.hi[i] ? r.hi[i] : x[i]);
+        z[i] = (v - r.mean[i]) / r.scale[i];
+    }
+    for (int j = 0; j < kClHidden1; j++) h1[j] = r.b1[j];
+    for (int i = 0; i < kClInputs; i++)
+        for (int j = 0; j < kClHidden1; j++) h1[j] += z[i] * r.w1[i][j];
+    for (int j = 0; j < kClHidden1; j++) h1[j] = std::tanh(h1[j]);
+    for (int k = 0; k < kClHidden2; k++) h2[k] = r.b2[k];
+    for (int j = 0; j < kClHidden1; j++)
+        for (int k = 0; k < kClHidden2; k++) h2[k] += h1[j] * r.w2[j][k];
+    for (int k = 0; k < kClHidden2; k++) h2[k] = std::tanh(h2[k]);
+    double y = r.b3;
+    for (int k = 0; k < kClHidden2; k++) y += h2[k] * r.w3[k];
+    return y < -kClResidualLimit ? -kClResidualLimit : (y > kClResidualLimit ? kClResidualLimit : y);
+}
+
+// Estimated duration of a candidate: the formula times the learned correction.
+inline double cl_predict_us(const ClShape &s, const ClCandidate &c)
+{
+    double x[kClInputs];
+    const double physical = cl_physical_us(s, c, kClModel, x);
+    return physical * std::exp(cl_residual(x));
 }
 
 // The candidate with the smallest estimate among those that agree with the caller's plan `u` (zero fields are

@@ -8,8 +8,11 @@ The library chooses the launch plan of a channels-last call by estimating every 
 (``scanscam_amd/csrc/scan_cl_plan.hpp``: ``cl_predict_us``) and taking the smallest. This tool holds the same
 formula (``predict`` below; ``tests/test_host.py`` checks the two against each other through
 ``scanscam_predict_cl``), fits its constants to the dumped timings by least squares on the logarithm of the
-duration -- plans within 2.5 times of a shape's best only, weighted towards the best -- and prints the table the
-library is compiled with. To stderr it reports how far the plan the fitted model would pick is behind the best
+duration -- plans within 2.5 times of a shape's best only, weighted towards the best. What that formula leaves
+unexplained (about 7 % rms, against 1 % of run-to-run noise) a small network then learns from the same timings
+(``fit_residual``: 24 inputs that describe shape and plan, two hidden layers, the logarithm of measured over
+estimated duration as the target; scikit-learn trains it, the library only evaluates it), and the tool prints both
+tables, which the library is compiled with. To stderr it reports how far the plan the fitted model would pick is behind the best
 measured plan, per (shape, storage type, direction), on the training files and on ``--held-out`` files that took no
 part in the fit.
 
@@ -107,6 +110,51 @@ def predict(d, p):
     return q["launch"] + (q["launch_split"] if d["kind"] == 2 else 0.0) + stream_us + latency_us + chain_us
 
 
+N_FEATURES, HIDDEN, RESIDUAL_LIMIT = 24, (64, 32), 0.7
+
+
+def features(d, physical_us):
+    """cl_features() of scan_cl_plan.hpp: what the learned correction sees of a (shape, plan) pair."""
+    step_bytes = d["C"] * d["esize"]
+    workgroups = d["RG"] * d["tiles"] if d["kind"] == 2 else d["RG"]
+    return [math.log2(d["RG"]), math.log2(d["tiles"]), math.log2(d["T"]), math.log2(d["C"]), math.log2(d["batch"]),
+            d["fill"], float(d["steps"]), float(d["vec"]), float(d["waves"]), float(d["kind"]), float(d["esize"]),
+            float(d["rev"]), float(d["group"] < WAVE), math.log2(d["sub"]), float(d["ragged"]), registers(d),
+            math.log2(workgroups), ((workgroups - 1) % CUS + 1) / float(CUS), float(step_bytes % 128 == 0),
+            float(step_bytes % 16 == 0), math.log2(d["bytes"]), math.log(physical_us), math.log2(d["lane"]),
+            min(workgroups / float(CUS), 8.0)]
+
+
+class Residual:
+    """The learned correction: ln(measured / physical estimate) as a function of features(), clipped to
+    +-RESIDUAL_LIMIT; inputs are clipped to the range the training timings covered, so it never extrapolates."""
+
+    def __init__(self, lo, hi, mean, scale, w1, b1, w2, b2, w3, b3):
+        self.parts = [np.asarray(a, dtype=np.float64) for a in (lo, hi, mean, scale, w1, b1, w2, b2, w3)] + [float(b3)]
+
+    @classmethod
+    def zero(cls):
+        n, (h1, h2) = N_FEATURES, HIDDEN
+        return cls(np.full(n, -1e30), np.full(n, 1e30), np.zeros(n), np.ones(n), np.zeros((n, h1)), np.zeros(h1),
+                   np.zeros((h1, h2)), np.zeros(h2), np.zeros(h2), 0.0)
+
+    def correct(self, x):
+        """x: [rows, N_FEATURES] (or one row) -> the correction of ln(duration) per row."""
+        lo, hi, mean, scale, w1, b1, w2, b2, w3, b3 = self.parts
+        z = (np.clip(np.atleast_2d(np.asarray(x, dtype=np.float64)), lo, hi) - mean) / scale
+        y = np.tanh(np.tanh(z @ w1 + b1) @ w2 + b2) @ w3 + b3
+        return np.clip(y, -RESIDUAL_LIMIT, RESIDUAL_LIMIT)
+
+    def flat(self):
+        return np.concatenate([np.ravel(a) for a in self.parts[:-1]] + [[self.parts[-1]]])
+
+
+def estimate(d, p, r):
+    """cl_predict_us(): the physical estimate times the learned correction."""
+    physical = predict(d, p)
+    return physical * math.exp(float(r.correct(features(d, physical))[0]))
+
+
 FIELDS = ("steps", "vec", "waves", "rev", "esize", "group", "sub", "ragged", "kind", "RG", "tiles", "lane", "C", "G", "fill",
           "bytes")
 
@@ -172,7 +220,8 @@ def candidate(d):
     return d["waves"] in waves and not (d["kind"] == 2 and d["esize"] == 2 and d["vec"] == 8)
 
 
-def regret(by, p, out, label):
+def regret(by, p, out, label, r=None):
+    cost = (lambda d: estimate(d, p, r)) if r is not None else (lambda d: predict(d, p))
     picks, autos = [], []
     for key, timings in by.items():
         plans = [(d, us) for d, us in timings if d is not None]
@@ -183,7 +232,7 @@ def regret(by, p, out, label):
         if not cands:
             continue
         best = min(us for _, us in plans)
-        picks.append(min(cands, key=lambda t: predict(t[0], p))[1] / best)
+        picks.append(min(cands, key=lambda t: cost(t[0]))[1] / best)
         auto = [us for d, us in timings if d is None]
         if auto:
             autos.append(min(auto) / best)
@@ -241,7 +290,35 @@ def fit(by, evaluations=200):
     return p, float(np.sqrt((residual(sol.x) ** 2).mean())), set(seen), len(rows)
 
 
-def emit(p, seen, note, out):
+def fit_residual(by, p, seed=0, max_iter=600):
+    """Trains the correction on what the fitted formula leaves: ln(measured / physical estimate) of every timed plan
+    within 4 times of its shape's best. Returns (Residual, rms before, rms after) over those timings."""
+    from sklearn.neural_network import MLPRegressor
+    from sklearn.preprocessing import StandardScaler
+
+    x, y = [], []
+    for key, timings in by.items():
+        plans = [(d, us) for d, us in timings if d is not None and d["waves"] in (4, 8, 16)]
+        if not plans:
+            continue
+        best = min(us for _, us in plans)
+        for d, us in plans:
+            if us < 4.0 * best:
+                physical = predict(d, p)
+                x.append(features(d, physical))
+                y.append(math.log(us / physical))
+    x, y = np.array(x), np.array(y)
+    scaler = StandardScaler().fit(x)
+    net = MLPRegressor(hidden_layer_sizes=HIDDEN, activation="tanh", alpha=1e-3, max_iter=max_iter, random_state=seed,
+                       early_stopping=True, n_iter_no_change=25)
+    net.fit(scaler.transform(x), y)
+    r = Residual(x.min(0), x.max(0), scaler.mean_, scaler.scale_, net.coefs_[0], net.intercepts_[0], net.coefs_[1],
+                 net.intercepts_[1], net.coefs_[2][:, 0], net.intercepts_[2][0])
+    after = y - r.correct(x)
+    return r, float(np.sqrt((y ** 2).mean())), float(np.sqrt((after ** 2).mean()))
+
+
+def emit(p, seen, note, out, r=None):
     print("// Constants of the channels-last cost model (ClModel, scan_cl_plan.hpp). Printed by", file=out)
     print(f"//   python -m scanscam_amd.plan_fit {note}", file=out)
     print("// from timings written by `python -m scanscam_amd.plan_search --dump` on one MI355X; do not edit by hand.", file=out)
@@ -275,13 +352,38 @@ def emit(p, seen, note, out):
         print(f"    {q[name]:.4f},  // {name}", file=out)
     print("    {" + ", ".join(f"{q['line_%d' % b]:.4f}" for b in LANES) + "},  // line: lanes of 2, 4, 8, 16 bytes", file=out)
     print("};", file=out)
+    r = r if r is not None else Residual.zero()
+    lo, hi, mean, scale, w1, b1, w2, b2, w3, b3 = r.parts
+
+    def row(a):
+        return "{" + ", ".join(f"{v:.9g}" for v in a) + "}"
+
+    print("", file=out)
+    print("// The learned correction (ClResidual): ln(measured / estimate above) from cl_features(); trained by the same", file=out)
+    print("// command on the same timings. lo, hi: the range of each input in the training timings (inputs are clipped to it).", file=out)
+    print("const ClResidual kClResidual = {", file=out)
+    for name, a in (("lo", lo), ("hi", hi), ("mean", mean), ("scale", scale)):
+        print(f"    {row(a)},  // {name}", file=out)
+    print("    {  // w1[input][hidden 1]", file=out)
+    for a in w1:
+        print(f"        {row(a)},", file=out)
+    print("    },", file=out)
+    print(f"    {row(b1)},  // b1", file=out)
+    print("    {  // w2[hidden 1][hidden 2]", file=out)
+    for a in w2:
+        print(f"        {row(a)},", file=out)
+    print("    },", file=out)
+    print(f"    {row(b2)},  // b2", file=out)
+    print(f"    {row(w3)},  // w3", file=out)
+    print(f"    {b3:.9g},  // b3", file=out)
+    print("};", file=out)
 
 
 def read_table(path):
     """The constants of a scan_cl_model.inc as the vector predict() takes (the inverse of emit())."""
     import re
 
-    body = open(path).read().split("const ClModel kClModel")[1]
+    body = open(path).read().split("const ClModel kClModel")[1].split("\n};")[0]
     body = re.sub(r"/\*.*?\*/", "", body)
     body = re.sub(r"//[^\n]*", "", body)
     nums = [float(x) for x in re.findall(r"-?\d+\.\d+(?:e-?\d+)?", body)]
@@ -289,21 +391,48 @@ def read_table(path):
     return np.array(nums)
 
 
+def read_residual(path):
+    """The learned correction of a scan_cl_model.inc (the inverse of emit()'s second table)."""
+    import re
+
+    body = open(path).read().split("const ClResidual kClResidual")[1].split("\n};")[0]
+    body = re.sub(r"//[^\n]*", "", body)
+    nums = [float(x) for x in re.findall(r"-?(?:\d+\.?\d*|\.\d+)(?:[eE][-+]?\d+)?", body)]
+    n, (h1, h2) = N_FEATURES, HIDDEN
+    sizes = [n, n, n, n, n * h1, h1, h1 * h2, h2, h2, 1]
+    assert len(nums) == sum(sizes), (len(nums), sum(sizes))
+    parts, at = [], 0
+    for size in sizes:
+        parts.append(np.array(nums[at:at + size]))
+        at += size
+    parts[4], parts[6] = parts[4].reshape(n, h1), parts[6].reshape(h1, h2)
+    return Residual(*parts[:9], parts[9][0])
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     ap.add_argument("dumps", nargs="+", help="files written by plan_search --dump")
     ap.add_argument("--held-out", nargs="*", default=[], help="dumps that take no part in the fit, for the report")
     ap.add_argument("--evaluations", type=int, default=200)
+    ap.add_argument("--no-residual", action="store_true", help="fit the formula only; the correction is printed as zero")
     args = ap.parse_args(argv)
     by = load(args.dumps)
     p, rms, seen, n = fit(by, args.evaluations)
     print(f"fitted {N_RATE + len(SCALARS)} constants ({len(seen)} of {N_RATE} rates exercised) to {n} timings of "
           f"{len(by)} cases; rms error of log(duration) {rms:.3f}", file=sys.stderr)
-    regret(by, p, sys.stderr, "training files")
-    if args.held_out:
-        regret(load(args.held_out), p, sys.stderr, "held-out files")
-    emit(p, seen, " ".join(a.split("/")[-1] for a in args.dumps), sys.stdout)
-
+    held = load(args.held_out) if args.held_out else None
+    regret(by, p, sys.stderr, "training files, formula alone")
+    if held:
+        regret(held, p, sys.stderr, "held-out files, formula alone")
+    r = None
+    if not args.no_residual:
+        r, before, after = fit_residual(by, p)
+        print(f"learned correction ({N_FEATURES} inputs, hidden layers of {HIDDEN[0]} and {HIDDEN[1]}): rms of ln(measured / "
+              f"estimate) over the plans within 4 times of the best {before:.3f} -> {after:.3f}", file=sys.stderr)
+        regret(by, p, sys.stderr, "training files, with the correction", r)
+        if held:
+            regret(held, p, sys.stderr, "held-out files, with the correction", r)
+    emit(p, seen, " ".join(a.split("/")[-1] for a in args.dumps), sys.stdout, r)
 
 if __name__ == "__main__":
     main()

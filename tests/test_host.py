@@ -280,6 +280,8 @@ def test_the_fitting_tool_recovers_a_table_from_timings_and_writes_it_back(tmp_p
     inc.write_text(text.getvalue())
     back = plan_fit.read_table(str(inc))
     assert back.shape == table.shape
+    # (printed without a learned correction, the second table is the zero one)
+    assert not plan_fit.read_residual(str(inc)).flat()[4 * plan_fit.N_FEATURES:].any()
     picked, ideal = [], []
     for key, timings in by.items():
         plans = [(d, us) for d, us in timings if d is not None and plan_fit.candidate(d)]
@@ -288,3 +290,40 @@ def test_the_fitting_tool_recovers_a_table_from_timings_and_writes_it_back(tmp_p
         picked.append(truth[choice])
         ideal.append(min(truth))
     assert np.mean(np.array(picked) / np.array(ideal)) < 1.02
+
+
+def test_the_learned_correction_is_trained_printed_and_read_back(tmp_path):
+    """fit_residual on timings that the formula misses by a known factor per lane width: the correction learns most of
+    it, stays within its limit, and survives the trip through the printed table."""
+    import io
+    import os
+
+    from scanscam_amd import plan_fit
+
+    root = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..")
+    table = plan_fit.read_table(os.path.join(root, "scanscam_amd", "csrc", "scan_cl_model.inc"))
+    rng = np.random.default_rng(12)
+    by = {}
+    for _ in range(80):
+        batch, T, C = int(2 ** rng.uniform(3, 10)), int(2 ** rng.uniform(8, 13)), 64 * int(rng.integers(1, 24))
+        for rev in (False, True):
+            timings = []
+            for mode in (2, 3):
+                for vec, steps in ((1, 16), (2, 8), (4, 4), (4, 8)):
+                    for waves in (4, 8):
+                        d = plan_fit.describe(batch, T, C, 4, rev, mode, vec, steps, waves)
+                        timings.append((d, plan_fit.predict(d, table) * (1.0 + 0.1 * vec) * float(np.exp(rng.normal(0, 0.01)))))
+            by[(batch, T, C, 4, rev)] = timings
+    r, before, after = plan_fit.fit_residual(by, table, max_iter=300)
+    assert before > 0.2 and after < 0.05, (before, after)
+    text = io.StringIO()
+    plan_fit.emit(table, set(range(plan_fit.N_RATE)), "synthetic", text, r)
+    inc = tmp_path / "model.inc"
+    inc.write_text(text.getvalue())
+    back = plan_fit.read_residual(str(inc))
+    d = plan_fit.describe(64, 2048, 1024, 4, False, 2, 2, 8, 8)
+    x = plan_fit.features(d, plan_fit.predict(d, table))
+    assert abs(float(back.correct(x)[0]) - float(r.correct(x)[0])) < 1e-6
+    assert abs(float(r.correct(x)[0]) - np.log(1.2)) < 0.05
+    wild = [1e9] * plan_fit.N_FEATURES
+    assert abs(float(r.correct(wild)[0])) <= plan_fit.RESIDUAL_LIMIT
