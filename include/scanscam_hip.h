@@ -265,8 +265,11 @@ int scanscam_resolve_plan_cl(int64_t batch, int64_t T, int64_t C, int dtype, int
  * The duration in microseconds that the library's cost model estimates for a channels-last call on dense
  * [batch, T, C] tensors with this plan (NULL or zero fields: with what the model itself chooses for them, i.e.
  * the estimate behind scanscam_resolve_plan_cl). The automatic plan is the candidate with the smallest such
- * estimate; the constants of the model are fitted to timings on one MI355X (scanscam_amd/plan_fit.py), so the
- * figure is a ranking aid with an error of about 10 %, not a promise. No counterpart in the reference.
+ * estimate; the model (a formula of a few physical terms and a learned correction on top of it) is fitted to
+ * timings on one MI355X (scanscam_amd/plan_fit.py), so the figure is a ranking aid with an error of about 5 %,
+ * not a promise. The first call for a (shape, plan) on a thread takes about 0.1 ms on the host (the choice is
+ * remembered per thread after that; nothing but speed depends on what is remembered). No counterpart in the
+ * reference.
  */
 int scanscam_predict_cl(int64_t batch, int64_t T, int64_t C, int dtype, int direction, const scanscam_plan *plan,
                         double *microseconds);
