@@ -235,6 +235,7 @@ def main(argv=None):
     ap.add_argument("--random", type=int, metavar="N",
                     help="N shapes drawn at random (channels-last, or rows when that layout is named), each in f32 and bf16")
     ap.add_argument("--seed", type=int, default=0, help="seed of --random")
+    ap.add_argument("--dtypes", default="f32,bf16", help="storage types of --suite and --random shapes (f32, bf16, f16, f64)")
     ap.add_argument("--reps", type=int, default=24)
     ap.add_argument("--every", action="store_true", help="also print every plan's timings")
     ap.add_argument("--dump", metavar="FILE", help="channels-last: time every plan of the full set and append each "
@@ -247,11 +248,11 @@ def main(argv=None):
     jobs = []
     if args.suite:
         layout, shapes = SUITES[args.suite]
-        jobs = [(layout, s, dt) for s in shapes for dt in (torch.float32, torch.bfloat16)]
+        jobs = [(layout, s, DTYPES[dt]) for s in shapes for dt in args.dtypes.split(",")]
     elif args.random:
         layout = args.layout or "cl"
         shapes = (random_row_shapes if layout == "rows" else random_cl_shapes)(args.random, args.seed)
-        jobs = [(layout, s, dt) for s in shapes for dt in (torch.float32, torch.bfloat16)]
+        jobs = [(layout, s, DTYPES[dt]) for s in shapes for dt in args.dtypes.split(",")]
     elif args.layout is None:
         ap.error("give a layout and shapes, --suite or --random")
     for spec in args.shapes:
